@@ -1,0 +1,65 @@
+"""ctypes binding of ``libmoba_hip.so`` (the C ABI declared in include/moba_hip.h).
+
+The library is loaded from the package directory and nowhere else; if it is missing
+the operator raises -- there is no fallback path.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import c_char_p, c_int, c_int64, c_size_t, c_void_p
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmoba_hip.so")
+
+_lib = None
+
+_SIGNATURES = {
+    "moba_version": (c_int, []),
+    "moba_strerror": (c_char_p, [c_int]),
+    "moba_chunk_mean_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
+    "moba_chunk_mean": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_void_p]),
+    "moba_gate_topk": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                               c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "moba_topk_from_scores": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_void_p]),
+    "moba_build_lists": (c_int, [c_void_p] * 9 + [c_int64] + [c_int] * 7 + [c_void_p]),
+    "moba_fwd_tile_rows": (c_int, []),
+    "moba_fwd": (c_int, [c_void_p] * 14 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_int64, c_void_p]),
+    "moba_bwd": (c_int, [c_void_p] * 20 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_int64, c_void_p]),
+}
+OPTIONAL = {"moba_bwd"}
+
+
+def load():
+    """Return the loaded library, building nothing: a missing library is an error."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it with `python -m moba_amd.build` (needs hipcc, gfx950). "
+            "moba_amd has no fallback implementation."
+        )
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in _SIGNATURES.items():
+        try:
+            fn = getattr(lib, name)
+        except AttributeError:
+            if name in OPTIONAL:
+                continue
+            raise
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def exported_symbols():
+    return list(_SIGNATURES)
+
+
+def check(code: int, what: str):
+    if code != 0:
+        msg = load().moba_strerror(code).decode()
+        raise RuntimeError(f"{what} failed with code {code}: {msg}")

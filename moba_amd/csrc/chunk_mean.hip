@@ -1,0 +1,109 @@
+// Key chunk-mean: kbar[f, h, :] = bf16( mean over the B tokens of filtered chunk f of K[., h, :] ).
+//
+// HBM-bound: K is read exactly once with 16-byte loads (a wave covers 1 KiB of
+// one token row); the algorithmic traffic is S*H*D*2 bytes.  Accumulation is
+// in fp64: the sum of a chunk of bf16 values is then exact, so the result
+// does not depend on how the chunk is split over workgroups, and the rounded
+// mean is reproducible bit for bit (fp64 -> fp32 -> bf16, round to nearest even).
+//
+// Stage 1: grid (column blocks, token splits, F); each thread owns 8 adjacent
+//          columns of the [H*D] token row and sums its token split.
+// Stage 2: sums the splits in order, divides by B, rounds.
+#include "common.h"
+
+namespace moba {
+
+__global__ __launch_bounds__(256) void chunk_mean_partial_kernel(
+    const bf16* __restrict__ k, const int* __restrict__ fchunk_tok, double* __restrict__ partial,
+    int HD8 /* H*D/8 */, int B, int nsplit, int tok_per_split) {
+  const int col = blockIdx.x * 256 + threadIdx.x;
+  if (col >= HD8) return;
+  const int split = blockIdx.y;
+  const int f = blockIdx.z;
+  const int t0 = split * tok_per_split;
+  const int t1 = min(B, t0 + tok_per_split);
+  const int64_t row_stride = (int64_t)HD8 * 8;
+  const bf16* src = k + ((int64_t)fchunk_tok[f] + t0) * row_stride + (int64_t)col * 8;
+  double acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.0;
+  int t = t0;
+  for (; t + 4 <= t1; t += 4) {
+    bf16x8 x0 = *reinterpret_cast<const bf16x8*>(src);
+    bf16x8 x1 = *reinterpret_cast<const bf16x8*>(src + row_stride);
+    bf16x8 x2 = *reinterpret_cast<const bf16x8*>(src + 2 * row_stride);
+    bf16x8 x3 = *reinterpret_cast<const bf16x8*>(src + 3 * row_stride);
+    src += 4 * row_stride;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      // the four-term sum of bf16 values is exact in fp64 whatever the order
+      acc[e] += ((double)(float)x0[e] + (double)(float)x1[e]) + ((double)(float)x2[e] + (double)(float)x3[e]);
+    }
+  }
+  for (; t < t1; ++t) {
+    bf16x8 x0 = *reinterpret_cast<const bf16x8*>(src);
+    src += row_stride;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] += (double)(float)x0[e];
+  }
+  double* dst = partial + ((int64_t)(f * nsplit + split) * HD8 + col) * 8;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) dst[e] = acc[e];
+}
+
+__global__ __launch_bounds__(256) void chunk_mean_finish_kernel(
+    const double* __restrict__ partial, bf16* __restrict__ kbar, int HD8, int B, int nsplit, int F) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;  // over F * HD8
+  if (idx >= (int64_t)F * HD8) return;
+  const int f = (int)(idx / HD8);
+  const int col = (int)(idx % HD8);
+  double acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.0;
+  for (int s = 0; s < nsplit; ++s) {
+    const double* src = partial + ((int64_t)(f * nsplit + s) * HD8 + col) * 8;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] += src[e];
+  }
+  bf16x8 o;
+  const double inv = (double)B;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) o[e] = (bf16)(float)(acc[e] / inv);
+  *reinterpret_cast<bf16x8*>(kbar + idx * 8) = o;
+}
+
+}  // namespace moba
+
+using namespace moba;
+
+static int pick_nsplit(int HD8, int F, int B) {
+  const int colblocks = (HD8 + 255) / 256;
+  int nsplit = 1;
+  // enough workgroups to fill 256 CUs several times over, at least 32 tokens per split
+  while ((int64_t)colblocks * F * nsplit < 4096 && B / (nsplit * 2) >= 32) nsplit *= 2;
+  return nsplit;
+}
+
+extern "C" size_t moba_chunk_mean_workspace_bytes(int H, int D, int F, int B) {
+  if (H <= 0 || D <= 0 || F <= 0 || B <= 0 || (H * D) % 8 != 0) return 0;
+  const int HD8 = H * D / 8;
+  return (size_t)F * pick_nsplit(HD8, F, B) * HD8 * 8 * sizeof(double);
+}
+
+extern "C" int moba_chunk_mean(const void* k, const int32_t* fchunk_tok, void* kbar, void* workspace,
+                               int64_t S, int H, int D, int F, int B, void* stream) {
+  if (F == 0) return MOBA_OK;
+  if (!k || !fchunk_tok || !kbar || !workspace || S <= 0 || H <= 0 || D <= 0 || F < 0 || B <= 0) return MOBA_ERR_ARG;
+  if ((H * D) % 8 != 0 || ((uintptr_t)k & 15) || ((uintptr_t)kbar & 15) || ((uintptr_t)workspace & 7)) return MOBA_ERR_ARG;
+  const int HD8 = H * D / 8;
+  const int nsplit = pick_nsplit(HD8, F, B);
+  const int tps = (B + nsplit - 1) / nsplit;
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid((HD8 + 255) / 256, nsplit, F);
+  hipLaunchKernelGGL(chunk_mean_partial_kernel, grid, dim3(256), 0, st, (const bf16*)k, fchunk_tok,
+                     (double*)workspace, HD8, B, nsplit, tps);
+  const int64_t n = (int64_t)F * HD8;
+  hipLaunchKernelGGL(chunk_mean_finish_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
+                     (const double*)workspace, (bf16*)kbar, HD8, B, nsplit, F);
+  return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
+}

@@ -1,0 +1,68 @@
+// Shared device helpers for the gfx950 MoBA kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace moba {
+
+typedef __bf16 bf16;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+
+constexpr int kHeadDim = 128;  // the MFMA kernels are specialised for D = 128
+constexpr int kWave = 64;
+
+// error codes returned by every extern "C" entry point
+enum : int {
+  MOBA_OK = 0,
+  MOBA_ERR_ARG = -1,        // bad argument (null pointer, unsupported size, misalignment)
+  MOBA_ERR_UNSUPPORTED = -2,
+  MOBA_ERR_LAUNCH = -3,     // hipGetLastError() after a launch
+  MOBA_ERR_LIMIT = -4,      // size beyond a stated limit
+};
+
+// S^T = K Q^T style product of one 32x32 tile, contraction depth 16:
+// lane l supplies A[l%32][8*(l/32)..+7] and B[8*(l/32)..+7][l%32]; the result
+// element e of lane l is C[8*(e/4) + 4*(l/32) + e%4][l%32].
+__device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+// value held by the lane 32 positions away (the other half of the wave)
+__device__ __forceinline__ float xhalf(float x) { return __shfl_xor(x, 32, 64); }
+
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  bf16x2 p;
+  p[0] = (bf16)lo;
+  p[1] = (bf16)hi;
+  return *reinterpret_cast<uint32_t*>(&p);
+}
+
+// largest i in [0, n) with a[i] <= x, for ascending a with a[0] <= x
+__device__ __forceinline__ int upper_row(const int* __restrict__ a, int n, int x) {
+  int lo = 0, hi = n;  // invariant: a[lo] <= x, a[hi] > x (hi == n means +inf)
+  while (hi - lo > 1) {
+    int mid = (lo + hi) >> 1;
+    if (a[mid] <= x) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+
+// Workgroup ids are dealt round-robin to the 8 XCDs (each with its own L2).
+// Remap so that a contiguous range of logical ids lands on one XCD.
+__device__ __forceinline__ int xcd_remap(int bid, int nblocks) {
+  constexpr int X = 8;
+  int per = (nblocks + X - 1) / X;
+  int logical = (bid % X) * per + bid / X;
+  return logical;  // may be >= nblocks for the padded tail: callers bound-check
+}
+
+}  // namespace moba

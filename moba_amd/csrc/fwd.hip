@@ -1,0 +1,354 @@
+// Fused MoBA forward for gfx950.
+//
+// One kernel covers both kinds of work, as tiles of 128 query rows of one head:
+//   history tile : 128 rows of the gather list of segment (filtered chunk f, head h),
+//                  against the B keys of chunk f, no mask
+//   self tile    : 128 consecutive rows of one chunk against the keys of the same
+//                  chunk up to the diagonal (causal); with the chunk table set to whole
+//                  sequences this is plain causal attention (the k <= 0 case)
+// Each tile runs a flash-style loop over 64-key tiles: K and V tiles are staged in LDS
+// (double buffered, bank-conflict-free swizzles), S^T = K Q^T and O^T += V^T P^T use
+// v_mfma_f32_32x32x16_bf16 with the query index in the lane dimension, so a row's
+// softmax statistics live in one lane pair; V^T fragments come from ds_read_b64_tr_b16.
+// A tile writes a normalised partial output (bf16) and its log2-sum-exp into the
+// row's slot; the merge kernel combines the K+1 slots of every (token, head).
+//
+// Algorithmic work: 4*D flops per attended (query, key) pair; the bound is the bf16
+// MFMA rate.  Compulsory HBM traffic is q, k, v once, the partials once each way.
+#include "common.h"
+
+namespace moba {
+
+constexpr int TM = 128;  // query rows per workgroup (32 per wave)
+constexpr int TN = 64;   // keys per inner iteration
+constexpr int kTileBytes = TN * kHeadDim * 2;
+constexpr int kFwdLds = 4 * kTileBytes;  // K[2], V[2]
+constexpr int kXcdBlock = 64;            // consecutive logical tiles that share an XCD
+
+struct FwdParams {
+  const bf16* q;
+  const bf16* k;
+  const bf16* v;
+  bf16* part_o;            // [S*H*K1, D]
+  float* part_lse;         // [S*H*K1], log2 domain
+  const int* seg_off;      // [F*H+1]
+  const int* tile_off;     // [F*H+1]
+  const int* seg_dest;     // [M]
+  const int* fchunk_tok;   // [F]
+  const int* chunk_tok;    // [N+1]
+  const int* self_tile_prefix;  // [N+1]
+  int S, H, K1, F, N, B;
+  int hist_bound;          // upper bound on history tiles (logical ids below it)
+  int self_total;          // self_tile_prefix[N] * H
+  float scale_log2;        // D^-0.5 * log2(e)
+};
+
+__device__ __forceinline__ int k_lds_off(int key, int c16) { return key * 256 + ((c16 ^ (key & 15)) << 4); }
+__device__ __forceinline__ int v_lds_off(int key, int c16) {
+  return key * 256 + ((((c16 >> 2) ^ (key & 3))) << 6) + ((c16 & 3) << 4);
+}
+
+__device__ __forceinline__ bf16x4 lds_read_tr(const char* p) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+      (__attribute__((address_space(3))) bf16x4*)(p));
+}
+
+__global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams p) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int n = lane & 31, hh = lane >> 5;
+  const int H = p.H;
+
+  // ---- which tile ----
+  int logical;
+  {
+    const int x = blockIdx.x & 7, y = blockIdx.x >> 3;
+    logical = ((y / kXcdBlock) * 8 + x) * kXcdBlock + (y % kXcdBlock);
+  }
+  int h, kv_tok0, nkeys, row_count, dest, tok, limit, wave_min_limit, wave_max_limit;
+  const int r = wave * 32 + n;
+  if (logical < p.hist_bound) {
+    const int FH = p.F * H;
+    if (FH == 0 || logical >= p.tile_off[FH]) return;
+    const int seg = upper_row(p.tile_off, FH, logical);
+    const int tile = logical - p.tile_off[seg];
+    const int f = seg / H;
+    h = seg - f * H;
+    const int base = p.seg_off[seg] + tile * TM;
+    row_count = min(TM, p.seg_off[seg + 1] - base);
+    kv_tok0 = p.fchunk_tok[f];
+    nkeys = p.B;
+    dest = p.seg_dest[base + min(r, row_count - 1)];
+    tok = dest / (H * p.K1);
+    limit = nkeys - 1;
+    wave_min_limit = limit;
+    wave_max_limit = limit;
+  } else {
+    const int st = logical - p.hist_bound;
+    if (st >= p.self_total) return;
+    // chunk c with self_tile_prefix[c]*H <= st
+    int lo = 0, hi = p.N;
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (p.self_tile_prefix[mid] * H <= st) lo = mid; else hi = mid;
+    }
+    const int c = lo;
+    const int rem = st - p.self_tile_prefix[c] * H;
+    const int nt = p.self_tile_prefix[c + 1] - p.self_tile_prefix[c];
+    h = rem / nt;
+    const int tin = nt - 1 - (rem - h * nt);  // longest tiles first
+    const int c0 = p.chunk_tok[c];
+    const int len = p.chunk_tok[c + 1] - c0;
+    const int r0 = tin * TM;
+    row_count = min(TM, len - r0);
+    kv_tok0 = c0;
+    nkeys = min(len, r0 + TM);
+    tok = c0 + r0 + min(r, row_count - 1);
+    dest = (tok * H + h) * p.K1;
+    limit = r0 + min(r, row_count - 1);
+    wave_min_limit = r0 + min(wave * 32, row_count - 1);
+    wave_max_limit = r0 + min(wave * 32 + 31, row_count - 1);
+  }
+  const bool row_valid = r < row_count;
+
+  // ---- Q^T operand: lane (n, hh) holds q[tok][16*ks + 8*hh .. +7] ----
+  bf16x8 bq[8];
+  {
+    const bf16* src = p.q + ((int64_t)tok * H + h) * kHeadDim + 8 * hh;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) bq[ks] = *reinterpret_cast<const bf16x8*>(src + 16 * ks);
+  }
+
+  // ---- K/V tile loader: thread owns key (tid/16 + 16*i), 16-byte column tid%16 ----
+  const int ld_key = tid >> 4, ld_c16 = tid & 15;
+  const int64_t row_elems = (int64_t)H * kHeadDim;
+  const bf16* kbase = p.k + (int64_t)h * kHeadDim + ld_c16 * 8;
+  const bf16* vbase = p.v + (int64_t)h * kHeadDim + ld_c16 * 8;
+  bf16x8 kreg[4], vreg[4];
+  auto load_tile = [&](int kt) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int key = kt * TN + ld_key + 16 * i;
+      const bool ok = key < nkeys;
+      const int64_t t = min(kv_tok0 + key, p.S - 1);
+      bf16x8 kk = *reinterpret_cast<const bf16x8*>(kbase + t * row_elems);
+      bf16x8 vv = *reinterpret_cast<const bf16x8*>(vbase + t * row_elems);
+      if (!ok) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { kk[e] = (bf16)0.f; vv[e] = (bf16)0.f; }
+      }
+      kreg[i] = kk;
+      vreg[i] = vv;
+    }
+  };
+  auto store_tile = [&](int buf) {
+    char* ks = smem + buf * kTileBytes;
+    char* vs = smem + (2 + buf) * kTileBytes;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int key = ld_key + 16 * i;
+      *reinterpret_cast<bf16x8*>(ks + k_lds_off(key, ld_c16)) = kreg[i];
+      *reinterpret_cast<bf16x8*>(vs + v_lds_off(key, ld_c16)) = vreg[i];
+    }
+  };
+
+  const int nkt = (nkeys + TN - 1) / TN;
+  load_tile(0);
+  store_tile(0);
+  __syncthreads();
+
+  f32x16 oacc[4];
+#pragma unroll
+  for (int db = 0; db < 4; ++db)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) oacc[db][e] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+  const float sl2 = p.scale_log2;
+
+  // per-lane pieces of the V^T fragment address
+  const int g16 = lane >> 4, i0 = (lane & 15) >> 2, i1 = lane & 3;
+  const int v_lane_off = 32 * (g16 & 1) + 8 * i1;
+
+  for (int kt = 0; kt < nkt; ++kt) {
+    const int buf = kt & 1;
+    const bool has_next = kt + 1 < nkt;
+    if (has_next) load_tile(kt + 1);
+
+    if (kt * TN <= wave_max_limit) {  // wave-uniform: skip tiles entirely above the diagonal
+      const char* ks = smem + buf * kTileBytes;
+      const char* vs = smem + (2 + buf) * kTileBytes;
+      // S^T (keys x queries), two 32-key blocks
+      f32x16 sacc[2];
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) sacc[kb][e] = 0.f;
+        const int key = 32 * kb + n;
+#pragma unroll
+        for (int s8 = 0; s8 < 8; ++s8) {
+          const bf16x8 a = *reinterpret_cast<const bf16x8*>(ks + k_lds_off(key, 2 * s8 + hh));
+          sacc[kb] = mfma32(a, bq[s8], sacc[kb]);
+        }
+      }
+      if (kt * TN + TN - 1 > wave_min_limit) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            const int key = kt * TN + 32 * kb + 8 * (e >> 2) + 4 * hh + (e & 3);
+            if (key > limit) sacc[kb][e] = -INFINITY;
+          }
+      }
+      float mx = sacc[0][0];
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) mx = fmaxf(mx, sacc[kb][e]);
+      mx = fmaxf(mx, xhalf(mx));
+      const float m_new = fmaxf(m_run, mx * sl2);
+      const float alpha = fast_exp2(m_run - m_new);
+      m_run = m_new;
+      float rs = 0.f;
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const float pe = fast_exp2(sacc[kb][e] * sl2 - m_new);
+          sacc[kb][e] = pe;
+          rs += pe;
+        }
+      l_run = l_run * alpha + rs;
+      if (__any(alpha != 1.f)) {
+#pragma unroll
+        for (int db = 0; db < 4; ++db)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) oacc[db][e] *= alpha;
+      }
+      // P^T operand for the four 16-key steps
+      bf16x8 pb[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int kb = j >> 1, e0 = 8 * (j & 1);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) pb[j][e] = (bf16)sacc[kb][e0 + e];
+      }
+      // O^T += V^T P^T
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int keyA = 16 * j + 4 * hh + i0;
+        const int keyB = keyA + 8;
+#pragma unroll
+        for (int db = 0; db < 4; ++db) {
+          const bf16x4 va = lds_read_tr(vs + keyA * 256 + ((db ^ (keyA & 3)) << 6) + v_lane_off);
+          const bf16x4 vb = lds_read_tr(vs + keyB * 256 + ((db ^ (keyB & 3)) << 6) + v_lane_off);
+          bf16x8 a;
+          a[0] = va[0]; a[1] = va[1]; a[2] = va[2]; a[3] = va[3];
+          a[4] = vb[0]; a[5] = vb[1]; a[6] = vb[2]; a[7] = vb[3];
+          oacc[db] = mfma32(a, pb[j], oacc[db]);
+        }
+      }
+    }
+    if (has_next) store_tile(buf ^ 1);
+    __syncthreads();
+  }
+
+  // ---- epilogue: normalise, write the partial ----
+  const float l_tot = l_run + xhalf(l_run);
+  const float inv = 1.f / l_tot;
+  if (row_valid) {
+    bf16* dst = p.part_o + (int64_t)dest * kHeadDim;
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        u32x2 w;
+        w[0] = pack_bf16(oacc[db][4 * g + 0] * inv, oacc[db][4 * g + 1] * inv);
+        w[1] = pack_bf16(oacc[db][4 * g + 2] * inv, oacc[db][4 * g + 3] * inv);
+        *reinterpret_cast<u32x2*>(dst + 32 * db + 8 * g + 4 * hh) = w;
+      }
+    if (hh == 0) p.part_lse[dest] = m_run + fast_log2(l_tot);
+  }
+}
+
+// Combine the K1 slots of each (token, head): slot 0 is the self part, slot 1+j the
+// j-th selected history chunk (present iff sel[row, j] >= 0).  16 lanes per row.
+__global__ __launch_bounds__(256) void moba_merge_kernel(const bf16* __restrict__ part_o,
+                                                         const float* __restrict__ part_lse,
+                                                         const int* __restrict__ sel, bf16* __restrict__ out,
+                                                         float* __restrict__ lse, int64_t rows, int K1) {
+  const int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+  if (row >= rows) return;
+  const int c8 = threadIdx.x & 15;
+  const int K = K1 - 1;
+  const float* pl = part_lse + row * K1;
+  const int* ps = sel + row * K;
+  float mx = pl[0];
+  for (int j = 0; j < K; ++j)
+    if (ps[j] >= 0) mx = fmaxf(mx, pl[1 + j]);
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+  float wsum = 0.f;
+  const bf16* po = part_o + row * K1 * kHeadDim + c8 * 8;
+  for (int j = 0; j < K1; ++j) {
+    if (j > 0 && ps[j - 1] < 0) continue;
+    const float w = fast_exp2(pl[j] - mx);
+    wsum += w;
+    const bf16x8 x = *reinterpret_cast<const bf16x8*>(po + (int64_t)j * kHeadDim);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] += w * (float)x[e];
+  }
+  const float inv = 1.f / wsum;
+  bf16x8 o;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) o[e] = (bf16)(acc[e] * inv);
+  *reinterpret_cast<bf16x8*>(out + row * kHeadDim + c8 * 8) = o;
+  if (c8 == 0) lse[row] = (mx + fast_log2(wsum)) * 0.6931471805599453f;
+}
+
+}  // namespace moba
+
+using namespace moba;
+
+extern "C" int moba_fwd_tile_rows(void) { return TM; }
+
+// hist_bound: any upper bound on the number of history tiles (floor(M/128) + F*H is one).
+extern "C" int moba_fwd(const void* q, const void* k, const void* v, void* part_o, float* part_lse,
+                        const int32_t* sel, const int32_t* seg_off, const int32_t* tile_off,
+                        const int32_t* seg_dest, const int32_t* fchunk_tok, const int32_t* chunk_tok,
+                        const int32_t* self_tile_prefix, void* out, float* lse, int64_t S, int H, int D, int K,
+                        int F, int N, int B, int64_t hist_bound, int64_t self_tiles, void* stream) {
+  if (!q || !k || !v || !part_o || !part_lse || !chunk_tok || !self_tile_prefix || !out || !lse) return MOBA_ERR_ARG;
+  if (K > 0 && (!sel || !seg_off || !tile_off || !seg_dest || !fchunk_tok)) return MOBA_ERR_ARG;
+  if (D != kHeadDim) return MOBA_ERR_UNSUPPORTED;
+  if (S <= 0 || H <= 0 || K < 0 || F < 0 || N <= 0 || B <= 0 || hist_bound < 0 || self_tiles <= 0) return MOBA_ERR_ARG;
+  if (((uintptr_t)q & 15) || ((uintptr_t)k & 15) || ((uintptr_t)v & 15) || ((uintptr_t)part_o & 15) ||
+      ((uintptr_t)out & 15))
+    return MOBA_ERR_ARG;
+  if ((int64_t)S * H * (K + 1) >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
+  const int64_t total = hist_bound + self_tiles * H;
+  const int64_t grid = (total + 8 * kXcdBlock - 1) / (8 * kXcdBlock) * (8 * kXcdBlock);
+  if (grid >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
+  FwdParams p;
+  p.q = (const bf16*)q; p.k = (const bf16*)k; p.v = (const bf16*)v;
+  p.part_o = (bf16*)part_o; p.part_lse = part_lse;
+  p.seg_off = seg_off; p.tile_off = tile_off; p.seg_dest = seg_dest; p.fchunk_tok = fchunk_tok;
+  p.chunk_tok = chunk_tok; p.self_tile_prefix = self_tile_prefix;
+  p.S = (int)S; p.H = H; p.K1 = K + 1; p.F = (K > 0) ? F : 0; p.N = N; p.B = B;
+  p.hist_bound = (K > 0) ? (int)hist_bound : 0;
+  p.self_total = (int)(self_tiles * H);
+  p.scale_log2 = (float)(1.4426950408889634 / sqrt((double)D));
+  hipStream_t st = (hipStream_t)stream;
+  static bool attr_set = false;
+  if (!attr_set) {
+    if (hipFuncSetAttribute((const void*)moba_fwd_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kFwdLds) !=
+        hipSuccess)
+      return MOBA_ERR_LAUNCH;
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(moba_fwd_kernel, dim3((unsigned)grid), dim3(256), kFwdLds, st, p);
+  const int64_t rows = S * H;
+  hipLaunchKernelGGL(moba_merge_kernel, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st, (const bf16*)part_o,
+                     (const float*)part_lse, sel, (bf16*)out, lse, rows, K + 1);
+  return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
+}

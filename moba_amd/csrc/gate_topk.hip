@@ -1,0 +1,194 @@
+// Parameter-less gate and causal top-k.
+//
+// score(s, h, f) = <q[s,h,:], kbar[f,h,:]> in fp32 (bf16 x bf16 products are exact in
+// fp32; the MFMA accumulates them in fp32).  A token s in the c-th chunk of its
+// sequence may pick among the c earlier chunks of the same sequence, whose
+// filtered-chunk ids are [fb, fb + c) with fb the first filtered id of the
+// sequence.  The K best are kept; ties go to the lower chunk id; a -inf or NaN
+// score is never picked.  Output sel[s, h, 0..K) holds filtered-chunk ids in
+// descending score order, -1 padded.
+//
+// One wave handles 64 consecutive tokens of one head: the score tile
+// (32 chunks x 64 tokens) is two 32x32x16 MFMA accumulators, staged through LDS
+// so that each lane then owns one token and runs an insertion top-k held in
+// registers.  Scores never reach HBM (except through the optional debug output).
+#include "common.h"
+
+namespace moba {
+
+template <int KMAX>
+struct TopK {
+  float val[KMAX];
+  int idx[KMAX];
+  __device__ __forceinline__ void init() {
+#pragma unroll
+    for (int j = 0; j < KMAX; ++j) {
+      val[j] = -INFINITY;
+      idx[j] = -1;
+    }
+  }
+  // keep the list sorted by descending value; an equal value stays behind the
+  // entries already present, so among equal scores the lower id (seen first) wins
+  __device__ __forceinline__ void push(float x, int id) {
+    if (x > val[KMAX - 1]) {
+#pragma unroll
+      for (int j = KMAX - 1; j >= 1; --j) {
+        const bool shift = x > val[j - 1];
+        const bool here = !shift && (x > val[j]);
+        val[j] = shift ? val[j - 1] : (here ? x : val[j]);
+        idx[j] = shift ? idx[j - 1] : (here ? id : idx[j]);
+      }
+      if (x > val[0]) {
+        val[0] = x;
+        idx[0] = id;
+      }
+    }
+  }
+};
+
+// locate the sequence of token s: largest b with cu[b] <= s
+__device__ __forceinline__ int find_seq(const int* __restrict__ cu, int nseq, int s) {
+  return upper_row(cu, nseq, s);
+}
+
+template <int KMAX>
+__global__ __launch_bounds__(256) void gate_topk_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ kbar, const int* __restrict__ cu_seqlens,
+    const int* __restrict__ seq_fbase, int* __restrict__ sel, float* __restrict__ scores_out,
+    int S, int H, int nseq, int F, int B, int K) {
+  __shared__ float sc[4][64][33];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int n = lane & 31, hh = lane >> 5;
+  const int tok0 = blockIdx.x * 64;
+  const int h = blockIdx.y * 4 + wave;
+  const bool head_ok = h < H;
+  const int hc = head_ok ? h : H - 1;
+
+  // this lane's own token (selection phase)
+  const int s = tok0 + lane;
+  int fb = 0, c = 0;
+  if (s < S) {
+    const int b = find_seq(cu_seqlens, nseq, s);
+    fb = seq_fbase[b];
+    c = (s - cu_seqlens[b]) / B;
+  }
+  // union of the candidate ranges of the 64 tokens (identical for the 4 waves)
+  int flo = c > 0 ? fb : 0x7fffffff;
+  int fhi = c > 0 ? fb + c : 0;
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) {
+    flo = min(flo, __shfl_xor(flo, o, 64));
+    fhi = max(fhi, __shfl_xor(fhi, o, 64));
+  }
+
+  TopK<KMAX> top;
+  top.init();
+
+  if (fhi > 0) {  // wave-uniform (and block-uniform)
+    // Q^T operand: lane (n, hh) holds q[token n (+32)][16*ks + 8*hh .. +7]
+    bf16x8 bq[2][8];
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) {
+      const int tok = min(tok0 + 32 * qb + n, S - 1);
+      const bf16* src = q + ((int64_t)tok * H + hc) * kHeadDim + 8 * hh;
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) bq[qb][ks] = *reinterpret_cast<const bf16x8*>(src + 16 * ks);
+    }
+    for (int f0 = flo; f0 < fhi; f0 += 32) {
+      const int fr = min(f0 + n, F - 1);
+      const bf16* src = kbar + ((int64_t)fr * H + hc) * kHeadDim + 8 * hh;
+      f32x16 acc0 = {0}, acc1 = {0};
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(src + 16 * ks);
+        acc0 = mfma32(a, bq[0][ks], acc0);
+        acc1 = mfma32(a, bq[1][ks], acc1);
+      }
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int ch = 8 * (e >> 2) + 4 * hh + (e & 3);
+        sc[wave][n][ch] = acc0[e];
+        sc[wave][32 + n][ch] = acc1[e];
+      }
+      __syncthreads();
+#pragma unroll 4
+      for (int j = 0; j < 32; ++j) {
+        const int f = f0 + j;
+        const float x = sc[wave][lane][j];
+        const bool valid = (f >= fb) && (f < fb + c);
+        if (valid) {
+          top.push(x, f);
+          if (scores_out && head_ok) scores_out[((int64_t)s * H + h) * F + f] = x;
+        }
+      }
+      __syncthreads();
+    }
+  }
+  if (s < S && head_ok) {
+    int* dst = sel + ((int64_t)s * H + h) * K;
+#pragma unroll
+    for (int j = 0; j < KMAX; ++j)
+      if (j < K) dst[j] = top.idx[j];
+  }
+}
+
+// Selection alone, on scores supplied by the caller ([S, H, F] fp32, -inf where a
+// chunk is not a valid candidate).  Same insertion routine as the fused kernel.
+template <int KMAX>
+__global__ __launch_bounds__(256) void topk_from_scores_kernel(const float* __restrict__ scores,
+                                                               int* __restrict__ sel, int64_t rows, int F, int K) {
+  const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (r >= rows) return;
+  TopK<KMAX> top;
+  top.init();
+  const float* src = scores + r * F;
+  for (int f = 0; f < F; ++f) top.push(src[f], f);
+  int* dst = sel + r * K;
+#pragma unroll
+  for (int j = 0; j < KMAX; ++j)
+    if (j < K) dst[j] = top.idx[j];
+}
+
+}  // namespace moba
+
+using namespace moba;
+
+#define MOBA_DISPATCH_K(K, CALL)            \
+  if ((K) <= 2) { CALL(2); }                \
+  else if ((K) <= 4) { CALL(4); }           \
+  else if ((K) <= 8) { CALL(8); }           \
+  else if ((K) <= 12) { CALL(12); }         \
+  else if ((K) <= 16) { CALL(16); }         \
+  else if ((K) <= 32) { CALL(32); }         \
+  else if ((K) <= 64) { CALL(64); }         \
+  else return MOBA_ERR_LIMIT;
+
+extern "C" int moba_gate_topk(const void* q, const void* kbar, const int32_t* cu_seqlens, const int32_t* seq_fbase,
+                              int32_t* sel, float* scores_out, int64_t S, int H, int D, int nseq, int F, int B,
+                              int K, void* stream) {
+  if (!q || !kbar || !cu_seqlens || !seq_fbase || !sel) return MOBA_ERR_ARG;
+  if (S <= 0 || S > 0x7fffffff - 64 || H <= 0 || nseq <= 0 || F <= 0 || B <= 0 || K <= 0) return MOBA_ERR_ARG;
+  if (D != kHeadDim) return MOBA_ERR_UNSUPPORTED;
+  if (((uintptr_t)q & 15) || ((uintptr_t)kbar & 15)) return MOBA_ERR_ARG;
+  dim3 grid((unsigned)((S + 63) / 64), (unsigned)((H + 3) / 4));
+  hipStream_t st = (hipStream_t)stream;
+#define CALL(KM)                                                                                              \
+  hipLaunchKernelGGL(gate_topk_kernel<KM>, grid, dim3(256), 0, st, (const bf16*)q, (const bf16*)kbar, cu_seqlens, \
+                     seq_fbase, sel, scores_out, (int)S, H, nseq, F, B, K)
+  MOBA_DISPATCH_K(K, CALL)
+#undef CALL
+  return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
+}
+
+extern "C" int moba_topk_from_scores(const float* scores, int32_t* sel, int64_t S, int H, int F, int K,
+                                     void* stream) {
+  if (!scores || !sel || S <= 0 || H <= 0 || F <= 0 || K <= 0) return MOBA_ERR_ARG;
+  const int64_t rows = S * H;
+  dim3 grid((unsigned)((rows + 255) / 256));
+  hipStream_t st = (hipStream_t)stream;
+#define CALL(KM) \
+  hipLaunchKernelGGL(topk_from_scores_kernel<KM>, grid, dim3(256), 0, st, scores, sel, rows, F, K)
+  MOBA_DISPATCH_K(K, CALL)
+#undef CALL
+  return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
+}

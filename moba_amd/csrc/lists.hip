@@ -1,0 +1,218 @@
+// Varlen gather lists: for every (filtered chunk f, head h) the ascending list of
+// query tokens that selected it, as a counting sort keyed by (f, h) that is stable
+// in the token index -- integer work, no copy of q or kv.
+//
+//   pass 1  count    one workgroup per (query chunk, head): how many of its tokens
+//                    picked each earlier chunk of the sequence -> cnt[(f, h, query chunk)]
+//   pass 2  scan     exclusive prefix sum of cnt in (f, h, query chunk) order: that is
+//                    the list position of the first such token, because query chunks
+//                    of a sequence are visited in ascending token order
+//   pass 3  fill     same decomposition as pass 1; inside a workgroup the four waves own
+//                    consecutive quarters of the chunk, and inside a 64-token batch
+//                    the rank of a token among those with the same pick comes from a
+//                    64-bit lane mask built with LDS atomics (order independent)
+//   pass 4  segment offsets and per-segment tile counts, then their prefix sum
+//
+// List entries are destination rows of the partial-result buffers:
+// dest = (token * H + h) * (K + 1) + 1 + slot, from which the token is recovered by
+// one division.
+#include "common.h"
+
+namespace moba {
+
+__device__ __forceinline__ int cnt_index(const int* __restrict__ pair_off, int f, int h, int H, int crel) {
+  const int p0 = pair_off[f];
+  const int nq = pair_off[f + 1] - p0;
+  return p0 * H + h * nq + crel;
+}
+
+__global__ __launch_bounds__(256) void lists_count_kernel(
+    const int* __restrict__ sel, const int* __restrict__ chunk_tok, const int* __restrict__ chunk_fb,
+    const int* __restrict__ chunk_local, const int* __restrict__ pair_off, int* __restrict__ cnt, int H, int K) {
+  extern __shared__ int lds[];
+  const int cq = blockIdx.x, h = blockIdx.y;
+  const int c = chunk_local[cq];
+  if (c == 0) return;
+  const int fb = chunk_fb[cq];
+  const int t0 = chunk_tok[cq], t1 = chunk_tok[cq + 1];
+  for (int i = threadIdx.x; i < c; i += 256) lds[i] = 0;
+  __syncthreads();
+  for (int s = t0 + threadIdx.x; s < t1; s += 256) {
+    const int* src = sel + ((int64_t)s * H + h) * K;
+    for (int j = 0; j < K; ++j) {
+      const int i = src[j] - fb;
+      if ((unsigned)i < (unsigned)c) atomicAdd(&lds[i], 1);
+    }
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < c; i += 256) cnt[cnt_index(pair_off, fb + i, h, H, c - i - 1)] = lds[i];
+}
+
+__global__ __launch_bounds__(256) void lists_fill_kernel(
+    const int* __restrict__ sel, const int* __restrict__ chunk_tok, const int* __restrict__ chunk_fb,
+    const int* __restrict__ chunk_local, const int* __restrict__ pair_off, const int* __restrict__ base,
+    int* __restrict__ seg_dest, int H, int K) {
+  extern __shared__ int lds[];
+  const int cq = blockIdx.x, h = blockIdx.y;
+  const int c = chunk_local[cq];
+  if (c == 0) return;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  int* pos = lds;                                            // [4][c] running list position per wave
+  unsigned* bits = reinterpret_cast<unsigned*>(lds + 4 * c);  // [4][c][2] lanes of the batch that picked i
+  const int fb = chunk_fb[cq];
+  const int t0 = chunk_tok[cq], t1 = chunk_tok[cq + 1];
+  const int qlen = (t1 - t0 + 3) / 4;
+  const int w0 = min(t1, t0 + wave * qlen), w1 = min(t1, w0 + qlen);
+  const int K1 = K + 1;
+  for (int i = threadIdx.x; i < 4 * c; i += 256) {
+    pos[i] = 0;
+    bits[2 * i] = 0;
+    bits[2 * i + 1] = 0;
+  }
+  __syncthreads();
+  // per-wave counts
+  for (int s = w0 + lane; s < w1; s += 64) {
+    const int* src = sel + ((int64_t)s * H + h) * K;
+    for (int j = 0; j < K; ++j) {
+      const int i = src[j] - fb;
+      if ((unsigned)i < (unsigned)c) atomicAdd(&pos[wave * c + i], 1);
+    }
+  }
+  __syncthreads();
+  // counts -> start positions: global base of (f, h, this query chunk) plus the earlier waves
+  for (int i = threadIdx.x; i < c; i += 256) {
+    int run = base[cnt_index(pair_off, fb + i, h, H, c - i - 1)];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const int n = pos[w * c + i];
+      pos[w * c + i] = run;
+      run += n;
+    }
+  }
+  __syncthreads();
+  const int nbatch = (qlen + 63) / 64;  // same for the four waves
+  int* wpos = pos + wave * c;
+  unsigned* wbits = bits + 2 * wave * c;
+  const uint64_t below = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+  for (int bi = 0; bi < nbatch; ++bi) {
+    const int s = w0 + bi * 64 + lane;
+    const bool active = s < w1;
+    const int* src = sel + ((int64_t)(active ? s : t0) * H + h) * K;
+    for (int j = 0; j < K; ++j) {
+      const int i = src[j] - fb;
+      if (active && (unsigned)i < (unsigned)c) atomicOr(&wbits[2 * i + (lane >> 5)], 1u << (lane & 31));
+    }
+    __syncthreads();
+    for (int j = 0; j < K; ++j) {
+      const int i = src[j] - fb;
+      if (active && (unsigned)i < (unsigned)c) {
+        const uint64_t m = (uint64_t)wbits[2 * i] | ((uint64_t)wbits[2 * i + 1] << 32);
+        const int rank = __popcll(m & below);
+        seg_dest[wpos[i] + rank] = (s * H + h) * K1 + 1 + j;
+      }
+    }
+    __syncthreads();
+    for (int j = 0; j < K; ++j) {
+      const int i = src[j] - fb;
+      if (active && (unsigned)i < (unsigned)c) {
+        const uint64_t m = (uint64_t)wbits[2 * i] | ((uint64_t)wbits[2 * i + 1] << 32);
+        if ((m & below) == 0) {  // the first lane of this pick closes the batch for it
+          wpos[i] += __popcll(m);
+          wbits[2 * i] = 0;
+          wbits[2 * i + 1] = 0;
+        }
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// exclusive prefix sum of a[0..n) in place, total stored at a[n]; one workgroup.
+__global__ __launch_bounds__(1024) void scan_kernel(int* __restrict__ a, int n) {
+  __shared__ int wsum[16];
+  __shared__ int carry_s;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (tid == 0) carry_s = 0;
+  __syncthreads();
+  for (int base = 0; base < n; base += 4096) {
+    const int i0 = base + tid * 4;
+    int v[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = (i0 + e < n) ? a[i0 + e] : 0;
+    const int tsum = v[0] + v[1] + v[2] + v[3];
+    int inc = tsum;  // inclusive scan across the wave
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int t = __shfl_up(inc, o, 64);
+      if (lane >= o) inc += t;
+    }
+    if (lane == 63) wsum[wave] = inc;
+    __syncthreads();
+    int woff = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) {
+      const int x = wsum[w];
+      if (w < wave) woff += x;
+      total += x;
+    }
+    const int carry = carry_s;
+    int run = carry + woff + inc - tsum;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if (i0 + e < n) a[i0 + e] = run;
+      run += v[e];
+    }
+    __syncthreads();
+    if (tid == 0) carry_s = carry + total;
+    __syncthreads();
+  }
+  if (tid == 0) a[n] = carry_s;
+}
+
+// per (f, h): list start and number of row tiles
+__global__ __launch_bounds__(256) void lists_segments_kernel(const int* __restrict__ base,
+                                                             const int* __restrict__ pair_off,
+                                                             int* __restrict__ seg_off, int* __restrict__ tile_off,
+                                                             int F, int H, int tile_rows) {
+  const int fh = blockIdx.x * 256 + threadIdx.x;
+  if (fh > F * H) return;
+  if (fh == F * H) {
+    seg_off[fh] = base[pair_off[F] * H];
+    return;
+  }
+  const int f = fh / H, h = fh % H;
+  const int p0 = pair_off[f];
+  const int nq = pair_off[f + 1] - p0;
+  const int start = base[p0 * H + h * nq];
+  const int end = base[p0 * H + (h + 1) * nq];
+  seg_off[fh] = start;
+  tile_off[fh] = (end - start + tile_rows - 1) / tile_rows;
+}
+
+}  // namespace moba
+
+using namespace moba;
+
+// Limits: chunks per sequence minus one (cmax) is bounded by the LDS the fill pass
+// needs, 48 bytes per candidate chunk.
+extern "C" int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, const int32_t* chunk_fb,
+                                const int32_t* chunk_local, const int32_t* pair_off, int32_t* cnt,
+                                int32_t* seg_off, int32_t* tile_off, int32_t* seg_dest, int64_t S, int H, int K,
+                                int N, int F, int P, int cmax, int tile_rows, void* stream) {
+  if (!sel || !chunk_tok || !chunk_fb || !chunk_local || !pair_off || !cnt || !seg_off || !tile_off || !seg_dest)
+    return MOBA_ERR_ARG;
+  if (S <= 0 || H <= 0 || K <= 0 || N <= 0 || F <= 0 || P <= 0 || cmax <= 0 || tile_rows <= 0) return MOBA_ERR_ARG;
+  if ((int64_t)S * H * (K + 1) >= 0x7fffffffLL || (int64_t)P * H >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
+  if (H > 65535 || (size_t)cmax * 48 > 160 * 1024) return MOBA_ERR_LIMIT;
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid(N, H);
+  hipLaunchKernelGGL(lists_count_kernel, grid, dim3(256), (size_t)cmax * 4, st, sel, chunk_tok, chunk_fb,
+                     chunk_local, pair_off, cnt, H, K);
+  hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(1024), 0, st, cnt, P * H);
+  hipLaunchKernelGGL(lists_fill_kernel, grid, dim3(256), (size_t)cmax * 48, st, sel, chunk_tok, chunk_fb,
+                     chunk_local, pair_off, (const int*)cnt, seg_dest, H, K);
+  hipLaunchKernelGGL(lists_segments_kernel, dim3((F * H + 1 + 255) / 256), dim3(256), 0, st, (const int*)cnt,
+                     pair_off, seg_off, tile_off, F, H, tile_rows);
+  hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(1024), 0, st, tile_off, F * H);
+  return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
+}

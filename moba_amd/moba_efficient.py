@@ -1,0 +1,196 @@
+"""``moba_attn_varlen`` on MI355X: same signature and semantics as the reference
+operator (moba/moba_efficient.py:270-443), computed by the hand-written HIP kernels of
+``libmoba_hip.so``.  PyTorch owns every buffer; this module only validates arguments,
+sizes workspaces and sequences the launches on the current stream.
+
+Stages (each also callable on its own, which is how the tests reach them):
+  chunk_mean        key chunk representatives         (moba_efficient.py:326-340)
+  gate_topk         fp32 gate + causal top-k          (moba_efficient.py:341-371)
+  build_lists       varlen gather lists               (moba_efficient.py:373-423)
+  forward kernels   self + history attention + merge  (moba_efficient.py:69-183)
+  backward kernels  dq, dk, dv                        (moba_efficient.py:185-267)
+"""
+
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import _lib
+from .plan import MobaPlan, TILE_ROWS, make_plan
+
+HEAD_DIM = 128
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _stream(device) -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _check_qkv(q, k, v):
+    if not (q.is_cuda and k.is_cuda and v.is_cuda):
+        raise RuntimeError("moba_attn_varlen needs tensors on an AMD GPU (there is no CPU path)")
+    if q.dtype != torch.bfloat16 or k.dtype != q.dtype or v.dtype != q.dtype:
+        raise TypeError("moba_attn_varlen supports bfloat16 q, k, v")
+    if q.dim() != 3 or q.shape != k.shape or q.shape != v.shape:
+        raise ValueError("q, k, v must all be [seqlen, heads, head_dim] with the same number of heads")
+    if q.shape[2] != HEAD_DIM:
+        raise ValueError(f"head_dim must be {HEAD_DIM}")
+
+
+# ----------------------------------------------------------------------------- stages
+def chunk_mean(k: torch.Tensor, plan: MobaPlan) -> torch.Tensor:
+    """kbar [F, H, D] bf16: mean of K over every filtered chunk (exact sum, rounded once)."""
+    lib = _lib.load()
+    S, H, D = k.shape
+    kbar = torch.empty((plan.F, H, D), dtype=k.dtype, device=k.device)
+    nbytes = lib.moba_chunk_mean_workspace_bytes(H, D, plan.F, plan.chunk_size)
+    ws = torch.empty(nbytes // 8, dtype=torch.float64, device=k.device)
+    _lib.check(lib.moba_chunk_mean(_ptr(k), _ptr(plan.tables["fchunk_tok"]), _ptr(kbar), _ptr(ws), S, H, D, plan.F,
+                                   plan.chunk_size, _stream(k.device)), "moba_chunk_mean")
+    return kbar
+
+
+def gate_topk(q: torch.Tensor, kbar: torch.Tensor, plan: MobaPlan, return_scores: bool = False):
+    """sel [S, H, K] int32: selected filtered-chunk ids per (token, head), -1 padded."""
+    lib = _lib.load()
+    S, H, D = q.shape
+    sel = torch.empty((S, H, plan.K), dtype=torch.int32, device=q.device)
+    scores = None
+    if return_scores:
+        scores = torch.full((S, H, plan.F), float("-inf"), dtype=torch.float32, device=q.device)
+    _lib.check(lib.moba_gate_topk(_ptr(q), _ptr(kbar), _ptr(plan.tables["cu_seqlens"]), _ptr(plan.tables["seq_fbase"]),
+                                  _ptr(sel), _ptr(scores), S, H, D, plan.nseq, plan.F, plan.chunk_size, plan.K,
+                                  _stream(q.device)), "moba_gate_topk")
+    return (sel, scores) if return_scores else sel
+
+
+def topk_from_scores(scores: torch.Tensor, K: int) -> torch.Tensor:
+    """Selection stage alone on caller-supplied fp32 scores [S, H, F] (-inf = not a candidate)."""
+    lib = _lib.load()
+    S, H, F = scores.shape
+    scores = scores.contiguous()
+    sel = torch.empty((S, H, K), dtype=torch.int32, device=scores.device)
+    _lib.check(lib.moba_topk_from_scores(_ptr(scores), _ptr(sel), S, H, F, K, _stream(scores.device)),
+               "moba_topk_from_scores")
+    return sel
+
+
+def build_lists(sel: torch.Tensor, plan: MobaPlan):
+    """(seg_off [F*H+1], tile_off [F*H+1], seg_dest [M]) int32 -- see csrc/lists.hip."""
+    lib = _lib.load()
+    S, H, K = sel.shape
+    dev = sel.device
+    M = plan.pairs_per_head * H
+    cnt = torch.empty(plan.P * H + 1, dtype=torch.int32, device=dev)
+    seg_off = torch.empty(plan.F * H + 1, dtype=torch.int32, device=dev)
+    tile_off = torch.empty(plan.F * H + 1, dtype=torch.int32, device=dev)
+    seg_dest = torch.empty(max(M, 1), dtype=torch.int32, device=dev)
+    t = plan.tables
+    _lib.check(lib.moba_build_lists(_ptr(sel), _ptr(t["chunk_tok"]), _ptr(t["chunk_fb"]), _ptr(t["chunk_local"]),
+                                    _ptr(t["pair_off"]), _ptr(cnt), _ptr(seg_off), _ptr(tile_off), _ptr(seg_dest),
+                                    S, H, K, plan.N, plan.F, plan.P, plan.cmax, TILE_ROWS, _stream(dev)),
+               "moba_build_lists")
+    return seg_off, tile_off, seg_dest
+
+
+def _forward(q, k, v, plan: MobaPlan):
+    lib = _lib.load()
+    S, H, D = q.shape
+    dev = q.device
+    K = plan.K
+    t = plan.tables
+    if plan.fallback:
+        sel = seg_off = tile_off = seg_dest = None
+    else:
+        kbar = chunk_mean(k, plan)
+        sel = gate_topk(q, kbar, plan)
+        seg_off, tile_off, seg_dest = build_lists(sel, plan)
+    part_o = torch.empty((S * H * (K + 1), D), dtype=q.dtype, device=dev)
+    part_lse = torch.empty((S * H * (K + 1),), dtype=torch.float32, device=dev)
+    out = torch.empty_like(q)
+    lse = torch.empty((S, H), dtype=torch.float32, device=dev)
+    _lib.check(lib.moba_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(part_o), _ptr(part_lse), _ptr(sel), _ptr(seg_off),
+                            _ptr(tile_off), _ptr(seg_dest), _ptr(t.get("fchunk_tok")), _ptr(t["chunk_tok"]),
+                            _ptr(t["self_tile_prefix"]), _ptr(out), _ptr(lse), S, H, D, K, plan.F, plan.N,
+                            plan.chunk_size, plan.hist_tile_bound(H), plan.self_tiles, _stream(dev)), "moba_fwd")
+    return out, lse, sel, seg_off, tile_off, seg_dest
+
+
+def _backward(dout, q, k, v, out, lse, sel, seg_off, tile_off, seg_dest, plan: MobaPlan):
+    lib = _lib.load()
+    if not hasattr(lib, "moba_bwd"):
+        raise RuntimeError("libmoba_hip.so was built without the backward kernels")
+    S, H, D = q.shape
+    dev = q.device
+    K = plan.K
+    t = plan.tables
+    dq = torch.empty_like(q)
+    dk = torch.empty_like(k)
+    dv = torch.empty_like(v)
+    delta = torch.empty((S, H), dtype=torch.float32, device=dev)
+    part_dq = torch.empty((S * H * (K + 1), D), dtype=torch.float32, device=dev)
+    _lib.check(lib.moba_bwd(_ptr(dout), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(sel), _ptr(seg_off),
+                            _ptr(tile_off), _ptr(seg_dest), _ptr(t.get("fchunk_tok")), _ptr(t["chunk_tok"]),
+                            _ptr(t["self_tile_prefix"]), _ptr(t.get("chunk_fb")), _ptr(t.get("chunk_local")),
+                            _ptr(delta), _ptr(part_dq), _ptr(dq), _ptr(dk), _ptr(dv),
+                            S, H, D, K, plan.F, plan.N, plan.chunk_size, plan.hist_tile_bound(H), plan.self_tiles,
+                            _stream(dev)), "moba_bwd")
+    return dq, dk, dv
+
+
+class _MobaAttention(torch.autograd.Function):
+    """Counterpart of ``MixedAttention`` (moba/moba_efficient.py:67-267)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, plan):
+        out, lse, sel, seg_off, tile_off, seg_dest = _forward(q, k, v, plan)
+        ctx.plan = plan
+        ctx.aux = (sel, seg_off, tile_off, seg_dest)
+        ctx.save_for_backward(q, k, v, out, lse)
+        ctx.mark_non_differentiable(lse)
+        return out, lse
+
+    @staticmethod
+    def backward(ctx, dout, _dlse):
+        q, k, v, out, lse = ctx.saved_tensors
+        sel, seg_off, tile_off, seg_dest = ctx.aux
+        dq, dk, dv = _backward(dout.contiguous(), q, k, v, out, lse, sel, seg_off, tile_off, seg_dest, ctx.plan)
+        return dq, dk, dv, None
+
+
+def moba_attn_varlen(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    cu_seqlens: torch.Tensor,
+    max_seqlen: int,
+    moba_chunk_size: int,
+    moba_topk: int,
+) -> torch.Tensor:
+    """Mixture-of-block attention over a packed batch.
+
+    Args (as moba/moba_efficient.py:270-297):
+        q, k, v: [seqlen, heads, head_dim] bf16, same number of heads
+        cu_seqlens: int32 cumulative sequence lengths, starting at 0 and ending at seqlen
+        max_seqlen: longest sequence (accepted for signature compatibility; sizes come from cu_seqlens)
+        moba_chunk_size, moba_topk: block size and number of attended blocks (the current one included)
+    Returns:
+        [seqlen, heads, head_dim] in q's dtype.  Softmax scale is head_dim ** -0.5.
+    """
+    return moba_attn_varlen_with_lse(q, k, v, cu_seqlens, max_seqlen, moba_chunk_size, moba_topk)[0]
+
+
+def moba_attn_varlen_with_lse(q, k, v, cu_seqlens, max_seqlen, moba_chunk_size, moba_topk):
+    """As ``moba_attn_varlen`` but also returns the natural-log LSE [seqlen, heads] fp32."""
+    _check_qkv(q, k, v)
+    plan = make_plan(cu_seqlens, moba_chunk_size, moba_topk, device=q.device)
+    if plan.S != q.shape[0]:
+        raise ValueError(f"cu_seqlens ends at {plan.S} but q has {q.shape[0]} tokens")
+    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    return _MobaAttention.apply(q, k, v, plan)

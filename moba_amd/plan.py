@@ -1,0 +1,135 @@
+"""Chunk metadata of a packed batch, computed on the host from ``cu_seqlens``.
+
+Counterpart of ``calc_chunks`` (moba/moba_efficient.py:14-64) plus everything else
+that depends only on the sequence lengths: buffer sizes, tile counts and the small
+int32 tables the kernels index.  All sizes are data independent (a token in the c-th
+chunk of its sequence selects exactly min(k, c) history chunks), so one device-to-host
+read of ``cu_seqlens`` is the only synchronisation of a forward call; plans are cached
+per (tensor identity, tensor version, chunk size, top-k).
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Tuple
+
+import numpy as np
+import torch
+
+TILE_ROWS = 128  # query rows per workgroup of the attention kernels
+
+
+@dataclass
+class MobaPlan:
+    cu: List[int]
+    chunk_size: int
+    moba_topk: int
+    S: int
+    nseq: int
+    N: int              # chunks
+    F: int              # filtered chunks (possible history chunks)
+    k_eff: int          # min(moba_topk - 1, F)   (moba/moba_efficient.py:314)
+    K: int              # slots per (token, head): min(k_eff, most history chunks any token has)
+    fallback: bool      # k_eff <= 0: full causal attention (moba/moba_efficient.py:318-321)
+    P: int              # (filtered chunk, later chunk of the same sequence) pairs
+    cmax: int           # max chunks per sequence minus one
+    pairs_per_head: int  # selected (token, chunk) pairs per head  (M / H)
+    self_tiles: int     # row tiles of the self part, per head
+    flops_per_head: float
+    tables: Dict[str, torch.Tensor] = field(default_factory=dict)
+    host: Dict[str, np.ndarray] = field(default_factory=dict)
+
+    def hist_tile_bound(self, H: int) -> int:
+        return (self.pairs_per_head * H) // TILE_ROWS + self.F * H
+
+
+def _host_tables(cu: np.ndarray, B: int, topk: int):
+    lens = np.diff(cu)
+    nseq = lens.size
+    n_chunks = (lens + B - 1) // B
+    F = int((n_chunks - 1).sum())
+    k_eff = min(topk - 1, F)
+    fallback = k_eff <= 0
+    if fallback:
+        # one "chunk" per sequence: the self part alone is full causal attention
+        n_chunks = np.ones_like(n_chunks)
+        chunk_tok = cu.copy()
+        chunk_len = lens
+    else:
+        seq_of_chunk = np.repeat(np.arange(nseq), n_chunks)
+        cbase = np.concatenate([[0], np.cumsum(n_chunks)])[:-1]
+        local = np.arange(int(n_chunks.sum())) - cbase[seq_of_chunk]
+        chunk_start = cu[seq_of_chunk] + local * B
+        chunk_len = np.minimum(B, cu[seq_of_chunk + 1] - chunk_start)
+        chunk_tok = np.concatenate([chunk_start, [cu[-1]]])
+    N = int(n_chunks.sum())
+    tiles = (chunk_len + TILE_ROWS - 1) // TILE_ROWS
+    self_tile_prefix = np.concatenate([[0], np.cumsum(tiles)])
+    out = dict(chunk_tok=chunk_tok, self_tile_prefix=self_tile_prefix)
+    info = dict(nseq=nseq, N=N, F=0 if fallback else F, k_eff=k_eff, fallback=fallback, K=0, P=0, cmax=0,
+                pairs_per_head=0, self_tiles=int(tiles.sum()))
+    pairs_self = int((chunk_len.astype(np.int64) * (chunk_len + 1) // 2).sum())
+    if not fallback:
+        seq_fbase = np.concatenate([[0], np.cumsum(n_chunks - 1)])
+        is_last = local == n_chunks[seq_of_chunk] - 1
+        fidx = np.nonzero(~is_last)[0]
+        fchunk_tok = chunk_start[fidx]
+        nq = (n_chunks[seq_of_chunk] - 1 - local)[fidx]          # later chunks of the same sequence
+        pair_off = np.concatenate([[0], np.cumsum(nq)])
+        cmax = int(n_chunks.max() - 1)
+        K = min(k_eff, cmax)
+        pairs = int((chunk_len.astype(np.int64) * np.minimum(K, local)).sum())
+        out.update(seq_fbase=seq_fbase, fchunk_tok=fchunk_tok, chunk_fb=seq_fbase[seq_of_chunk], chunk_local=local,
+                   pair_off=pair_off)
+        info.update(K=K, P=int(nq.sum()), cmax=cmax, pairs_per_head=pairs)
+        flops = 4.0 * (pairs_self + pairs * B)
+    else:
+        flops = 4.0 * pairs_self
+    info["flops_per_head_per_d"] = flops
+    return out, info
+
+
+_CACHE: Dict[Tuple, MobaPlan] = {}
+
+
+def make_plan(cu_seqlens, chunk_size: int, moba_topk: int, device=None) -> MobaPlan:
+    """Build (or fetch) the plan for a batch.  ``cu_seqlens`` may be a device tensor (read
+    once, then cached on identity + version) or a Python sequence."""
+    key = None
+    if torch.is_tensor(cu_seqlens):
+        device = cu_seqlens.device if device is None else device
+        key = (cu_seqlens.data_ptr(), cu_seqlens._version, cu_seqlens.numel(), str(device), chunk_size, moba_topk)
+        hit = _CACHE.get(key)
+        if hit is not None:
+            return hit
+        cu = cu_seqlens.detach().to("cpu", torch.int64).numpy()
+    else:
+        cu = np.asarray(list(cu_seqlens), dtype=np.int64)
+    if cu.ndim != 1 or cu.size < 2:
+        raise ValueError("cu_seqlens must be a 1-D tensor with at least two entries")
+    if cu[0] != 0 or (np.diff(cu) <= 0).any():
+        raise ValueError("cu_seqlens must start at 0 and be strictly increasing (zero-length sequences are unsupported)")
+    if chunk_size <= 0 or moba_topk <= 0:
+        raise ValueError("moba_chunk_size and moba_topk must be positive")
+    host, info = _host_tables(cu, int(chunk_size), int(moba_topk))
+    plan = MobaPlan(cu=cu.tolist(), chunk_size=int(chunk_size), moba_topk=int(moba_topk), S=int(cu[-1]),
+                    nseq=info["nseq"], N=info["N"], F=info["F"], k_eff=info["k_eff"], K=info["K"],
+                    fallback=info["fallback"], P=info["P"], cmax=info["cmax"], pairs_per_head=info["pairs_per_head"],
+                    self_tiles=info["self_tiles"], flops_per_head=info["flops_per_head_per_d"], host=host)
+    if device is not None and torch.device(device).type != "cpu":
+        names = list(host)
+        flat = np.concatenate([host[n_].astype(np.int32) for n_ in names])
+        dev = torch.from_numpy(flat).to(device)
+        off = 0
+        for n_ in names:
+            plan.tables[n_] = dev[off:off + host[n_].size]
+            off += host[n_].size
+        if torch.is_tensor(cu_seqlens) and cu_seqlens.dtype == torch.int32 and cu_seqlens.is_contiguous():
+            plan.tables["cu_seqlens"] = cu_seqlens
+        else:
+            plan.tables["cu_seqlens"] = torch.from_numpy(cu.astype(np.int32)).to(device)
+    if key is not None:
+        if len(_CACHE) >= 16:
+            _CACHE.pop(next(iter(_CACHE)))
+        _CACHE[key] = plan
+    return plan

@@ -1,0 +1,79 @@
+"""transformers attention-interface adapter, mirroring moba/wrapper.py:29-84.
+
+Prefill (q_len == kv_len) converts the HF layout [batch, heads, seq, dim] to the packed
+varlen layout, expands KV heads to the query heads and calls the MoBA operator.
+Decode (q_len != kv_len) is full causal attention over the KV cache, as in the
+reference (moba/wrapper.py:76-82), done with PyTorch's scaled_dot_product_attention.
+"""
+
+from typing import Callable, Optional, Tuple
+
+import torch
+import torch.nn.functional as F
+
+from .config import MoBAConfig
+
+
+def hf_to_fa(x: torch.Tensor) -> torch.Tensor:
+    """[batch, heads, seqlen, head_dim] -> [batch * seqlen, heads, head_dim] (moba/wrapper.py:7-15)."""
+    b, h, s, d = x.shape
+    return x.transpose(1, 2).reshape(b * s, h, d)
+
+
+def fa_to_hf(x: torch.Tensor, batch: int) -> torch.Tensor:
+    """[batch * seqlen, heads, head_dim] -> [batch, heads, seqlen, head_dim] (moba/wrapper.py:18-26)."""
+    return x.view(batch, -1, x.shape[1], x.shape[2]).transpose(1, 2)
+
+
+def moba_layer(
+    moba_impl: Callable,
+    moba_config: MoBAConfig,
+    module: torch.nn.Module,
+    query: torch.Tensor,
+    key: torch.Tensor,
+    value: torch.Tensor,
+    *args,
+    dropout: float = 0.0,
+    scaling: Optional[float] = None,
+    **kwargs,
+) -> Tuple[torch.Tensor, None]:
+    """
+    Args:
+        query: [batch, q_heads, q_len, head_dim]
+        key, value: [batch, kv_heads, kv_len, head_dim]
+    Returns:
+        (attn_output, None); prefill output is [batch * q_len, q_heads, head_dim], which the
+        caller's reshape(batch, q_len, -1) absorbs exactly as with the reference
+        (moba/wrapper.py:83 leaves the conversion back commented out).
+    """
+    assert module.is_causal
+    batch, q_heads, q_len, head_dim = query.shape
+    _, kv_heads, kv_len, _ = key.shape
+    if q_len == kv_len:
+        q = hf_to_fa(query)
+        k = hf_to_fa(key)
+        v = hf_to_fa(value)
+        rep = q_heads // kv_heads
+        if rep > 1:
+            k = torch.repeat_interleave(k, rep, dim=1)
+            v = torch.repeat_interleave(v, rep, dim=1)
+        cu_seqlens = torch.arange(0, (batch + 1) * kv_len, kv_len, dtype=torch.int32, device=query.device)
+        out = moba_impl(
+            q=q,
+            k=k,
+            v=v,
+            cu_seqlens=cu_seqlens,
+            max_seqlen=kv_len,
+            moba_chunk_size=moba_config.moba_chunk_size,
+            moba_topk=moba_config.moba_topk,
+        )
+    else:
+        # decode: every cached key is visible to the new queries (bottom-right aligned causal mask)
+        mask = None
+        if q_len > 1:
+            qi = torch.arange(q_len, device=query.device)[:, None] + (kv_len - q_len)
+            mask = torch.arange(kv_len, device=query.device)[None, :] <= qi
+        out = F.scaled_dot_product_attention(query, key, value, attn_mask=mask, dropout_p=dropout, scale=scaling,
+                                             enable_gqa=q_heads != kv_heads)
+        out = out.transpose(1, 2)
+    return out, None

@@ -1,0 +1,52 @@
+"""Host-side chunk metadata (moba_amd/plan.py) against the oracle's calc_chunks and
+closed forms; runs without a GPU."""
+
+import numpy as np
+import pytest
+
+from oracle import moba_oracle as O
+from moba_amd.plan import make_plan, TILE_ROWS
+
+
+def rand_cu(rng, nseq, lo, hi):
+    return np.concatenate([[0], np.cumsum(rng.integers(lo, hi, size=nseq))]).tolist()
+
+
+@pytest.mark.parametrize("seed", range(20))
+def test_plan_tables_match_oracle(seed):
+    rng = np.random.default_rng(seed)
+    cu = rand_cu(rng, int(rng.integers(1, 6)), 1, 400)
+    B = int(rng.integers(1, 80))
+    topk = int(rng.integers(1, 6))
+    plan = make_plan(cu, B, topk)
+    m = O.calc_chunks(cu, B)
+    k = O.effective_topk(topk, m["num_filtered_chunk"])
+    assert plan.k_eff == k and plan.fallback == (k <= 0)
+    if plan.fallback:
+        assert plan.host["chunk_tok"].tolist() == cu
+        assert plan.N == len(cu) - 1 and plan.K == 0
+        return
+    assert plan.N == len(m["cu_chunk"]) - 1 and plan.F == m["num_filtered_chunk"]
+    assert plan.host["chunk_tok"].tolist() == m["cu_chunk"].tolist()
+    assert plan.host["fchunk_tok"].tolist() == m["cu_chunk"][m["filtered_chunk_indices"]].tolist()
+    assert plan.host["seq_fbase"][:-1].tolist() == m["first_filtered"].tolist()
+    assert plan.K == min(k, int(m["n_chunks"].max()) - 1)
+    assert plan.pairs_per_head == O.expected_pair_count(cu, B, k, 1)
+    assert plan.P == int(sum(n * (n - 1) // 2 for n in m["n_chunks"]))
+    assert plan.flops_per_head * 128 == pytest.approx(O.attention_flops(cu, B, topk, 1, 128))
+    lens = np.diff(m["cu_chunk"])
+    assert plan.self_tiles == int(((lens + TILE_ROWS - 1) // TILE_ROWS).sum())
+
+
+def test_plan_headline_config_sizes():
+    plan = make_plan([0, 131072], 4096, 12)
+    assert (plan.N, plan.F, plan.K, plan.P) == (32, 31, 11, 496)
+    assert plan.pairs_per_head * 32 == 37486592
+    assert plan.flops_per_head * 128 * 32 == pytest.approx(8.301e13, rel=1e-3)
+
+
+def test_plan_rejects_bad_input():
+    with pytest.raises(ValueError):
+        make_plan([0, 5, 5, 9], 4, 3)
+    with pytest.raises(ValueError):
+        make_plan([1, 5], 4, 3)
