@@ -1,0 +1,160 @@
+#!/usr/bin/env python3
+"""Benchmark of the MoBA attention path on one MI355X.
+
+A step is one forward pass of ``moba_attn_varlen`` (chunk-mean, gate + top-k, gather
+lists, fused attention, merge) over one synthetic batch already resident in HBM.
+The default workload is the headline configuration: one sequence of 131072 tokens,
+32 query heads (8 KV heads repeated to 32 before the operator, outside the timed
+region), head_dim 128, chunk 4096, top-k 12, bf16.
+
+Prints one JSON line: whole-operator effective TFLOP/s on the FLOPs actually required
+(4*D per attended query/key pair), ms per layer, the roofline figures of the dominant
+kernel measured with device events inside the timed region, per-stage times, and a CPU
+baseline (the dense-mask oracle on a bounded sample, timed on this host's cores).
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import random
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
+HBM_PEAK_GBS = 8000.0
+
+WORKLOADS = {
+    # name: (seq lens or None, heads, kv_heads, chunk, topk, normalise, backward)
+    "cfg1_L4096_h4_c512_k3": ([4096], 4, 4, 512, 3, False, False),
+    "cfg2_L32768_h1_c2048_k3": ([32768], 1, 1, 2048, 3, False, True),
+    "cfg3_varlen8_h32_c2048_k3": (None, 32, 32, 2048, 3, False, True),
+    "cfg4_L131072_h32_c4096_k12": ([131072], 32, 8, 4096, 12, True, False),
+    "cfg5_L1048576_h32_c4096_k12": ([1048576], 32, 8, 4096, 12, False, False),
+}
+DEFAULT = "cfg4_L131072_h32_c4096_k12"
+
+
+def make_inputs(name, device):
+    lens, H, Hkv, B, topk, normalise, _ = WORKLOADS[name]
+    if lens is None:
+        rng = random.Random(0)
+        lens = [rng.randint(4096, 65536) for _ in range(8)]
+    S = sum(lens)
+    g = torch.Generator(device=device).manual_seed(0)
+
+    def draw(h):
+        x = torch.randn((S, h, 128), generator=g, device=device, dtype=torch.float32)
+        if normalise:
+            x = x / x.pow(2).mean(dim=-1, keepdim=True).sqrt()
+        return x.to(torch.bfloat16)
+
+    q = draw(H)
+    k = draw(Hkv)
+    v = draw(Hkv)
+    if Hkv != H:  # the wrapper's repeat_kv (moba/wrapper.py:59-61), outside the timed region
+        k = torch.repeat_interleave(k, H // Hkv, dim=1).contiguous()
+        v = torch.repeat_interleave(v, H // Hkv, dim=1).contiguous()
+    cu = [0]
+    for L in lens:
+        cu.append(cu[-1] + L)
+    return q, k, v, cu, max(lens), B, topk
+
+
+def cpu_baseline(q, k, v, B, topk, budget_tokens=32768, heads=4):
+    """Dense-mask oracle (restatement of moba_naive) on the first ``budget_tokens`` tokens of
+    ``heads`` heads of the same data, one head at a time, on this host's cores."""
+    from oracle import moba_oracle as O
+
+    L = min(budget_tokens, q.shape[0])
+    heads = min(heads, q.shape[1])
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    dt = 0.0
+    for h in range(heads):
+        qc, kc, vc = (x[:L, h:h + 1].cpu().contiguous() for x in (q, k, v))
+        t0 = time.perf_counter()
+        O.moba_attn_varlen_naive(qc, kc, vc, [0, L], L, B, topk)
+        dt += time.perf_counter() - t0
+    flops = O.attention_flops([0, L], B, topk, heads, 128)
+    return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"{heads} heads x first {L} tokens of the same q/k/v, chunk {B}, top-k {topk}, dense-mask fp32 "
+                      f"algorithm of moba_naive, {dt:.1f} s"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default=DEFAULT, choices=list(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+
+    from moba_amd import moba_efficient as E
+    from moba_amd.plan import make_plan
+
+    dev = torch.device("cuda:0")
+    q, k, v, cu, max_seqlen, B, topk = make_inputs(args.workload, dev)
+    S, H, D = q.shape
+    cu_t = torch.tensor(cu, dtype=torch.int32, device=dev)
+    plan = make_plan(cu_t, B, topk)
+    flops = plan.flops_per_head * D * H
+
+    for _ in range(args.warmup):
+        E.moba_attn_varlen(q, k, v, cu_t, max_seqlen, B, topk)
+    torch.cuda.synchronize()
+    timer = E.StageTimer()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        E.moba_attn_varlen_with_lse(q, k, v, cu_t, max_seqlen, B, topk, timer=timer)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+    stage_ms = {name: sum(x) / len(x) for name, x in timer.ms().items()}
+
+    kern_ms = stage_ms["fwd_partials"]
+    achieved = flops / (kern_ms * 1e-3) / 1e12
+    result = {
+        "metric": "moba_fwd_effective_tflops_128k" if args.workload == DEFAULT else "moba_fwd_effective_tflops",
+        "value": flops / dt / 1e12,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": dt * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": args.workload, "tokens": S, "heads": H, "head_dim": D, "chunk": B, "topk": topk,
+                   "sequences": len(cu) - 1, "fwd_flops": flops},
+        "pct_mfma_peak_whole_op": 100.0 * flops / dt / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+        "stage_ms": stage_ms,
+        "roofline": {"kernel": "moba_fwd_kernel", "bound": "mfma", "achieved": achieved,
+                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
+                     "traffic": None},
+    }
+    if "chunk_mean" in stage_ms:
+        gbs = S * H * D * 2 / (stage_ms["chunk_mean"] * 1e-3) / 1e9
+        result["chunk_mean_hbm"] = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                    "frac": gbs / HBM_PEAK_GBS}
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(q, k, v, B, topk)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

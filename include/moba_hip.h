@@ -1,0 +1,103 @@
+/* C ABI of libmoba_hip.so: the MI355X (gfx950) kernels behind moba_attn_varlen.
+ *
+ * The reference (MoonshotAI/MoBA) has no native code: its hot path is torch ops plus
+ * the private varlen entry points of the flash-attn wheel.  Each entry point below
+ * names the reference lines whose arithmetic it replaces.  All pointers are device
+ * pointers unless stated otherwise; tensors are contiguous; `stream` is a hipStream_t.
+ * The library allocates nothing, frees nothing, and never synchronises the device:
+ * every launch is enqueued on `stream`.  Return value: 0, or a negative code that
+ * moba_strerror() explains.  bf16 data, head_dim 128.
+ *
+ * Shapes use: S packed tokens, H heads, D head_dim, B chunk size, N chunks,
+ * F filtered chunks (chunks that are not the last of their sequence), K selected
+ * history chunks per (token, head), M = number of selected (token, head, chunk)
+ * triples, P = number of (filtered chunk, later chunk of the same sequence) pairs.
+ */
+#ifndef MOBA_HIP_H
+#define MOBA_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+int moba_version(void);
+const char* moba_strerror(int code);
+
+/* Key chunk-mean.  Replaces moba/moba_efficient.py:326-340 (index_select of the
+ * filtered chunks, .mean(dim=1) on bf16, .float()).
+ *   k          [S,H,D] bf16
+ *   fchunk_tok [F] int32, first token of each filtered chunk
+ *   kbar       [F,H,D] bf16 out
+ *   workspace  moba_chunk_mean_workspace_bytes() bytes, 8-byte aligned */
+size_t moba_chunk_mean_workspace_bytes(int H, int D, int F, int B);
+int moba_chunk_mean(const void* k, const int32_t* fchunk_tok, void* kbar, void* workspace, int64_t S, int H, int D,
+                    int F, int B, void* stream);
+
+/* Gate scores + causal top-k.  Replaces moba/moba_efficient.py:341-371 (fp32 einsum,
+ * -inf mask, torch.topk, dropping -inf picks).
+ *   cu_seqlens [nseq+1] int32; seq_fbase [nseq+1] int32, first filtered id of each sequence
+ *   sel        [S,H,K] int32 out: filtered-chunk ids, descending score, -1 padded
+ *   scores_out optional [S,H,F] fp32, pre-filled with -inf by the caller; receives the
+ *              score of every valid candidate (debug / test output), may be NULL
+ * K <= 64. */
+int moba_gate_topk(const void* q, const void* kbar, const int32_t* cu_seqlens, const int32_t* seq_fbase, int32_t* sel,
+                   float* scores_out, int64_t S, int H, int D, int nseq, int F, int B, int K, void* stream);
+
+/* The selection step of moba/moba_efficient.py:365-371 alone, on caller-supplied
+ * scores [S,H,F] fp32 (-inf = not a candidate).  Same routine as moba_gate_topk. */
+int moba_topk_from_scores(const float* scores, int32_t* sel, int64_t S, int H, int F, int K, void* stream);
+
+/* Varlen gather lists.  Replaces moba/moba_efficient.py:373-423 (nonzero, per-segment
+ * counts, gathered q and kv copies): index lists only, in the same (chunk, head, token)
+ * order.
+ *   chunk_tok [N+1], chunk_fb [N] (first filtered id of the chunk's sequence),
+ *   chunk_local [N] (index of the chunk inside its sequence), pair_off [F+1]
+ *   (prefix sum of the number of later chunks in the same sequence)   -- int32 tables
+ *   cnt      [P*H+1] int32 scratch
+ *   seg_off  [F*H+1] out, list start of segment (f,h);  tile_off [F*H+1] out, prefix
+ *            sum of ceil(rows/tile_rows);  seg_dest [M] out, entries
+ *            (token*H + h)*(K+1) + 1 + slot
+ * cmax = most chunks in a sequence minus one. */
+int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, const int32_t* chunk_fb, const int32_t* chunk_local,
+                     const int32_t* pair_off, int32_t* cnt, int32_t* seg_off, int32_t* tile_off, int32_t* seg_dest,
+                     int64_t S, int H, int K, int N, int F, int P, int cmax, int tile_rows, void* stream);
+
+/* Attention.  Replaces MixedAttention.forward, moba/moba_efficient.py:69-183 (two
+ * flash-attn varlen forwards and the LSE merge), and with K = 0 and one chunk per
+ * sequence the full-causal case of moba/moba_efficient.py:318-321.
+ *   part_o [S*H*(K+1), D] bf16 and part_lse [S*H*(K+1)] fp32: per-slot partial results
+ *   self_tile_prefix [N+1] int32: prefix sum of ceil(chunk_len / moba_fwd_tile_rows())
+ *   out [S,H,D] bf16, lse [S,H] fp32 (natural log)
+ *   hist_bound: upper bound on the number of history tiles, e.g. M/tile_rows + F*H
+ *   self_tiles: self_tile_prefix[N] */
+int moba_fwd_tile_rows(void);
+int moba_fwd_partials(const void* q, const void* k, const void* v, void* part_o, float* part_lse,
+                      const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest,
+                      const int32_t* fchunk_tok, const int32_t* chunk_tok, const int32_t* self_tile_prefix, int64_t S,
+                      int H, int D, int K, int F, int N, int B, int64_t hist_bound, int64_t self_tiles, void* stream);
+int moba_fwd_merge(const void* part_o, const float* part_lse, const int32_t* sel, void* out, float* lse, int64_t S,
+                   int H, int D, int K, void* stream);
+int moba_fwd(const void* q, const void* k, const void* v, void* part_o, float* part_lse, const int32_t* sel,
+             const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest, const int32_t* fchunk_tok,
+             const int32_t* chunk_tok, const int32_t* self_tile_prefix, void* out, float* lse, int64_t S, int H, int D,
+             int K, int F, int N, int B, int64_t hist_bound, int64_t self_tiles, void* stream);
+
+/* Backward.  Replaces MixedAttention.backward, moba/moba_efficient.py:185-267, and the
+ * autograd scatter of its gathered gradients.  Deterministic (no floating-point atomics).
+ *   dout, q, k, v, out [S,H,D] bf16; lse [S,H] fp32 from the forward
+ *   delta [S,H] fp32 scratch; part_dq [S*H*(K+1), D] fp32 scratch
+ *   dq, dk, dv [S,H,D] bf16 out */
+int moba_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out, const float* lse,
+             const int32_t* sel, const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest,
+             const int32_t* fchunk_tok, const int32_t* chunk_tok, const int32_t* self_tile_prefix,
+             const int32_t* chunk_fb, const int32_t* chunk_local, float* delta, float* part_dq, void* dq, void* dk,
+             void* dv, int64_t S, int H, int D, int K, int F, int N, int B, int64_t hist_bound, int64_t self_tiles,
+             void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

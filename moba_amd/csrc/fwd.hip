@@ -313,20 +313,18 @@ using namespace moba;
 extern "C" int moba_fwd_tile_rows(void) { return TM; }
 
 // hist_bound: any upper bound on the number of history tiles (floor(M/128) + F*H is one).
-extern "C" int moba_fwd(const void* q, const void* k, const void* v, void* part_o, float* part_lse,
-                        const int32_t* sel, const int32_t* seg_off, const int32_t* tile_off,
-                        const int32_t* seg_dest, const int32_t* fchunk_tok, const int32_t* chunk_tok,
-                        const int32_t* self_tile_prefix, void* out, float* lse, int64_t S, int H, int D, int K,
-                        int F, int N, int B, int64_t hist_bound, int64_t self_tiles, void* stream) {
-  if (!q || !k || !v || !part_o || !part_lse || !chunk_tok || !self_tile_prefix || !out || !lse) return MOBA_ERR_ARG;
-  if (K > 0 && (!sel || !seg_off || !tile_off || !seg_dest || !fchunk_tok)) return MOBA_ERR_ARG;
+extern "C" int moba_fwd_partials(const void* q, const void* k, const void* v, void* part_o, float* part_lse,
+                                 const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest,
+                                 const int32_t* fchunk_tok, const int32_t* chunk_tok,
+                                 const int32_t* self_tile_prefix, int64_t S, int H, int D, int K, int F, int N, int B,
+                                 int64_t hist_bound, int64_t self_tiles, void* stream) {
+  if (!q || !k || !v || !part_o || !part_lse || !chunk_tok || !self_tile_prefix) return MOBA_ERR_ARG;
+  if (K > 0 && (!seg_off || !tile_off || !seg_dest || !fchunk_tok)) return MOBA_ERR_ARG;
   if (D != kHeadDim) return MOBA_ERR_UNSUPPORTED;
   if (S <= 0 || H <= 0 || K < 0 || F < 0 || N <= 0 || B <= 0 || hist_bound < 0 || self_tiles <= 0) return MOBA_ERR_ARG;
-  if (((uintptr_t)q & 15) || ((uintptr_t)k & 15) || ((uintptr_t)v & 15) || ((uintptr_t)part_o & 15) ||
-      ((uintptr_t)out & 15))
-    return MOBA_ERR_ARG;
+  if (((uintptr_t)q & 15) || ((uintptr_t)k & 15) || ((uintptr_t)v & 15) || ((uintptr_t)part_o & 15)) return MOBA_ERR_ARG;
   if ((int64_t)S * H * (K + 1) >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
-  const int64_t total = hist_bound + self_tiles * H;
+  const int64_t total = (K > 0 ? hist_bound : 0) + self_tiles * H;
   const int64_t grid = (total + 8 * kXcdBlock - 1) / (8 * kXcdBlock) * (8 * kXcdBlock);
   if (grid >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
   FwdParams p;
@@ -347,8 +345,28 @@ extern "C" int moba_fwd(const void* q, const void* k, const void* v, void* part_
     attr_set = true;
   }
   hipLaunchKernelGGL(moba_fwd_kernel, dim3((unsigned)grid), dim3(256), kFwdLds, st, p);
-  const int64_t rows = S * H;
-  hipLaunchKernelGGL(moba_merge_kernel, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st, (const bf16*)part_o,
-                     (const float*)part_lse, sel, (bf16*)out, lse, rows, K + 1);
   return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
+}
+
+extern "C" int moba_fwd_merge(const void* part_o, const float* part_lse, const int32_t* sel, void* out, float* lse,
+                              int64_t S, int H, int D, int K, void* stream) {
+  if (!part_o || !part_lse || !out || !lse || (K > 0 && !sel)) return MOBA_ERR_ARG;
+  if (D != kHeadDim) return MOBA_ERR_UNSUPPORTED;
+  if (S <= 0 || H <= 0 || K < 0 || ((uintptr_t)part_o & 15) || ((uintptr_t)out & 15)) return MOBA_ERR_ARG;
+  const int64_t rows = S * H;
+  hipLaunchKernelGGL(moba_merge_kernel, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, (hipStream_t)stream,
+                     (const bf16*)part_o, part_lse, sel, (bf16*)out, lse, rows, K + 1);
+  return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
+}
+
+// Whole attention stage: partial attentions of every tile, then the merge.
+extern "C" int moba_fwd(const void* q, const void* k, const void* v, void* part_o, float* part_lse,
+                        const int32_t* sel, const int32_t* seg_off, const int32_t* tile_off,
+                        const int32_t* seg_dest, const int32_t* fchunk_tok, const int32_t* chunk_tok,
+                        const int32_t* self_tile_prefix, void* out, float* lse, int64_t S, int H, int D, int K,
+                        int F, int N, int B, int64_t hist_bound, int64_t self_tiles, void* stream) {
+  int rc = moba_fwd_partials(q, k, v, part_o, part_lse, seg_off, tile_off, seg_dest, fchunk_tok, chunk_tok,
+                             self_tile_prefix, S, H, D, K, F, N, B, hist_bound, self_tiles, stream);
+  if (rc != MOBA_OK) return rc;
+  return moba_fwd_merge(part_o, part_lse, sel, out, lse, S, H, D, K, stream);
 }

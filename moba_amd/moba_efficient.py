@@ -99,26 +99,72 @@ def build_lists(sel: torch.Tensor, plan: MobaPlan):
     return seg_off, tile_off, seg_dest
 
 
-def _forward(q, k, v, plan: MobaPlan):
+class StageTimer:
+    """Optional per-stage device timing: events are recorded on the launch stream around
+    each stage, so reading them never perturbs the launches themselves."""
+
+    def __init__(self):
+        self.events = {}
+
+    def span(self, name, device):
+        timer = self
+
+        class _Span:
+            def __enter__(self_inner):
+                self_inner.a = torch.cuda.Event(enable_timing=True)
+                self_inner.b = torch.cuda.Event(enable_timing=True)
+                self_inner.a.record(torch.cuda.current_stream(device))
+                return self_inner
+
+            def __exit__(self_inner, *exc):
+                self_inner.b.record(torch.cuda.current_stream(device))
+                timer.events.setdefault(name, []).append((self_inner.a, self_inner.b))
+                return False
+
+        return _Span()
+
+    def ms(self):
+        """stage -> list of elapsed milliseconds (call after a synchronize)."""
+        return {k: [a.elapsed_time(b) for a, b in v] for k, v in self.events.items()}
+
+
+class _NoSpan:
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        return False
+
+
+def _forward(q, k, v, plan: MobaPlan, timer: Optional[StageTimer] = None):
     lib = _lib.load()
     S, H, D = q.shape
     dev = q.device
     K = plan.K
     t = plan.tables
+    span = (lambda name: timer.span(name, dev)) if timer is not None else (lambda name: _NoSpan())
     if plan.fallback:
         sel = seg_off = tile_off = seg_dest = None
     else:
-        kbar = chunk_mean(k, plan)
-        sel = gate_topk(q, kbar, plan)
-        seg_off, tile_off, seg_dest = build_lists(sel, plan)
+        with span("chunk_mean"):
+            kbar = chunk_mean(k, plan)
+        with span("gate_topk"):
+            sel = gate_topk(q, kbar, plan)
+        with span("build_lists"):
+            seg_off, tile_off, seg_dest = build_lists(sel, plan)
     part_o = torch.empty((S * H * (K + 1), D), dtype=q.dtype, device=dev)
     part_lse = torch.empty((S * H * (K + 1),), dtype=torch.float32, device=dev)
     out = torch.empty_like(q)
     lse = torch.empty((S, H), dtype=torch.float32, device=dev)
-    _lib.check(lib.moba_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(part_o), _ptr(part_lse), _ptr(sel), _ptr(seg_off),
-                            _ptr(tile_off), _ptr(seg_dest), _ptr(t.get("fchunk_tok")), _ptr(t["chunk_tok"]),
-                            _ptr(t["self_tile_prefix"]), _ptr(out), _ptr(lse), S, H, D, K, plan.F, plan.N,
-                            plan.chunk_size, plan.hist_tile_bound(H), plan.self_tiles, _stream(dev)), "moba_fwd")
+    with span("fwd_partials"):
+        _lib.check(lib.moba_fwd_partials(_ptr(q), _ptr(k), _ptr(v), _ptr(part_o), _ptr(part_lse), _ptr(seg_off),
+                                         _ptr(tile_off), _ptr(seg_dest), _ptr(t.get("fchunk_tok")),
+                                         _ptr(t["chunk_tok"]), _ptr(t["self_tile_prefix"]), S, H, D, K, plan.F, plan.N,
+                                         plan.chunk_size, plan.hist_tile_bound(H), plan.self_tiles, _stream(dev)),
+                   "moba_fwd_partials")
+    with span("fwd_merge"):
+        _lib.check(lib.moba_fwd_merge(_ptr(part_o), _ptr(part_lse), _ptr(sel), _ptr(out), _ptr(lse), S, H, D, K,
+                                      _stream(dev)), "moba_fwd_merge")
     return out, lse, sel, seg_off, tile_off, seg_dest
 
 
@@ -148,8 +194,8 @@ class _MobaAttention(torch.autograd.Function):
     """Counterpart of ``MixedAttention`` (moba/moba_efficient.py:67-267)."""
 
     @staticmethod
-    def forward(ctx, q, k, v, plan):
-        out, lse, sel, seg_off, tile_off, seg_dest = _forward(q, k, v, plan)
+    def forward(ctx, q, k, v, plan, timer=None):
+        out, lse, sel, seg_off, tile_off, seg_dest = _forward(q, k, v, plan, timer)
         ctx.plan = plan
         ctx.aux = (sel, seg_off, tile_off, seg_dest)
         ctx.save_for_backward(q, k, v, out, lse)
@@ -161,7 +207,7 @@ class _MobaAttention(torch.autograd.Function):
         q, k, v, out, lse = ctx.saved_tensors
         sel, seg_off, tile_off, seg_dest = ctx.aux
         dq, dk, dv = _backward(dout.contiguous(), q, k, v, out, lse, sel, seg_off, tile_off, seg_dest, ctx.plan)
-        return dq, dk, dv, None
+        return dq, dk, dv, None, None
 
 
 def moba_attn_varlen(
@@ -186,11 +232,12 @@ def moba_attn_varlen(
     return moba_attn_varlen_with_lse(q, k, v, cu_seqlens, max_seqlen, moba_chunk_size, moba_topk)[0]
 
 
-def moba_attn_varlen_with_lse(q, k, v, cu_seqlens, max_seqlen, moba_chunk_size, moba_topk):
-    """As ``moba_attn_varlen`` but also returns the natural-log LSE [seqlen, heads] fp32."""
+def moba_attn_varlen_with_lse(q, k, v, cu_seqlens, max_seqlen, moba_chunk_size, moba_topk, timer=None):
+    """As ``moba_attn_varlen`` but also returns the natural-log LSE [seqlen, heads] fp32.
+    ``timer`` (a StageTimer) collects per-stage device times."""
     _check_qkv(q, k, v)
     plan = make_plan(cu_seqlens, moba_chunk_size, moba_topk, device=q.device)
     if plan.S != q.shape[0]:
         raise ValueError(f"cu_seqlens ends at {plan.S} but q has {q.shape[0]} tokens")
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
-    return _MobaAttention.apply(q, k, v, plan)
+    return _MobaAttention.apply(q, k, v, plan, timer)
