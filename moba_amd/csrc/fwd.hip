@@ -53,6 +53,23 @@ __device__ __forceinline__ bf16x4 lds_read_tr(const char* p) {
       (__attribute__((address_space(3))) bf16x4*)(p));
 }
 
+// asynchronous 16-byte copy global -> LDS: lane i of the wave fills lds_wave_base + 16*i.
+// Issued as inline assembly so that completion is tracked by the explicit wait_vmem()
+// before the tile barrier only (the copy must stay in flight across the compute phase).
+__device__ __forceinline__ void async_copy16(const void* gsrc, uint32_t lds_wave_base) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+               :
+               : "v"(gsrc), "s"(lds_wave_base)
+               : "memory", "m0");
+}
+__device__ __forceinline__ uint32_t lds_addr(const char* p) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
+}
+// wait until this wave's outstanding global loads (including global -> LDS copies) have landed
+__device__ __forceinline__ void wait_vmem() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
+constexpr float kRescaleThreshold = 8.f;  // log2 units: the running max may lag the true max by this much
+
 __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -119,42 +136,51 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams p) {
     for (int ks = 0; ks < 8; ++ks) bq[ks] = *reinterpret_cast<const bf16x8*>(src + 16 * ks);
   }
 
-  // ---- K/V tile loader: thread owns key (tid/16 + 16*i), 16-byte column tid%16 ----
-  const int ld_key = tid >> 4, ld_c16 = tid & 15;
-  const int64_t row_elems = (int64_t)H * kHeadDim;
-  const bf16* kbase = p.k + (int64_t)h * kHeadDim + ld_c16 * 8;
-  const bf16* vbase = p.v + (int64_t)h * kHeadDim + ld_c16 * 8;
-  bf16x8 kreg[4], vreg[4];
-  auto load_tile = [&](int kt) {
+  // ---- K/V tile loader: global -> LDS without passing through registers.
+  // A wave copy fills 1 KiB = 4 keys x 16 columns of 16 bytes; wave w issues slabs
+  // w, w+4, w+8, w+12 of K and of V.  Lane i lands at slab + 16*i, so the lane picks the
+  // global column whose swizzled LDS position is i.
+  const int64_t row_bytes = (int64_t)H * kHeadDim * 2;
+  const uint32_t lds_base = lds_addr(smem);
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  const int ld_kin = lane >> 4;                     // key within the slab
+  const int ld_pc = lane & 15;                      // physical 16-byte column
+  auto issue_tile = [&](int kt, int buf) {
+    const uint32_t kdst = lds_base + buf * kTileBytes;
+    const uint32_t vdst = lds_base + (2 + buf) * kTileBytes;
+    const int key0 = kt * TN;
+    const bool full = (key0 + TN <= nkeys) && (kv_tok0 + key0 + TN <= p.S);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int key = kt * TN + ld_key + 16 * i;
-      const bool ok = key < nkeys;
-      const int64_t t = min(kv_tok0 + key, p.S - 1);
-      bf16x8 kk = *reinterpret_cast<const bf16x8*>(kbase + t * row_elems);
-      bf16x8 vv = *reinterpret_cast<const bf16x8*>(vbase + t * row_elems);
-      if (!ok) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) { kk[e] = (bf16)0.f; vv[e] = (bf16)0.f; }
-      }
-      kreg[i] = kk;
-      vreg[i] = vv;
+      const int slab = 4 * i + wave_u;
+      const int key = 4 * slab + ld_kin;            // key within the tile
+      const int kc16 = ld_pc ^ (key & 15);
+      const int vc16 = ((((ld_pc >> 2) ^ (key & 3))) << 2) | (ld_pc & 3);
+      int64_t t = kv_tok0 + key0 + key;
+      if (!full) t = min(t, (int64_t)p.S - 1);
+      const char* krow = (const char*)p.k + t * row_bytes + h * (kHeadDim * 2);
+      const char* vrow = (const char*)p.v + t * row_bytes + h * (kHeadDim * 2);
+      async_copy16(krow + kc16 * 16, kdst + slab * 1024);
+      async_copy16(vrow + vc16 * 16, vdst + slab * 1024);
     }
   };
-  auto store_tile = [&](int buf) {
-    char* ks = smem + buf * kTileBytes;
-    char* vs = smem + (2 + buf) * kTileBytes;
+  // rows of V past the end of the key range must not reach the MFMA (0 * NaN): clear them
+  auto scrub_tile = [&](int kt, int buf) {
+    const int key0 = kt * TN;
+    if (key0 + TN <= nkeys) return;
+    char* vdst = smem + (2 + buf) * kTileBytes;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int key = ld_key + 16 * i;
-      *reinterpret_cast<bf16x8*>(ks + k_lds_off(key, ld_c16)) = kreg[i];
-      *reinterpret_cast<bf16x8*>(vs + v_lds_off(key, ld_c16)) = vreg[i];
+      const int slab = 4 * i + wave;
+      const int key = 4 * slab + ld_kin;
+      if (key0 + key >= nkeys) *reinterpret_cast<u32x4*>(vdst + slab * 1024 + lane * 16) = u32x4{0, 0, 0, 0};
     }
   };
 
   const int nkt = (nkeys + TN - 1) / TN;
-  load_tile(0);
-  store_tile(0);
+  issue_tile(0, 0);
+  wait_vmem();
+  scrub_tile(0, 0);
   __syncthreads();
 
   f32x16 oacc[4];
@@ -165,31 +191,45 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams p) {
   float m_run = -INFINITY, l_run = 0.f;
   const float sl2 = p.scale_log2;
 
-  // per-lane pieces of the V^T fragment address
+  // per-lane pieces of the fragment addresses
   const int g16 = lane >> 4, i0 = (lane & 15) >> 2, i1 = lane & 3;
   const int v_lane_off = 32 * (g16 & 1) + 8 * i1;
+  int k_frag_off[2];
+#pragma unroll
+  for (int kb = 0; kb < 2; ++kb) k_frag_off[kb] = (32 * kb + n) * 256;
+  const int k_sw = n & 15;  // (32*kb + n) & 15
 
   for (int kt = 0; kt < nkt; ++kt) {
     const int buf = kt & 1;
     const bool has_next = kt + 1 < nkt;
-    if (has_next) load_tile(kt + 1);
+    if (has_next) issue_tile(kt + 1, buf ^ 1);
 
     if (kt * TN <= wave_max_limit) {  // wave-uniform: skip tiles entirely above the diagonal
       const char* ks = smem + buf * kTileBytes;
       const char* vs = smem + (2 + buf) * kTileBytes;
-      // S^T (keys x queries), two 32-key blocks
+      // S^T (keys x queries), two 32-key blocks: fetch all K fragments, then two
+      // interleaved accumulation chains
+      bf16x8 ka[2][8];
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int s8 = 0; s8 < 8; ++s8)
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+          ka[kb][s8] = *reinterpret_cast<const bf16x8*>(ks + k_frag_off[kb] + (((2 * s8 + hh) ^ k_sw) << 4));
       f32x16 sacc[2];
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
+      for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
         for (int e = 0; e < 16; ++e) sacc[kb][e] = 0.f;
-        const int key = 32 * kb + n;
 #pragma unroll
-        for (int s8 = 0; s8 < 8; ++s8) {
-          const bf16x8 a = *reinterpret_cast<const bf16x8*>(ks + k_lds_off(key, 2 * s8 + hh));
-          sacc[kb] = mfma32(a, bq[s8], sacc[kb]);
-        }
-      }
+      for (int s8 = 0; s8 < 8; ++s8)
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) sacc[kb] = mfma32(ka[kb][s8], bq[s8], sacc[kb]);
+      // keep all 16 LDS reads in flight ahead of the MFMA chain
+      __builtin_amdgcn_sched_group_barrier(0x100, 16, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 16, 0);
+      __builtin_amdgcn_sched_barrier(0);
+
       if (kt * TN + TN - 1 > wave_min_limit) {
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
@@ -199,31 +239,33 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams p) {
             if (key > limit) sacc[kb][e] = -INFINITY;
           }
       }
-      float mx = sacc[0][0];
+      float mx = fmaxf(sacc[0][0], sacc[1][0]);
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) mx = fmaxf(mx, sacc[kb][e]);
-      mx = fmaxf(mx, xhalf(mx));
-      const float m_new = fmaxf(m_run, mx * sl2);
-      const float alpha = fast_exp2(m_run - m_new);
-      m_run = m_new;
-      float rs = 0.f;
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const float pe = fast_exp2(sacc[kb][e] * sl2 - m_new);
-          sacc[kb][e] = pe;
-          rs += pe;
-        }
-      l_run = l_run * alpha + rs;
-      if (__any(alpha != 1.f)) {
+        for (int e = 1; e < 16; ++e) mx = fmaxf(mx, sacc[kb][e]);
+      mx = fmaxf(mx, xhalf(mx)) * sl2;
+      // lazy running max: move it only when the tile max exceeds it by the threshold
+      if (__any(mx > m_run + kRescaleThreshold)) {
+        const float m_new = fmaxf(m_run, mx);
+        const float alpha = fast_exp2(m_run - m_new);
+        m_run = m_new;
+        l_run *= alpha;
 #pragma unroll
         for (int db = 0; db < 4; ++db)
 #pragma unroll
           for (int e = 0; e < 16; ++e) oacc[db][e] *= alpha;
       }
+      float rs = 0.f;
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const float pe = fast_exp2(sacc[kb][e] * sl2 - m_run);
+          sacc[kb][e] = pe;
+          rs += pe;
+        }
+      l_run += rs;
       // P^T operand for the four 16-key steps
       bf16x8 pb[4];
 #pragma unroll
@@ -248,7 +290,10 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams p) {
         }
       }
     }
-    if (has_next) store_tile(buf ^ 1);
+    if (has_next) {
+      wait_vmem();
+      scrub_tile(kt + 1, buf ^ 1);
+    }
     __syncthreads();
   }
 
