@@ -88,14 +88,14 @@ int moba_fwd(const void* q, const void* k, const void* v, void* part_o, float* p
 /* Backward.  Replaces MixedAttention.backward, moba/moba_efficient.py:185-267, and the
  * autograd scatter of its gathered gradients.  Deterministic (no floating-point atomics).
  *   dout, q, k, v, out [S,H,D] bf16; lse [S,H] fp32 from the forward
+ *   chunk_fid [N] int32: filtered id of each chunk, -1 for the last chunk of a sequence
  *   delta [S,H] fp32 scratch; part_dq [S*H*(K+1), D] fp32 scratch
  *   dq, dk, dv [S,H,D] bf16 out */
 int moba_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out, const float* lse,
              const int32_t* sel, const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest,
              const int32_t* fchunk_tok, const int32_t* chunk_tok, const int32_t* self_tile_prefix,
-             const int32_t* chunk_fb, const int32_t* chunk_local, float* delta, float* part_dq, void* dq, void* dk,
-             void* dv, int64_t S, int H, int D, int K, int F, int N, int B, int64_t hist_bound, int64_t self_tiles,
-             void* stream);
+             const int32_t* chunk_fid, float* delta, float* part_dq, void* dq, void* dk, void* dv, int64_t S, int H,
+             int D, int K, int F, int N, int B, int64_t hist_bound, int64_t self_tiles, void* stream);
 
 #ifdef __cplusplus
 }

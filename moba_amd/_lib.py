@@ -28,9 +28,9 @@ _SIGNATURES = {
     "moba_fwd_partials": (c_int, [c_void_p] * 11 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_int64, c_void_p]),
     "moba_fwd_merge": (c_int, [c_void_p] * 5 + [c_int64, c_int, c_int, c_int, c_void_p]),
     "moba_fwd": (c_int, [c_void_p] * 14 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_int64, c_void_p]),
-    "moba_bwd": (c_int, [c_void_p] * 20 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_int64, c_void_p]),
+    "moba_bwd": (c_int, [c_void_p] * 19 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_int64, c_void_p]),
 }
-OPTIONAL = {"moba_bwd"}
+OPTIONAL = set()
 
 
 def load():

@@ -28,7 +28,7 @@ FLAGS = [
 def _compile(src: str, force: bool) -> str:
     path = os.path.join(CSRC, src)
     obj = os.path.join(OBJ, src.replace(".hip", ".o"))
-    deps = [path, os.path.join(CSRC, "common.h"), os.path.abspath(__file__)]
+    deps = [path, os.path.join(CSRC, "common.h"), os.path.join(CSRC, "attn_common.h"), os.path.abspath(__file__)]
     if not force and os.path.exists(obj) and all(os.path.getmtime(obj) > os.path.getmtime(d) for d in deps):
         return obj
     cmd = [HIPCC, *FLAGS, "-c", path, "-o", obj]

@@ -1,0 +1,127 @@
+// Pieces shared by the forward and backward attention kernels: the tile tables, the
+// decoding of a workgroup id into a tile of query rows, LDS swizzles and the
+// asynchronous global -> LDS copy.
+#pragma once
+#include "common.h"
+
+namespace moba {
+
+constexpr int TM = 128;  // query rows per workgroup (32 per wave)
+constexpr int TN = 64;   // keys per inner iteration
+constexpr int kTileBytes = TN * kHeadDim * 2;
+constexpr int kXcdBlock = 64;  // consecutive logical tiles that share an XCD
+
+// Index tables that define the tiles of one call.
+struct TileTables {
+  const int* seg_off;           // [F*H+1] list start of segment (f, h)
+  const int* tile_off;          // [F*H+1] prefix sum of row tiles per segment
+  const int* seg_dest;          // [M] (token*H + h)*K1 + 1 + slot
+  const int* fchunk_tok;        // [F] first token of filtered chunk f
+  const int* chunk_tok;         // [N+1] first token of every chunk
+  const int* self_tile_prefix;  // [N+1] prefix sum of row tiles per chunk
+  int S, H, K1, F, N, B;
+  int hist_bound;               // logical tile ids below it are history tiles
+  int self_total;               // self_tile_prefix[N] * H
+};
+
+// One tile of up to TM query rows of one head, as seen by a lane.
+struct Tile {
+  int h;          // head
+  int kv_tok0;    // token of key 0
+  int nkeys;      // keys the tile attends (before masking)
+  int row_count;  // valid rows
+  int dest;       // this lane's row: destination slot row (token*H + h)*K1 + slot
+  int tok;        // this lane's row: token
+  int limit;      // this lane's row attends keys <= limit
+  int wave_min_limit, wave_max_limit;  // over the wave's 32 rows
+};
+
+// Workgroup ids are dealt round-robin to the 8 XCDs; give each XCD runs of kXcdBlock
+// consecutive logical tiles so that tiles sharing a K/V chunk share an L2.
+__device__ __forceinline__ int logical_tile_id() {
+  const int x = blockIdx.x & 7, y = blockIdx.x >> 3;
+  return ((y / kXcdBlock) * 8 + x) * kXcdBlock + (y % kXcdBlock);
+}
+
+// r = row of this lane inside the tile (wave*32 + lane%32).  Returns false for ids past the end.
+__device__ __forceinline__ bool decode_tile(const TileTables& p, int logical, int wave, int r, Tile& t) {
+  const int H = p.H;
+  if (logical < p.hist_bound) {
+    const int FH = p.F * H;
+    if (FH == 0 || logical >= p.tile_off[FH]) return false;
+    const int seg = upper_row(p.tile_off, FH, logical);
+    const int tile = logical - p.tile_off[seg];
+    const int f = seg / H;
+    t.h = seg - f * H;
+    const int base = p.seg_off[seg] + tile * TM;
+    t.row_count = min(TM, p.seg_off[seg + 1] - base);
+    t.kv_tok0 = p.fchunk_tok[f];
+    t.nkeys = p.B;
+    t.dest = p.seg_dest[base + min(r, t.row_count - 1)];
+    t.tok = t.dest / (H * p.K1);
+    t.limit = t.nkeys - 1;
+    t.wave_min_limit = t.limit;
+    t.wave_max_limit = t.limit;
+    return true;
+  }
+  const int st = logical - p.hist_bound;
+  if (st >= p.self_total) return false;
+  int lo = 0, hi = p.N;  // chunk c with self_tile_prefix[c]*H <= st
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (p.self_tile_prefix[mid] * H <= st) lo = mid; else hi = mid;
+  }
+  const int c = lo;
+  const int rem = st - p.self_tile_prefix[c] * H;
+  const int nt = p.self_tile_prefix[c + 1] - p.self_tile_prefix[c];
+  t.h = rem / nt;
+  const int tin = nt - 1 - (rem - t.h * nt);  // longest tiles first
+  const int c0 = p.chunk_tok[c];
+  const int len = p.chunk_tok[c + 1] - c0;
+  const int r0 = tin * TM;
+  t.row_count = min(TM, len - r0);
+  t.kv_tok0 = c0;
+  t.nkeys = min(len, r0 + TM);
+  t.tok = c0 + r0 + min(r, t.row_count - 1);
+  t.dest = (t.tok * H + t.h) * p.K1;
+  t.limit = r0 + min(r, t.row_count - 1);
+  t.wave_min_limit = r0 + min(wave * 32, t.row_count - 1);
+  t.wave_max_limit = r0 + min(wave * 32 + 31, t.row_count - 1);
+  return true;
+}
+
+// LDS layout of a [rows x 128] bf16 tile: row-major, 256 bytes per row, with the
+// 16-byte column index XORed by a function of the row so that both access patterns
+// are bank-conflict free: 16-byte row fragments read by 16 lanes holding 16 consecutive
+// rows, and ds_read_b64_tr_b16 quads (4 consecutive rows x 32 bytes).
+__device__ __forceinline__ int sw_col16(int row, int c16) { return c16 ^ ((row & 3) << 2) ^ ((row >> 2) & 3); }
+__device__ __forceinline__ int tile_off16(int row, int c16) { return row * 256 + (sw_col16(row, c16) << 4); }
+
+__device__ __forceinline__ bf16x4 lds_read_tr(const char* p) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) bf16x4*)(p));
+}
+
+// asynchronous 16-byte copy global -> LDS: lane i of the wave fills lds_wave_base + 16*i.
+// Issued as inline assembly so that completion is tracked by the explicit wait_vmem()
+// before the tile barrier only (the copy must stay in flight across the compute phase).
+// The statement overwrites M0, which nothing else in these kernels uses.
+__device__ __forceinline__ void async_copy16(const void* gsrc, uint32_t lds_wave_base) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+               :
+               : "v"(gsrc), "s"(lds_wave_base)
+               : "memory");
+}
+// same for 4 bytes per lane: lane i fills lds_wave_base + 4*i
+__device__ __forceinline__ void async_copy4(const void* gsrc, uint32_t lds_wave_base) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off"
+               :
+               : "v"(gsrc), "s"(lds_wave_base)
+               : "memory");
+}
+__device__ __forceinline__ uint32_t lds_addr(const char* p) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
+}
+// wait until this wave's outstanding global loads (including global -> LDS copies) have landed
+__device__ __forceinline__ void wait_vmem() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
+}  // namespace moba

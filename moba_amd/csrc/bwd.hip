@@ -1,0 +1,523 @@
+// MoBA backward for gfx950: dq, dk, dv of the attention over the fixed sparse pattern.
+//
+// With P = exp(scale * q k^T - LSE) (the global softmax probability, LSE from the
+// forward), delta = rowsum(dO * O) and dS = P * (dO V^T - delta):
+//     dV = P^T dO        dK = scale * dS^T Q        dQ = scale * dS K
+// Nothing is differentiated through the gate.  The result is deterministic: no
+// floating-point atomics, every output element is produced by one workgroup in a
+// fixed order.
+//
+//   bwd_delta_kernel     delta[token, head]
+//   bwd_dq_kernel        row-tile major, same tiling as the forward: each tile (128
+//                        query rows x the keys of one chunk) writes its fp32 partial dQ
+//                        into the row's slot; bwd_dq_reduce_kernel sums the K+1 slots
+//   bwd_dkv_kernel       key-tile major: a workgroup owns 128 keys of (chunk, head) and
+//                        walks first the causal rows of the same chunk, then the gather
+//                        list of rows that selected the chunk; dK/dV accumulate in
+//                        registers and are written once
+//
+// All matrix products use v_mfma_f32_32x32x16_bf16; transposed operands come from
+// ds_read_b64_tr_b16.  Algorithmic work: 10*D flops per attended (query, key) pair
+// (the recomputation of S and dO V^T in both kernels adds 4*D on top).
+#include "attn_common.h"
+
+namespace moba {
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr int TQ = 64;                                  // query rows per step of the dK/dV kernel
+constexpr int kBwdDqLds = 4 * kTileBytes;               // K[2], V[2]
+constexpr int kQStage = 2 * TQ * kHeadDim * 2 + 2 * TQ * 4;  // Q tile, dO tile, lse, delta
+constexpr int kBwdDkvLds = 2 * kQStage;
+
+struct BwdParams {
+  const bf16* q;
+  const bf16* k;
+  const bf16* v;
+  const bf16* dout;
+  const float* lse;    // [S*H] natural log
+  const float* delta;  // [S*H]
+  float* part_dq;      // [S*H*K1, D] fp32
+  bf16* dk;
+  bf16* dv;
+  const int* chunk_fid;  // [N] filtered id of a chunk, -1 for the last chunk of a sequence
+  TileTables t;
+  float scale_log2;
+  float scale;
+};
+
+__global__ __launch_bounds__(256) void bwd_delta_kernel(const bf16* __restrict__ dout, const bf16* __restrict__ out,
+                                                        float* __restrict__ delta, int64_t rows) {
+  const int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+  const int c8 = threadIdx.x & 15;
+  float acc = 0.f;
+  if (row < rows) {
+    const bf16x8 a = *reinterpret_cast<const bf16x8*>(dout + row * kHeadDim + c8 * 8);
+    const bf16x8 b = *reinterpret_cast<const bf16x8*>(out + row * kHeadDim + c8 * 8);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc += (float)a[e] * (float)b[e];
+  }
+#pragma unroll
+  for (int o = 8; o >= 1; o >>= 1) acc += __shfl_xor(acc, o, 64);
+  if (row < rows && c8 == 0) delta[row] = acc;
+}
+
+// ------------------------------------------------------------------------------------ dQ
+__global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int n = lane & 31, hh = lane >> 5;
+  const int H = p.t.H;
+
+  Tile t;
+  const int r = wave * 32 + n;
+  if (!decode_tile(p.t, logical_tile_id(), wave, r, t)) return;
+  const int h = t.h, nkeys = t.nkeys, kv_tok0 = t.kv_tok0, limit = t.limit;
+  const bool row_valid = r < t.row_count;
+
+  bf16x8 bq[8], bdo[8];
+  {
+    const int64_t off = ((int64_t)t.tok * H + h) * kHeadDim + 8 * hh;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      bq[ks] = *reinterpret_cast<const bf16x8*>(p.q + off + 16 * ks);
+      bdo[ks] = *reinterpret_cast<const bf16x8*>(p.dout + off + 16 * ks);
+    }
+  }
+  const float lse2 = p.lse[(int64_t)t.tok * H + h] * kLog2e;
+  const float dl = p.delta[(int64_t)t.tok * H + h];
+
+  const int64_t row_bytes = (int64_t)H * kHeadDim * 2;
+  const uint32_t lds_base = lds_addr(smem);
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  const int ld_kin = lane >> 4, ld_pc = lane & 15;
+  auto issue_tile = [&](int kt, int buf) {
+    const uint32_t kdst = lds_base + buf * kTileBytes;
+    const uint32_t vdst = lds_base + (2 + buf) * kTileBytes;
+    const int key0 = kt * TN;
+    const bool full = (key0 + TN <= nkeys) && (kv_tok0 + key0 + TN <= p.t.S);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int slab = 4 * i + wave_u;
+      const int key = 4 * slab + ld_kin;
+      const int c16 = sw_col16(key, ld_pc);
+      int64_t tk = kv_tok0 + key0 + key;
+      if (!full) tk = min(tk, (int64_t)p.t.S - 1);
+      const int64_t off = tk * row_bytes + h * (kHeadDim * 2) + c16 * 16;
+      async_copy16((const char*)p.k + off, kdst + slab * 1024);
+      async_copy16((const char*)p.v + off, vdst + slab * 1024);
+    }
+  };
+  // rows past the key range are multiplied by dS = 0: clear them so that no NaN can form
+  auto scrub_tile = [&](int kt, int buf) {
+    const int key0 = kt * TN;
+    if (key0 + TN <= nkeys) return;
+    char* kdst = smem + buf * kTileBytes;
+    char* vdst = smem + (2 + buf) * kTileBytes;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int slab = 4 * i + wave;
+      const int key = 4 * slab + ld_kin;
+      if (key0 + key >= nkeys) {
+        *reinterpret_cast<u32x4*>(kdst + slab * 1024 + lane * 16) = u32x4{0, 0, 0, 0};
+        *reinterpret_cast<u32x4*>(vdst + slab * 1024 + lane * 16) = u32x4{0, 0, 0, 0};
+      }
+    }
+  };
+
+  const int nkt = (nkeys + TN - 1) / TN;
+  issue_tile(0, 0);
+  wait_vmem();
+  scrub_tile(0, 0);
+  __syncthreads();
+
+  f32x16 dqacc[4];
+#pragma unroll
+  for (int db = 0; db < 4; ++db)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) dqacc[db][e] = 0.f;
+  const float sl2 = p.scale_log2;
+
+  const int g16 = lane >> 4, i0 = (lane & 15) >> 2, i1 = lane & 3;
+  const int row_off = n * 256;
+  const int row_sw = ((n & 3) << 2) ^ ((n >> 2) & 3);
+  const int tr_c16 = 2 * (g16 & 1) + (i1 >> 1);
+  const int tr_sub = (i1 & 1) * 8;
+
+  for (int kt = 0; kt < nkt; ++kt) {
+    const int buf = kt & 1;
+    const bool has_next = kt + 1 < nkt;
+    if (has_next) issue_tile(kt + 1, buf ^ 1);
+
+    if (kt * TN <= t.wave_max_limit) {
+      const char* ks = smem + buf * kTileBytes;
+      const char* vs = smem + (2 + buf) * kTileBytes;
+      const bool masked = kt * TN + TN - 1 > t.wave_min_limit;
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) {
+        // S^T and (dO V^T)^T for 32 keys x 32 queries: two independent MFMA chains
+        bf16x8 ka[8], va[8];
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s8 = 0; s8 < 8; ++s8) {
+          const int o = kb * 8192 + row_off + (((2 * s8 + hh) ^ row_sw) << 4);
+          ka[s8] = *reinterpret_cast<const bf16x8*>(ks + o);
+          va[s8] = *reinterpret_cast<const bf16x8*>(vs + o);
+        }
+        f32x16 sacc, dpacc;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) { sacc[e] = 0.f; dpacc[e] = 0.f; }
+#pragma unroll
+        for (int s8 = 0; s8 < 8; ++s8) {
+          sacc = mfma32(ka[s8], bq[s8], sacc);
+          dpacc = mfma32(va[s8], bdo[s8], dpacc);
+        }
+        // 8 fragment reads ahead, then reads and MFMAs in step (bounded register use)
+        __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (masked) {
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            const int key = kt * TN + 32 * kb + 8 * (e >> 2) + 4 * hh + (e & 3);
+            if (key > limit) sacc[e] = -INFINITY;
+          }
+        }
+        bf16x8 dsb[2];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const float pe = fast_exp2(sacc[e] * sl2 - lse2);
+          dsb[e >> 3][e & 7] = (bf16)(pe * (dpacc[e] - dl));
+        }
+        // dQ^T += K^T dS^T
+#pragma unroll
+        for (int j2 = 0; j2 < 2; ++j2) {
+          const int j = 2 * kb + j2;
+          const int keyA = 16 * j + 4 * hh + i0;
+          const int keyB = keyA + 8;
+#pragma unroll
+          for (int db = 0; db < 4; ++db) {
+            const int c16 = 4 * db + tr_c16;
+            const bf16x4 xa = lds_read_tr(ks + keyA * 256 + ((c16 ^ (i0 << 2) ^ hh) << 4) + tr_sub);
+            const bf16x4 xb = lds_read_tr(ks + keyB * 256 + ((c16 ^ (i0 << 2) ^ (hh + 2)) << 4) + tr_sub);
+            bf16x8 a;
+            a[0] = xa[0]; a[1] = xa[1]; a[2] = xa[2]; a[3] = xa[3];
+            a[4] = xb[0]; a[5] = xb[1]; a[6] = xb[2]; a[7] = xb[3];
+            dqacc[db] = mfma32(a, dsb[j2], dqacc[db]);
+          }
+        }
+      }
+    }
+    if (has_next) {
+      wait_vmem();
+      scrub_tile(kt + 1, buf ^ 1);
+    }
+    __syncthreads();
+  }
+
+  if (row_valid) {
+    float* dst = p.part_dq + (int64_t)t.dest * kHeadDim;
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        f32x4 w;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) w[e] = dqacc[db][4 * g + e];
+        *reinterpret_cast<f32x4*>(dst + 32 * db + 8 * g + 4 * hh) = w;
+      }
+  }
+}
+
+// dq[row] = scale * sum over the row's valid slots of part_dq; 16 lanes per row
+__global__ __launch_bounds__(256) void bwd_dq_reduce_kernel(const float* __restrict__ part_dq,
+                                                            const int* __restrict__ sel, bf16* __restrict__ dq,
+                                                            int64_t rows, int K1, float scale) {
+  const int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+  if (row >= rows) return;
+  const int c8 = threadIdx.x & 15;
+  const int K = K1 - 1;
+  const int* ps = sel + row * K;
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+  const float* src = part_dq + row * K1 * kHeadDim + c8 * 8;
+  for (int j = 0; j < K1; ++j) {
+    if (j > 0 && ps[j - 1] < 0) continue;
+    const f32x4 a = *reinterpret_cast<const f32x4*>(src + (int64_t)j * kHeadDim);
+    const f32x4 b = *reinterpret_cast<const f32x4*>(src + (int64_t)j * kHeadDim + 4);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) { acc[e] += a[e]; acc[4 + e] += b[e]; }
+  }
+  bf16x8 o;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) o[e] = (bf16)(acc[e] * scale);
+  *reinterpret_cast<bf16x8*>(dq + row * kHeadDim + c8 * 8) = o;
+}
+
+// ------------------------------------------------------------------------------------ dK, dV
+__global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams p) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int n = lane & 31, hh = lane >> 5;
+  const int H = p.t.H, K1 = p.t.K1;
+
+  // ---- which 128-key tile: same enumeration as the forward's self tiles ----
+  const int st = logical_tile_id();
+  if (st >= p.t.self_total) return;
+  int lo = 0, hi = p.t.N;
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (p.t.self_tile_prefix[mid] * H <= st) lo = mid; else hi = mid;
+  }
+  const int c = lo;
+  const int rem = st - p.t.self_tile_prefix[c] * H;
+  const int nt = p.t.self_tile_prefix[c + 1] - p.t.self_tile_prefix[c];
+  const int h = rem / nt;
+  const int tin = rem - h * nt;
+  const int c0 = p.t.chunk_tok[c];
+  const int len = p.t.chunk_tok[c + 1] - c0;
+  const int key0 = tin * TM;
+  const int mykey = key0 + wave * 32 + n;        // position inside the chunk
+  const bool key_valid = mykey < len;
+
+  // ---- the rows that attend these keys: causal rows of the chunk, then the gather list ----
+  const int self_rows = len - key0;              // chunk positions key0 .. len-1
+  const int nself = (self_rows + TQ - 1) / TQ;
+  int list_base = 0, list_rows = 0;
+  {
+    const int f = (p.chunk_fid && K1 > 1) ? p.chunk_fid[c] : -1;
+    if (f >= 0) {
+      list_base = p.t.seg_off[f * H + h];
+      list_rows = p.t.seg_off[f * H + h + 1] - list_base;
+    }
+  }
+  const int nhist = (list_rows + TQ - 1) / TQ;
+  const int ntile = nself + nhist;
+
+  // ---- K^T and V^T operands of this lane's key: [16*ks + 8*hh .. +7] ----
+  bf16x8 bk[8], bv[8];
+  {
+    const int64_t off = ((int64_t)(c0 + min(mykey, len - 1)) * H + h) * kHeadDim + 8 * hh;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      bk[ks] = *reinterpret_cast<const bf16x8*>(p.k + off + 16 * ks);
+      bv[ks] = *reinterpret_cast<const bf16x8*>(p.v + off + 16 * ks);
+    }
+  }
+
+  // ---- stage loader: TQ rows of Q and dO (16 KiB each) + lse + delta ----
+  const uint32_t lds_base = lds_addr(smem);
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  const int ld_rin = lane >> 4, ld_pc = lane & 15;
+  // token of row `row` (0..TQ-1) of query tile qi; rows past the end repeat the last row
+  auto row_token = [&](int qi, int row) -> int {
+    if (qi < nself) return c0 + key0 + min(qi * TQ + row, self_rows - 1);
+    const int idx = min((qi - nself) * TQ + row, list_rows - 1);
+    return p.t.seg_dest[list_base + idx] / (H * K1);
+  };
+  auto issue_stage = [&](int qi, int buf) {
+    const uint32_t qdst = lds_base + buf * kQStage;
+    const uint32_t odst = qdst + TQ * kHeadDim * 2;
+    // all row lookups first, so that the copies are issued back to back
+    int toks[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) toks[i] = row_token(qi, 4 * (4 * i + wave_u) + ld_rin);
+    const int tok_l = row_token(qi, lane);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int slab = 4 * i + wave_u;
+      const int row = 4 * slab + ld_rin;
+      const int c16 = sw_col16(row, ld_pc);
+      const int64_t off = (((int64_t)toks[i] * H + h) * kHeadDim + c16 * 8) * 2;
+      async_copy16((const char*)p.q + off, qdst + slab * 1024);
+      async_copy16((const char*)p.dout + off, odst + slab * 1024);
+    }
+    if (wave_u < 2) {
+      const float* src = (wave_u == 0 ? p.lse : p.delta) + ((int64_t)tok_l * H + h);
+      async_copy4(src, qdst + 2 * TQ * kHeadDim * 2 + wave_u * (TQ * 4));
+    }
+  };
+
+  f32x16 dkacc[4], dvacc[4];
+#pragma unroll
+  for (int db = 0; db < 4; ++db)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) { dkacc[db][e] = 0.f; dvacc[db][e] = 0.f; }
+  const float sl2 = p.scale_log2;
+
+  const int g16 = lane >> 4, i0 = (lane & 15) >> 2, i1 = lane & 3;
+  const int row_off = n * 256;
+  const int row_sw = ((n & 3) << 2) ^ ((n >> 2) & 3);
+  const int tr_c16 = 2 * (g16 & 1) + (i1 >> 1);
+  const int tr_sub = (i1 & 1) * 8;
+
+  if (ntile > 0) {
+    issue_stage(0, 0);
+    wait_vmem();
+  }
+  __syncthreads();
+
+  for (int qi = 0; qi < ntile; ++qi) {
+    const int buf = qi & 1;
+    const bool has_next = qi + 1 < ntile;
+    if (has_next) issue_stage(qi + 1, buf ^ 1);
+
+    const char* qs = smem + buf * kQStage;
+    const char* os = qs + TQ * kHeadDim * 2;
+    const float* lse_s = reinterpret_cast<const float*>(qs + 2 * TQ * kHeadDim * 2);
+    const float* del_s = lse_s + TQ;
+    const bool is_self = qi < nself;
+    // number of real rows in this tile, and for self tiles the chunk position of row 0
+    const int rows_here = is_self ? min(TQ, self_rows - qi * TQ) : min(TQ, list_rows - (qi - nself) * TQ);
+    const int qpos0 = key0 + qi * TQ;  // only meaningful for self tiles
+    // causal masking can only bite while the tile's first row is before the wave's last key
+    const bool masked = (rows_here < TQ) || (is_self && qpos0 < key0 + wave * 32 + 31);
+
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) {
+      // S (queries x keys) and dO V^T: lane = key, elements = queries 32*qb + 8g + 4hh + r
+      bf16x8 qa[8], oa[8];
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int s8 = 0; s8 < 8; ++s8) {
+        const int o = qb * 8192 + row_off + (((2 * s8 + hh) ^ row_sw) << 4);
+        qa[s8] = *reinterpret_cast<const bf16x8*>(qs + o);
+        oa[s8] = *reinterpret_cast<const bf16x8*>(os + o);
+      }
+      f32x16 sacc, dpacc;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) { sacc[e] = 0.f; dpacc[e] = 0.f; }
+#pragma unroll
+      for (int s8 = 0; s8 < 8; ++s8) {
+        sacc = mfma32(qa[s8], bk[s8], sacc);
+        dpacc = mfma32(oa[s8], bv[s8], dpacc);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x100, 16, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 16, 0);
+      __builtin_amdgcn_sched_barrier(0);
+
+      bf16x8 pb[2], dsb[2];
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const f32x4 l4 = *reinterpret_cast<const f32x4*>(lse_s + 32 * qb + 8 * g + 4 * hh);
+        const f32x4 d4 = *reinterpret_cast<const f32x4*>(del_s + 32 * qb + 8 * g + 4 * hh);
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) {
+          const int e = 4 * g + rr;
+          const int row = 32 * qb + 8 * g + 4 * hh + rr;
+          float pe = fast_exp2(sacc[e] * sl2 - l4[rr] * kLog2e);
+          if (masked) {
+            const bool ok = (row < rows_here) && (!is_self || qpos0 + row >= mykey);
+            pe = ok ? pe : 0.f;
+          }
+          pb[e >> 3][e & 7] = (bf16)pe;
+          dsb[e >> 3][e & 7] = (bf16)(pe * (dpacc[e] - d4[rr]));
+        }
+      }
+      // dV^T += dO^T P and dK^T += Q^T dS  (contraction over the 32 queries, two steps of 16)
+#pragma unroll
+      for (int j2 = 0; j2 < 2; ++j2) {
+        const int rowA = 32 * qb + 16 * j2 + 4 * hh + i0;
+        const int rowB = rowA + 8;
+#pragma unroll
+        for (int db = 0; db < 4; ++db) {
+          const int c16 = 4 * db + tr_c16;
+          const int offA = rowA * 256 + ((c16 ^ (i0 << 2) ^ hh) << 4) + tr_sub;
+          const int offB = rowB * 256 + ((c16 ^ (i0 << 2) ^ (hh + 2)) << 4) + tr_sub;
+          const bf16x4 oa4 = lds_read_tr(os + offA);
+          const bf16x4 ob4 = lds_read_tr(os + offB);
+          const bf16x4 qa4 = lds_read_tr(qs + offA);
+          const bf16x4 qb4 = lds_read_tr(qs + offB);
+          bf16x8 ao, aq;
+          ao[0] = oa4[0]; ao[1] = oa4[1]; ao[2] = oa4[2]; ao[3] = oa4[3];
+          ao[4] = ob4[0]; ao[5] = ob4[1]; ao[6] = ob4[2]; ao[7] = ob4[3];
+          aq[0] = qa4[0]; aq[1] = qa4[1]; aq[2] = qa4[2]; aq[3] = qa4[3];
+          aq[4] = qb4[0]; aq[5] = qb4[1]; aq[6] = qb4[2]; aq[7] = qb4[3];
+          dvacc[db] = mfma32(ao, pb[j2], dvacc[db]);
+          dkacc[db] = mfma32(aq, dsb[j2], dkacc[db]);
+        }
+      }
+    }
+    if (has_next) wait_vmem();
+    __syncthreads();
+  }
+
+  if (key_valid) {
+    const int64_t off = ((int64_t)(c0 + mykey) * H + h) * kHeadDim;
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        u32x2 wk, wv;
+        wk[0] = pack_bf16(dkacc[db][4 * g + 0] * p.scale, dkacc[db][4 * g + 1] * p.scale);
+        wk[1] = pack_bf16(dkacc[db][4 * g + 2] * p.scale, dkacc[db][4 * g + 3] * p.scale);
+        wv[0] = pack_bf16(dvacc[db][4 * g + 0], dvacc[db][4 * g + 1]);
+        wv[1] = pack_bf16(dvacc[db][4 * g + 2], dvacc[db][4 * g + 3]);
+        *reinterpret_cast<u32x2*>(p.dk + off + 32 * db + 8 * g + 4 * hh) = wk;
+        *reinterpret_cast<u32x2*>(p.dv + off + 32 * db + 8 * g + 4 * hh) = wv;
+      }
+  }
+}
+
+}  // namespace moba
+
+using namespace moba;
+
+extern "C" int moba_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out,
+                        const float* lse, const int32_t* sel, const int32_t* seg_off, const int32_t* tile_off,
+                        const int32_t* seg_dest, const int32_t* fchunk_tok, const int32_t* chunk_tok,
+                        const int32_t* self_tile_prefix, const int32_t* chunk_fid, float* delta, float* part_dq,
+                        void* dq, void* dk, void* dv, int64_t S, int H, int D, int K, int F, int N, int B,
+                        int64_t hist_bound, int64_t self_tiles, void* stream) {
+  if (!dout || !q || !k || !v || !out || !lse || !chunk_tok || !self_tile_prefix || !delta || !part_dq || !dq ||
+      !dk || !dv)
+    return MOBA_ERR_ARG;
+  if (K > 0 && (!sel || !seg_off || !tile_off || !seg_dest || !fchunk_tok || !chunk_fid)) return MOBA_ERR_ARG;
+  if (D != kHeadDim) return MOBA_ERR_UNSUPPORTED;
+  if (S <= 0 || H <= 0 || K < 0 || F < 0 || N <= 0 || B <= 0 || hist_bound < 0 || self_tiles <= 0) return MOBA_ERR_ARG;
+  const void* ptrs[] = {dout, q, k, v, out, part_dq, dq, dk, dv};
+  for (const void* x : ptrs)
+    if ((uintptr_t)x & 15) return MOBA_ERR_ARG;
+  if ((int64_t)S * H * (K + 1) >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
+  const int64_t per = 8 * kXcdBlock;
+  const int64_t total_q = (K > 0 ? hist_bound : 0) + self_tiles * H;
+  const int64_t grid_q = (total_q + per - 1) / per * per;
+  const int64_t grid_kv = (self_tiles * H + per - 1) / per * per;
+  if (grid_q >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
+
+  BwdParams p;
+  p.q = (const bf16*)q; p.k = (const bf16*)k; p.v = (const bf16*)v; p.dout = (const bf16*)dout;
+  p.lse = lse; p.delta = delta; p.part_dq = part_dq; p.dk = (bf16*)dk; p.dv = (bf16*)dv;
+  p.chunk_fid = chunk_fid;
+  p.t.seg_off = seg_off; p.t.tile_off = tile_off; p.t.seg_dest = seg_dest; p.t.fchunk_tok = fchunk_tok;
+  p.t.chunk_tok = chunk_tok; p.t.self_tile_prefix = self_tile_prefix;
+  p.t.S = (int)S; p.t.H = H; p.t.K1 = K + 1; p.t.F = (K > 0) ? F : 0; p.t.N = N; p.t.B = B;
+  p.t.hist_bound = (K > 0) ? (int)hist_bound : 0;
+  p.t.self_total = (int)(self_tiles * H);
+  p.scale = (float)(1.0 / sqrt((double)D));
+  p.scale_log2 = (float)(1.4426950408889634 / sqrt((double)D));
+
+  hipStream_t st = (hipStream_t)stream;
+  static bool attr_set = false;
+  if (!attr_set) {
+    if (hipFuncSetAttribute((const void*)bwd_dq_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdDqLds) !=
+            hipSuccess ||
+        hipFuncSetAttribute((const void*)bwd_dkv_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdDkvLds) !=
+            hipSuccess)
+      return MOBA_ERR_LAUNCH;
+    attr_set = true;
+  }
+  const int64_t rows = S * H;
+  hipLaunchKernelGGL(bwd_delta_kernel, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st, (const bf16*)dout,
+                     (const bf16*)out, delta, rows);
+  hipLaunchKernelGGL(bwd_dq_kernel, dim3((unsigned)grid_q), dim3(256), kBwdDqLds, st, p);
+  hipLaunchKernelGGL(bwd_dq_reduce_kernel, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st,
+                     (const float*)part_dq, sel, (bf16*)dq, rows, K + 1, p.scale);
+  hipLaunchKernelGGL(bwd_dkv_kernel, dim3((unsigned)grid_kv), dim3(256), kBwdDkvLds, st, p);
+  return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
+}

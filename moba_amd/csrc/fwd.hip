@@ -15,58 +15,21 @@
 //
 // Algorithmic work: 4*D flops per attended (query, key) pair; the bound is the bf16
 // MFMA rate.  Compulsory HBM traffic is q, k, v once, the partials once each way.
-#include "common.h"
+#include "attn_common.h"
 
 namespace moba {
 
-constexpr int TM = 128;  // query rows per workgroup (32 per wave)
-constexpr int TN = 64;   // keys per inner iteration
-constexpr int kTileBytes = TN * kHeadDim * 2;
 constexpr int kFwdLds = 4 * kTileBytes;  // K[2], V[2]
-constexpr int kXcdBlock = 64;            // consecutive logical tiles that share an XCD
 
 struct FwdParams {
   const bf16* q;
   const bf16* k;
   const bf16* v;
-  bf16* part_o;            // [S*H*K1, D]
-  float* part_lse;         // [S*H*K1], log2 domain
-  const int* seg_off;      // [F*H+1]
-  const int* tile_off;     // [F*H+1]
-  const int* seg_dest;     // [M]
-  const int* fchunk_tok;   // [F]
-  const int* chunk_tok;    // [N+1]
-  const int* self_tile_prefix;  // [N+1]
-  int S, H, K1, F, N, B;
-  int hist_bound;          // upper bound on history tiles (logical ids below it)
-  int self_total;          // self_tile_prefix[N] * H
-  float scale_log2;        // D^-0.5 * log2(e)
+  bf16* part_o;     // [S*H*K1, D]
+  float* part_lse;  // [S*H*K1], log2 domain
+  TileTables t;
+  float scale_log2;  // D^-0.5 * log2(e)
 };
-
-__device__ __forceinline__ int k_lds_off(int key, int c16) { return key * 256 + ((c16 ^ (key & 15)) << 4); }
-__device__ __forceinline__ int v_lds_off(int key, int c16) {
-  return key * 256 + ((((c16 >> 2) ^ (key & 3))) << 6) + ((c16 & 3) << 4);
-}
-
-__device__ __forceinline__ bf16x4 lds_read_tr(const char* p) {
-  return __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
-      (__attribute__((address_space(3))) bf16x4*)(p));
-}
-
-// asynchronous 16-byte copy global -> LDS: lane i of the wave fills lds_wave_base + 16*i.
-// Issued as inline assembly so that completion is tracked by the explicit wait_vmem()
-// before the tile barrier only (the copy must stay in flight across the compute phase).
-__device__ __forceinline__ void async_copy16(const void* gsrc, uint32_t lds_wave_base) {
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
-               :
-               : "v"(gsrc), "s"(lds_wave_base)
-               : "memory", "m0");
-}
-__device__ __forceinline__ uint32_t lds_addr(const char* p) {
-  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
-}
-// wait until this wave's outstanding global loads (including global -> LDS copies) have landed
-__device__ __forceinline__ void wait_vmem() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 
 constexpr float kRescaleThreshold = 8.f;  // log2 units: the running max may lag the true max by this much
 
@@ -74,64 +37,18 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int n = lane & 31, hh = lane >> 5;
-  const int H = p.H;
+  const int H = p.t.H;
 
-  // ---- which tile ----
-  int logical;
-  {
-    const int x = blockIdx.x & 7, y = blockIdx.x >> 3;
-    logical = ((y / kXcdBlock) * 8 + x) * kXcdBlock + (y % kXcdBlock);
-  }
-  int h, kv_tok0, nkeys, row_count, dest, tok, limit, wave_min_limit, wave_max_limit;
+  Tile t;
   const int r = wave * 32 + n;
-  if (logical < p.hist_bound) {
-    const int FH = p.F * H;
-    if (FH == 0 || logical >= p.tile_off[FH]) return;
-    const int seg = upper_row(p.tile_off, FH, logical);
-    const int tile = logical - p.tile_off[seg];
-    const int f = seg / H;
-    h = seg - f * H;
-    const int base = p.seg_off[seg] + tile * TM;
-    row_count = min(TM, p.seg_off[seg + 1] - base);
-    kv_tok0 = p.fchunk_tok[f];
-    nkeys = p.B;
-    dest = p.seg_dest[base + min(r, row_count - 1)];
-    tok = dest / (H * p.K1);
-    limit = nkeys - 1;
-    wave_min_limit = limit;
-    wave_max_limit = limit;
-  } else {
-    const int st = logical - p.hist_bound;
-    if (st >= p.self_total) return;
-    // chunk c with self_tile_prefix[c]*H <= st
-    int lo = 0, hi = p.N;
-    while (hi - lo > 1) {
-      const int mid = (lo + hi) >> 1;
-      if (p.self_tile_prefix[mid] * H <= st) lo = mid; else hi = mid;
-    }
-    const int c = lo;
-    const int rem = st - p.self_tile_prefix[c] * H;
-    const int nt = p.self_tile_prefix[c + 1] - p.self_tile_prefix[c];
-    h = rem / nt;
-    const int tin = nt - 1 - (rem - h * nt);  // longest tiles first
-    const int c0 = p.chunk_tok[c];
-    const int len = p.chunk_tok[c + 1] - c0;
-    const int r0 = tin * TM;
-    row_count = min(TM, len - r0);
-    kv_tok0 = c0;
-    nkeys = min(len, r0 + TM);
-    tok = c0 + r0 + min(r, row_count - 1);
-    dest = (tok * H + h) * p.K1;
-    limit = r0 + min(r, row_count - 1);
-    wave_min_limit = r0 + min(wave * 32, row_count - 1);
-    wave_max_limit = r0 + min(wave * 32 + 31, row_count - 1);
-  }
-  const bool row_valid = r < row_count;
+  if (!decode_tile(p.t, logical_tile_id(), wave, r, t)) return;
+  const int h = t.h, nkeys = t.nkeys, kv_tok0 = t.kv_tok0, limit = t.limit;
+  const bool row_valid = r < t.row_count;
 
   // ---- Q^T operand: lane (n, hh) holds q[tok][16*ks + 8*hh .. +7] ----
   bf16x8 bq[8];
   {
-    const bf16* src = p.q + ((int64_t)tok * H + h) * kHeadDim + 8 * hh;
+    const bf16* src = p.q + ((int64_t)t.tok * H + h) * kHeadDim + 8 * hh;
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) bq[ks] = *reinterpret_cast<const bf16x8*>(src + 16 * ks);
   }
@@ -143,25 +60,23 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams p) {
   const int64_t row_bytes = (int64_t)H * kHeadDim * 2;
   const uint32_t lds_base = lds_addr(smem);
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-  const int ld_kin = lane >> 4;                     // key within the slab
-  const int ld_pc = lane & 15;                      // physical 16-byte column
+  const int ld_kin = lane >> 4;  // key within the slab
+  const int ld_pc = lane & 15;   // physical 16-byte column
   auto issue_tile = [&](int kt, int buf) {
     const uint32_t kdst = lds_base + buf * kTileBytes;
     const uint32_t vdst = lds_base + (2 + buf) * kTileBytes;
     const int key0 = kt * TN;
-    const bool full = (key0 + TN <= nkeys) && (kv_tok0 + key0 + TN <= p.S);
+    const bool full = (key0 + TN <= nkeys) && (kv_tok0 + key0 + TN <= p.t.S);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int slab = 4 * i + wave_u;
-      const int key = 4 * slab + ld_kin;            // key within the tile
-      const int kc16 = ld_pc ^ (key & 15);
-      const int vc16 = ((((ld_pc >> 2) ^ (key & 3))) << 2) | (ld_pc & 3);
-      int64_t t = kv_tok0 + key0 + key;
-      if (!full) t = min(t, (int64_t)p.S - 1);
-      const char* krow = (const char*)p.k + t * row_bytes + h * (kHeadDim * 2);
-      const char* vrow = (const char*)p.v + t * row_bytes + h * (kHeadDim * 2);
-      async_copy16(krow + kc16 * 16, kdst + slab * 1024);
-      async_copy16(vrow + vc16 * 16, vdst + slab * 1024);
+      const int key = 4 * slab + ld_kin;  // key within the tile
+      const int c16 = sw_col16(key, ld_pc);  // the swizzle is an involution
+      int64_t tk = kv_tok0 + key0 + key;
+      if (!full) tk = min(tk, (int64_t)p.t.S - 1);
+      const int64_t off = tk * row_bytes + h * (kHeadDim * 2) + c16 * 16;
+      async_copy16((const char*)p.k + off, kdst + slab * 1024);
+      async_copy16((const char*)p.v + off, vdst + slab * 1024);
     }
   };
   // rows of V past the end of the key range must not reach the MFMA (0 * NaN): clear them
@@ -193,18 +108,19 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams p) {
 
   // per-lane pieces of the fragment addresses
   const int g16 = lane >> 4, i0 = (lane & 15) >> 2, i1 = lane & 3;
-  const int v_lane_off = 32 * (g16 & 1) + 8 * i1;
-  int k_frag_off[2];
-#pragma unroll
-  for (int kb = 0; kb < 2; ++kb) k_frag_off[kb] = (32 * kb + n) * 256;
-  const int k_sw = n & 15;  // (32*kb + n) & 15
+  // K row fragment: row 32*kb + n, column 2*s8 + hh
+  const int k_row_off = n * 256;
+  const int k_sw = ((n & 3) << 2) ^ ((n >> 2) & 3);
+  // V^T quad read: rows 16*j + 4*hh + i0 (+8), 8 bytes at d = 32*db + 16*(g16&1) + 4*i1
+  const int v_c16 = 2 * (g16 & 1) + (i1 >> 1);
+  const int v_sub = (i1 & 1) * 8;
 
   for (int kt = 0; kt < nkt; ++kt) {
     const int buf = kt & 1;
     const bool has_next = kt + 1 < nkt;
     if (has_next) issue_tile(kt + 1, buf ^ 1);
 
-    if (kt * TN <= wave_max_limit) {  // wave-uniform: skip tiles entirely above the diagonal
+    if (kt * TN <= t.wave_max_limit) {  // wave-uniform: skip tiles entirely above the diagonal
       const char* ks = smem + buf * kTileBytes;
       const char* vs = smem + (2 + buf) * kTileBytes;
       // S^T (keys x queries), two 32-key blocks: fetch all K fragments, then two
@@ -215,7 +131,7 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams p) {
       for (int s8 = 0; s8 < 8; ++s8)
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
-          ka[kb][s8] = *reinterpret_cast<const bf16x8*>(ks + k_frag_off[kb] + (((2 * s8 + hh) ^ k_sw) << 4));
+          ka[kb][s8] = *reinterpret_cast<const bf16x8*>(ks + kb * 8192 + k_row_off + (((2 * s8 + hh) ^ k_sw) << 4));
       f32x16 sacc[2];
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb)
@@ -230,7 +146,7 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams p) {
       __builtin_amdgcn_sched_group_barrier(0x008, 16, 0);
       __builtin_amdgcn_sched_barrier(0);
 
-      if (kt * TN + TN - 1 > wave_min_limit) {
+      if (kt * TN + TN - 1 > t.wave_min_limit) {
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
@@ -277,12 +193,13 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams p) {
       // O^T += V^T P^T
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const int keyA = 16 * j + 4 * hh + i0;
-        const int keyB = keyA + 8;
+        const int keyA = 16 * j + 4 * hh + i0;  // keyA & 3 == i0, (keyA >> 2) & 3 == hh
+        const int keyB = keyA + 8;              // (keyB >> 2) & 3 == hh + 2
 #pragma unroll
         for (int db = 0; db < 4; ++db) {
-          const bf16x4 va = lds_read_tr(vs + keyA * 256 + ((db ^ (keyA & 3)) << 6) + v_lane_off);
-          const bf16x4 vb = lds_read_tr(vs + keyB * 256 + ((db ^ (keyB & 3)) << 6) + v_lane_off);
+          const int c16 = 4 * db + v_c16;
+          const bf16x4 va = lds_read_tr(vs + keyA * 256 + ((c16 ^ (i0 << 2) ^ hh) << 4) + v_sub);
+          const bf16x4 vb = lds_read_tr(vs + keyB * 256 + ((c16 ^ (i0 << 2) ^ (hh + 2)) << 4) + v_sub);
           bf16x8 a;
           a[0] = va[0]; a[1] = va[1]; a[2] = va[2]; a[3] = va[3];
           a[4] = vb[0]; a[5] = vb[1]; a[6] = vb[2]; a[7] = vb[3];
@@ -301,7 +218,7 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams p) {
   const float l_tot = l_run + xhalf(l_run);
   const float inv = 1.f / l_tot;
   if (row_valid) {
-    bf16* dst = p.part_o + (int64_t)dest * kHeadDim;
+    bf16* dst = p.part_o + (int64_t)t.dest * kHeadDim;
 #pragma unroll
     for (int db = 0; db < 4; ++db)
 #pragma unroll
@@ -311,7 +228,7 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams p) {
         w[1] = pack_bf16(oacc[db][4 * g + 2] * inv, oacc[db][4 * g + 3] * inv);
         *reinterpret_cast<u32x2*>(dst + 32 * db + 8 * g + 4 * hh) = w;
       }
-    if (hh == 0) p.part_lse[dest] = m_run + fast_log2(l_tot);
+    if (hh == 0) p.part_lse[t.dest] = m_run + fast_log2(l_tot);
   }
 }
 
@@ -375,11 +292,11 @@ extern "C" int moba_fwd_partials(const void* q, const void* k, const void* v, vo
   FwdParams p;
   p.q = (const bf16*)q; p.k = (const bf16*)k; p.v = (const bf16*)v;
   p.part_o = (bf16*)part_o; p.part_lse = part_lse;
-  p.seg_off = seg_off; p.tile_off = tile_off; p.seg_dest = seg_dest; p.fchunk_tok = fchunk_tok;
-  p.chunk_tok = chunk_tok; p.self_tile_prefix = self_tile_prefix;
-  p.S = (int)S; p.H = H; p.K1 = K + 1; p.F = (K > 0) ? F : 0; p.N = N; p.B = B;
-  p.hist_bound = (K > 0) ? (int)hist_bound : 0;
-  p.self_total = (int)(self_tiles * H);
+  p.t.seg_off = seg_off; p.t.tile_off = tile_off; p.t.seg_dest = seg_dest; p.t.fchunk_tok = fchunk_tok;
+  p.t.chunk_tok = chunk_tok; p.t.self_tile_prefix = self_tile_prefix;
+  p.t.S = (int)S; p.t.H = H; p.t.K1 = K + 1; p.t.F = (K > 0) ? F : 0; p.t.N = N; p.t.B = B;
+  p.t.hist_bound = (K > 0) ? (int)hist_bound : 0;
+  p.t.self_total = (int)(self_tiles * H);
   p.scale_log2 = (float)(1.4426950408889634 / sqrt((double)D));
   hipStream_t st = (hipStream_t)stream;
   static bool attr_set = false;

@@ -170,8 +170,6 @@ def _forward(q, k, v, plan: MobaPlan, timer: Optional[StageTimer] = None):
 
 def _backward(dout, q, k, v, out, lse, sel, seg_off, tile_off, seg_dest, plan: MobaPlan):
     lib = _lib.load()
-    if not hasattr(lib, "moba_bwd"):
-        raise RuntimeError("libmoba_hip.so was built without the backward kernels")
     S, H, D = q.shape
     dev = q.device
     K = plan.K
@@ -183,7 +181,7 @@ def _backward(dout, q, k, v, out, lse, sel, seg_off, tile_off, seg_dest, plan: M
     part_dq = torch.empty((S * H * (K + 1), D), dtype=torch.float32, device=dev)
     _lib.check(lib.moba_bwd(_ptr(dout), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(sel), _ptr(seg_off),
                             _ptr(tile_off), _ptr(seg_dest), _ptr(t.get("fchunk_tok")), _ptr(t["chunk_tok"]),
-                            _ptr(t["self_tile_prefix"]), _ptr(t.get("chunk_fb")), _ptr(t.get("chunk_local")),
+                            _ptr(t["self_tile_prefix"]), _ptr(t.get("chunk_fid")),
                             _ptr(delta), _ptr(part_dq), _ptr(dq), _ptr(dk), _ptr(dv),
                             S, H, D, K, plan.F, plan.N, plan.chunk_size, plan.hist_tile_bound(H), plan.self_tiles,
                             _stream(dev)), "moba_bwd")

@@ -79,8 +79,10 @@ def _host_tables(cu: np.ndarray, B: int, topk: int):
         cmax = int(n_chunks.max() - 1)
         K = min(k_eff, cmax)
         pairs = int((chunk_len.astype(np.int64) * np.minimum(K, local)).sum())
+        chunk_fid = np.full(N, -1, dtype=np.int64)
+        chunk_fid[fidx] = np.arange(F)
         out.update(seq_fbase=seq_fbase, fchunk_tok=fchunk_tok, chunk_fb=seq_fbase[seq_of_chunk], chunk_local=local,
-                   pair_off=pair_off)
+                   pair_off=pair_off, chunk_fid=chunk_fid)
         info.update(K=K, P=int(nq.sum()), cmax=cmax, pairs_per_head=pairs)
         flops = 4.0 * (pairs_self + pairs * B)
     else:

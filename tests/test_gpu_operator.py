@@ -1,0 +1,143 @@
+"""End-to-end parity of moba_attn_varlen (forward + backward) against the CPU oracle,
+reproducing the reference's own test matrix and data recipe
+(tests/test_moba_attn.py:8-42) and its tolerances (:85-100).  GPU only; every call
+goes through the C ABI."""
+
+import itertools
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import make_case
+from oracle import moba_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+# bf16 tolerances: the north-star bound and the reference test's own bounds
+MAX_ABS, MEAN_ABS = 2e-2, 2e-3
+REF_MAX_ABS, REF_MEAN_ABS = 4e-2, 4e-4
+
+
+def run_case(batch, seqlen, heads, B, topk, seed=0, check_grad=True):
+    from moba_amd import moba_efficient as E
+    from moba_amd.plan import make_plan
+
+    q, k, v, do, cu, mx = make_case(batch, seqlen, heads, seed=seed)
+    dev = torch.device("cuda")
+    cu_t = torch.tensor(cu, dtype=torch.int32, device=dev)
+    qg, kg, vg = (x.to(dev).requires_grad_(True) for x in (q, k, v))
+    out = E.moba_attn_varlen(qg, kg, vg, cu_t, mx, moba_chunk_size=B, moba_topk=topk)
+    if check_grad:
+        torch.autograd.backward(out, do.to(dev))
+    plan = make_plan(cu_t, B, topk)
+    sel = None
+    if not plan.fallback:
+        sel = E.gate_topk(qg.detach(), E.chunk_mean(kg.detach(), plan), plan).cpu()
+        # the kernel's selection must agree with the oracle's except at numerical near-ties
+        kbar = O.chunk_mean(k, cu, B)
+        gate = O.gate_scores(q, kbar, cu, B)
+        want = O.select_topk(gate, plan.K)
+        got = torch.sort(torch.where(sel < 0, torch.full_like(sel, 1 << 30), sel), dim=-1).values
+        got = torch.where(got == 1 << 30, torch.full_like(got, -1), got)
+        diff_rows = (got != want).any(dim=-1)
+        if diff_rows.any():
+            # every disagreement must be a near-tie of the fp32 scores
+            for s_, h_ in diff_rows.nonzero().tolist():
+                a = set(got[s_, h_].tolist()) - {-1}
+                b = set(want[s_, h_].tolist()) - {-1}
+                gap = max(abs(float(gate[s_, h_, x]) - float(gate[s_, h_, y])) for x in a ^ b for y in a ^ b)
+                assert gap < 1e-4, (s_, h_, a, b, gap)
+        assert diff_rows.float().mean() < 1e-3
+    qc, kc, vc = (x.clone().requires_grad_(True) for x in (q, k, v))
+    ref = O.moba_attn_varlen_oracle(qc, kc, vc, cu, mx, B, topk, sel=sel)
+    err = (out.detach().cpu().float() - ref.detach()).abs()
+    assert err.max() < MAX_ABS and err.mean() < MEAN_ABS, ("out", err.max().item(), err.mean().item())
+    assert err.max() < REF_MAX_ABS and err.mean() < REF_MEAN_ABS
+    if check_grad:
+        ref.backward(do.float())
+        got_g = torch.stack([qg.grad.cpu().float(), kg.grad.cpu().float(), vg.grad.cpu().float()], dim=1)
+        ref_g = torch.stack([qc.grad, kc.grad, vc.grad], dim=1)
+        gerr = (got_g - ref_g).abs()
+        assert gerr.max() < REF_MAX_ABS and gerr.mean() < REF_MEAN_ABS, ("grad", gerr.max().item(), gerr.mean().item())
+        # per-tensor, relative to the tensor's scale
+        for i, name in enumerate(("dq", "dk", "dv")):
+            e = gerr[:, i]
+            scale = ref_g[:, i].abs().max().clamp_min(1.0)
+            assert e.max() < MAX_ABS * scale, (name, e.max().item(), scale.item())
+    return err
+
+
+GRID = list(itertools.product([1, 4, 7], [1, 2, 4, 8], [512, 1024, 2048], [128, 256, 1024], [2, 3, 4]))
+
+
+@pytest.mark.parametrize("chunk", range(12))
+def test_reference_grid(chunk):
+    """The reference's 324 cases (batch x heads x seqlen x chunk x topk), 27 per test."""
+    cases = GRID[chunk * 27:(chunk + 1) * 27]
+    for batch, heads, seqlen, B, topk in cases:
+        print("case", batch, heads, seqlen, B, topk, flush=True)
+        run_case(batch, seqlen, heads, B, topk)
+
+
+@pytest.mark.parametrize("batch,seqlen,heads,B,topk", [
+    (3, 1500, 3, 100, 3),      # chunk size that is not a multiple of any tile size
+    (1, 2048, 2, 128, 1),      # topk = 1: full causal attention, as the efficient reference path
+    (2, 4096, 2, 64, 12),      # many chunks, k = 11
+    (5, 2000, 2, 128, 64),     # topk beyond the chunk count: everything selected
+    (6, 777, 5, 96, 2),        # odd sizes, 1-token tails
+    (1, 8192, 1, 512, 3),
+])
+def test_edge_shapes(batch, seqlen, heads, B, topk):
+    run_case(batch, seqlen, heads, B, topk, seed=7)
+
+
+def test_one_token_sequences():
+    from moba_amd import moba_efficient as E
+    g = torch.Generator().manual_seed(3)
+    S, H = 300, 2
+    q, k, v = (torch.randn((S, H, 128), generator=g).to(torch.bfloat16) for _ in range(3))
+    cu = [0, 1, 2, 130, 131, 300]
+    cu_t = torch.tensor(cu, dtype=torch.int32, device="cuda")
+    out = E.moba_attn_varlen(q.cuda(), k.cuda(), v.cuda(), cu_t, 169, 32, 3).cpu().float()
+    # a 1-token sequence attends only itself
+    assert torch.equal(out[0], v[0].float()) and torch.equal(out[130], v[130].float())
+    ref = O.moba_attn_varlen_oracle(q, k, v, cu, 169, 32, 3)
+    assert (out - ref).abs().max() < MAX_ABS
+
+
+def test_uniform_v_gives_v():
+    from moba_amd import moba_efficient as E
+    q, k, v, do, cu, mx = make_case(3, 2048, 2, seed=11)
+    v = torch.full_like(v, 0.75)
+    cu_t = torch.tensor(cu, dtype=torch.int32, device="cuda")
+    out = E.moba_attn_varlen(q.cuda(), k.cuda(), v.cuda(), cu_t, mx, 128, 3).cpu().float()
+    assert (out - 0.75).abs().max() < 4e-3
+
+
+def test_backward_is_deterministic():
+    from moba_amd import moba_efficient as E
+    q, k, v, do, cu, mx = make_case(4, 4096, 4, seed=13)
+    cu_t = torch.tensor(cu, dtype=torch.int32, device="cuda")
+    grads = []
+    for _ in range(2):
+        qg, kg, vg = (x.cuda().requires_grad_(True) for x in (q, k, v))
+        out = E.moba_attn_varlen(qg, kg, vg, cu_t, mx, 256, 4)
+        out.backward(do.cuda())
+        grads.append([out.detach().clone(), qg.grad.clone(), kg.grad.clone(), vg.grad.clone()])
+    for a, b in zip(*grads):
+        assert torch.equal(a, b)
+
+
+def test_argument_validation():
+    from moba_amd import moba_attn_varlen
+    q = torch.zeros((64, 2, 128), dtype=torch.bfloat16, device="cuda")
+    cu = torch.tensor([0, 64], dtype=torch.int32, device="cuda")
+    with pytest.raises(TypeError):
+        moba_attn_varlen(q.float(), q.float(), q.float(), cu, 64, 16, 2)
+    with pytest.raises(ValueError):
+        moba_attn_varlen(q, q[:, :1], q, cu, 64, 16, 2)
+    with pytest.raises(ValueError):
+        moba_attn_varlen(q, q, q, torch.tensor([0, 32], dtype=torch.int32, device="cuda"), 64, 16, 2)
+    with pytest.raises(RuntimeError):
+        moba_attn_varlen(q.cpu(), q.cpu(), q.cpu(), cu, 64, 16, 2)
