@@ -11,7 +11,8 @@ import os
 from ctypes import c_char_p, c_int, c_int64, c_size_t, c_void_p
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libmoba_hip.so")
+# MOBA_HIP_LIBRARY overrides the location (e.g. to try a differently built library)
+LIB_PATH = os.environ.get("MOBA_HIP_LIBRARY") or os.path.join(_HERE, "libmoba_hip.so")
 
 _lib = None
 

@@ -34,6 +34,7 @@ struct Tile {
   int tok;        // this lane's row: token
   int limit;      // this lane's row attends keys <= limit
   int wave_min_limit, wave_max_limit;  // over the wave's 32 rows
+  int rot;        // history tiles may visit their key tiles in any order: start offset
 };
 
 // Workgroup ids are dealt round-robin to the 8 XCDs; give each XCD runs of kXcdBlock
@@ -62,6 +63,7 @@ __device__ __forceinline__ bool decode_tile(const TileTables& p, int logical, in
     t.limit = t.nkeys - 1;
     t.wave_min_limit = t.limit;
     t.wave_max_limit = t.limit;
+    t.rot = tile;
     return true;
   }
   const int st = logical - p.hist_bound;
@@ -87,7 +89,20 @@ __device__ __forceinline__ bool decode_tile(const TileTables& p, int logical, in
   t.limit = r0 + min(r, t.row_count - 1);
   t.wave_min_limit = r0 + min(wave * 32, t.row_count - 1);
   t.wave_max_limit = r0 + min(wave * 32 + 31, t.row_count - 1);
+  t.rot = 0;
   return true;
+}
+
+// max over the two halves of the wave (lane l and lane l^32), without LDS traffic
+__device__ __forceinline__ float max_xhalf(float x) {
+  const uint32_t u = __builtin_bit_cast(uint32_t, x);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return fmaxf(__builtin_bit_cast(float, (uint32_t)r[0]), __builtin_bit_cast(float, (uint32_t)r[1]));
+}
+__device__ __forceinline__ float sum_xhalf(float x) {
+  const uint32_t u = __builtin_bit_cast(uint32_t, x);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __builtin_bit_cast(float, (uint32_t)r[0]) + __builtin_bit_cast(float, (uint32_t)r[1]);
 }
 
 // LDS layout of a [rows x 128] bf16 tile: row-major, 256 bytes per row, with the
@@ -109,6 +124,17 @@ __device__ __forceinline__ void async_copy16(const void* gsrc, uint32_t lds_wave
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
                :
                : "v"(gsrc), "s"(lds_wave_base)
+               : "memory");
+}
+// same with the global address split into a wave-uniform base and a per-lane byte offset
+__device__ __forceinline__ void async_copy16_sv(const void* uniform_base, uint32_t lane_off, uint32_t lds_wave_base) {
+  const uint64_t b = (uint64_t)uniform_base;
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)b);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(b >> 32));
+  const uint64_t sb = ((uint64_t)hi << 32) | lo;
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :
+               : "v"(lane_off), "s"(sb), "s"(lds_wave_base)
                : "memory");
 }
 // same for 4 bytes per lane: lane i fills lds_wave_base + 4*i

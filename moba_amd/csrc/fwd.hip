@@ -62,21 +62,40 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams p) {
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   const int ld_kin = lane >> 4;  // key within the slab
   const int ld_pc = lane & 15;   // physical 16-byte column
+  // per-lane byte offset of the lane's 16 bytes inside a 64-key tile, for each of the 4 slabs
+  uint32_t ld_off[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int key = 4 * (4 * i + wave_u) + ld_kin;
+    ld_off[i] = (uint32_t)(key * row_bytes + sw_col16(key, ld_pc) * 16);  // the swizzle is an involution
+  }
+  const char* k_head = (const char*)p.k + (int64_t)kv_tok0 * row_bytes + h * (kHeadDim * 2);
+  const char* v_head = (const char*)p.v + (int64_t)kv_tok0 * row_bytes + h * (kHeadDim * 2);
   auto issue_tile = [&](int kt, int buf) {
     const uint32_t kdst = lds_base + buf * kTileBytes;
     const uint32_t vdst = lds_base + (2 + buf) * kTileBytes;
     const int key0 = kt * TN;
     const bool full = (key0 + TN <= nkeys) && (kv_tok0 + key0 + TN <= p.t.S);
+    if (full) {  // uniform tile base in SGPRs + constant per-lane offsets: no address arithmetic
+      const char* kb = k_head + (int64_t)key0 * row_bytes;
+      const char* vb = v_head + (int64_t)key0 * row_bytes;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int slab = 4 * i + wave_u;
-      const int key = 4 * slab + ld_kin;  // key within the tile
-      const int c16 = sw_col16(key, ld_pc);  // the swizzle is an involution
-      int64_t tk = kv_tok0 + key0 + key;
-      if (!full) tk = min(tk, (int64_t)p.t.S - 1);
-      const int64_t off = tk * row_bytes + h * (kHeadDim * 2) + c16 * 16;
-      async_copy16((const char*)p.k + off, kdst + slab * 1024);
-      async_copy16((const char*)p.v + off, vdst + slab * 1024);
+      for (int i = 0; i < 4; ++i) {
+        const int slab = 4 * i + wave_u;
+        async_copy16_sv(kb, ld_off[i], kdst + slab * 1024);
+        async_copy16_sv(vb, ld_off[i], vdst + slab * 1024);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int slab = 4 * i + wave_u;
+        const int key = 4 * slab + ld_kin;  // key within the tile
+        const int c16 = sw_col16(key, ld_pc);
+        const int64_t tk = min((int64_t)kv_tok0 + key0 + key, (int64_t)p.t.S - 1);
+        const int64_t off = tk * row_bytes + h * (kHeadDim * 2) + c16 * 16;
+        async_copy16((const char*)p.k + off, kdst + slab * 1024);
+        async_copy16((const char*)p.v + off, vdst + slab * 1024);
+      }
     }
   };
   // rows of V past the end of the key range must not reach the MFMA (0 * NaN): clear them
@@ -92,10 +111,15 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams p) {
     }
   };
 
+  // Tiles that run side by side on an XCD work on the same chunk; starting each at a
+  // different key tile spreads their first touches of the chunk over all of it, instead of
+  // every workgroup waiting on the same cache miss at every step.
   const int nkt = (nkeys + TN - 1) / TN;
-  issue_tile(0, 0);
+  const int rot = t.rot % nkt;
+  auto key_tile = [&](int it) { const int x = it + rot; return x >= nkt ? x - nkt : x; };
+  issue_tile(key_tile(0), 0);
   wait_vmem();
-  scrub_tile(0, 0);
+  scrub_tile(key_tile(0), 0);
   __syncthreads();
 
   f32x16 oacc[4];
@@ -115,10 +139,11 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams p) {
   const int v_c16 = 2 * (g16 & 1) + (i1 >> 1);
   const int v_sub = (i1 & 1) * 8;
 
-  for (int kt = 0; kt < nkt; ++kt) {
-    const int buf = kt & 1;
-    const bool has_next = kt + 1 < nkt;
-    if (has_next) issue_tile(kt + 1, buf ^ 1);
+  for (int it = 0; it < nkt; ++it) {
+    const int buf = it & 1;
+    const bool has_next = it + 1 < nkt;
+    const int kt = key_tile(it);
+    if (has_next) issue_tile(key_tile(it + 1), buf ^ 1);
 
     if (kt * TN <= t.wave_max_limit) {  // wave-uniform: skip tiles entirely above the diagonal
       const char* ks = smem + buf * kTileBytes;
@@ -141,9 +166,14 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams p) {
       for (int s8 = 0; s8 < 8; ++s8)
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) sacc[kb] = mfma32(ka[kb][s8], bq[s8], sacc[kb]);
-      // keep all 16 LDS reads in flight ahead of the MFMA chain
-      __builtin_amdgcn_sched_group_barrier(0x100, 16, 0);
-      __builtin_amdgcn_sched_group_barrier(0x008, 16, 0);
+      // 8 fragment reads ahead, then reads and MFMAs in step
+      __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
       __builtin_amdgcn_sched_barrier(0);
 
       if (kt * TN + TN - 1 > t.wave_min_limit) {
@@ -160,7 +190,7 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams p) {
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
         for (int e = 1; e < 16; ++e) mx = fmaxf(mx, sacc[kb][e]);
-      mx = fmaxf(mx, xhalf(mx)) * sl2;
+      mx = max_xhalf(mx) * sl2;
       // lazy running max: move it only when the tile max exceeds it by the threshold
       if (__any(mx > m_run + kRescaleThreshold)) {
         const float m_new = fmaxf(m_run, mx);
@@ -209,13 +239,13 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams p) {
     }
     if (has_next) {
       wait_vmem();
-      scrub_tile(kt + 1, buf ^ 1);
+      scrub_tile(key_tile(it + 1), buf ^ 1);
     }
     __syncthreads();
   }
 
   // ---- epilogue: normalise, write the partial ----
-  const float l_tot = l_run + xhalf(l_run);
+  const float l_tot = sum_xhalf(l_run);
   const float inv = 1.f / l_tot;
   if (row_valid) {
     bf16* dst = p.part_o + (int64_t)t.dest * kHeadDim;
