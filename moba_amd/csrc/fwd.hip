@@ -15,6 +15,7 @@
 //
 // Algorithmic work: 4*D flops per attended (query, key) pair; the bound is the bf16
 // MFMA rate.  Compulsory HBM traffic is q, k, v once, the partials once each way.
+#include <type_traits>
 #include "attn_common.h"
 
 namespace moba {
@@ -33,6 +34,12 @@ struct FwdParams {
 
 constexpr float kRescaleThreshold = 8.f;  // log2 units: the running max may lag the true max by this much
 
+// The loop is software pipelined by hand at the granularity of a 32-key block u:
+//     phase 1:  S^T(u+1)      8 MFMA   with   exponentials 8..15 of block u, packing of P(u)
+//     phase 2:  O^T += V^T P^T(u)  8 MFMA   with   row max of block u+1 and its exponentials 0..7
+// so the vector work of one block executes under the MFMAs of its neighbours, and the
+// fragment reads from LDS run a few MFMAs ahead.  K and V tiles (64 keys) are double
+// buffered separately: K(t+1) must be resident half a tile before V(t+1).
 __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -55,14 +62,13 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams p) {
 
   // ---- K/V tile loader: global -> LDS without passing through registers.
   // A wave copy fills 1 KiB = 4 keys x 16 columns of 16 bytes; wave w issues slabs
-  // w, w+4, w+8, w+12 of K and of V.  Lane i lands at slab + 16*i, so the lane picks the
-  // global column whose swizzled LDS position is i.
+  // w, w+4, w+8, w+12.  Lane i lands at slab + 16*i, so the lane picks the global column
+  // whose swizzled LDS position is i.  LDS: K stages at 0 and 16 KiB, V stages at 32 and 48 KiB.
   const int64_t row_bytes = (int64_t)H * kHeadDim * 2;
   const uint32_t lds_base = lds_addr(smem);
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   const int ld_kin = lane >> 4;  // key within the slab
   const int ld_pc = lane & 15;   // physical 16-byte column
-  // per-lane byte offset of the lane's 16 bytes inside a 64-key tile, for each of the 4 slabs
   uint32_t ld_off[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -71,38 +77,30 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams p) {
   }
   const char* k_head = (const char*)p.k + (int64_t)kv_tok0 * row_bytes + h * (kHeadDim * 2);
   const char* v_head = (const char*)p.v + (int64_t)kv_tok0 * row_bytes + h * (kHeadDim * 2);
-  auto issue_tile = [&](int kt, int buf) {
-    const uint32_t kdst = lds_base + buf * kTileBytes;
-    const uint32_t vdst = lds_base + (2 + buf) * kTileBytes;
+  auto issue = [&](const char* head, const char* tensor, int kt, uint32_t dst) __attribute__((always_inline)) {
     const int key0 = kt * TN;
     const bool full = (key0 + TN <= nkeys) && (kv_tok0 + key0 + TN <= p.t.S);
     if (full) {  // uniform tile base in SGPRs + constant per-lane offsets: no address arithmetic
-      const char* kb = k_head + (int64_t)key0 * row_bytes;
-      const char* vb = v_head + (int64_t)key0 * row_bytes;
+      const char* base = head + (int64_t)key0 * row_bytes;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int slab = 4 * i + wave_u;
-        async_copy16_sv(kb, ld_off[i], kdst + slab * 1024);
-        async_copy16_sv(vb, ld_off[i], vdst + slab * 1024);
-      }
+      for (int i = 0; i < 4; ++i) async_copy16_sv(base, ld_off[i], dst + (4 * i + wave_u) * 1024);
     } else {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int slab = 4 * i + wave_u;
-        const int key = 4 * slab + ld_kin;  // key within the tile
-        const int c16 = sw_col16(key, ld_pc);
+        const int key = 4 * slab + ld_kin;
         const int64_t tk = min((int64_t)kv_tok0 + key0 + key, (int64_t)p.t.S - 1);
-        const int64_t off = tk * row_bytes + h * (kHeadDim * 2) + c16 * 16;
-        async_copy16((const char*)p.k + off, kdst + slab * 1024);
-        async_copy16((const char*)p.v + off, vdst + slab * 1024);
+        async_copy16(tensor + tk * row_bytes + h * (kHeadDim * 2) + sw_col16(key, ld_pc) * 16, dst + slab * 1024);
       }
     }
   };
+  auto issue_k = [&](int kt, int stage) __attribute__((always_inline)) { issue(k_head, (const char*)p.k, kt, lds_base + stage * kTileBytes); };
+  auto issue_v = [&](int kt, int stage) __attribute__((always_inline)) { issue(v_head, (const char*)p.v, kt, lds_base + (2 + stage) * kTileBytes); };
   // rows of V past the end of the key range must not reach the MFMA (0 * NaN): clear them
-  auto scrub_tile = [&](int kt, int buf) {
+  auto scrub_v = [&](int kt, int stage) __attribute__((always_inline)) {
     const int key0 = kt * TN;
     if (key0 + TN <= nkeys) return;
-    char* vdst = smem + (2 + buf) * kTileBytes;
+    char* vdst = smem + (2 + stage) * kTileBytes;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int slab = 4 * i + wave;
@@ -110,17 +108,48 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams p) {
       if (key0 + key >= nkeys) *reinterpret_cast<u32x4*>(vdst + slab * 1024 + lane * 16) = u32x4{0, 0, 0, 0};
     }
   };
+  auto wait_newer4 = [&](bool newer_issued) __attribute__((always_inline)) {  // all copies landed except the newest group of 4
+    if (newer_issued) __builtin_amdgcn_s_waitcnt(0x0F74); else wait_vmem();
+  };
 
   // Tiles that run side by side on an XCD work on the same chunk; starting each at a
-  // different key tile spreads their first touches of the chunk over all of it, instead of
-  // every workgroup waiting on the same cache miss at every step.
+  // different key tile spreads their first touches of the chunk over all of it.
   const int nkt = (nkeys + TN - 1) / TN;
   const int rot = t.rot % nkt;
-  auto key_tile = [&](int it) { const int x = it + rot; return x >= nkt ? x - nkt : x; };
-  issue_tile(key_tile(0), 0);
-  wait_vmem();
-  scrub_tile(key_tile(0), 0);
-  __syncthreads();
+  auto key_tile = [&](int it) __attribute__((always_inline)) { const int x = it + rot; return x >= nkt ? x - nkt : x; };
+
+  // ---- fragment addressing: per-lane byte offsets inside a tile, everything else is an immediate ----
+  const int g16 = lane >> 4, i0 = (lane & 15) >> 2, i1 = lane & 3;
+  // K row fragment (row 32*kb + n, 16-byte column 2*s8 + hh)
+  int koff[8];
+  {
+    const int k_sw = ((n & 3) << 2) ^ ((n >> 2) & 3);
+#pragma unroll
+    for (int s8 = 0; s8 < 8; ++s8) koff[s8] = n * 256 + (((2 * s8 + hh) ^ k_sw) << 4);
+  }
+  // V^T quads: rows 32*kb + 16*j2 + 4*hh + i0 (A) and +8 (B), 8 bytes at d = 32*db + 16*(g16&1) + 4*i1
+  int voffA[4], voffB[4];
+  {
+    const int v_c16 = 2 * (g16 & 1) + (i1 >> 1);
+    const int v_sub = (i1 & 1) * 8;
+#pragma unroll
+    for (int db = 0; db < 4; ++db) {
+      const int c16 = 4 * db + v_c16;
+      voffA[db] = (4 * hh + i0) * 256 + ((c16 ^ (i0 << 2) ^ hh) << 4) + v_sub;
+      voffB[db] = (4 * hh + i0 + 8) * 256 + ((c16 ^ (i0 << 2) ^ (hh + 2)) << 4) + v_sub;
+    }
+  }
+  auto k_frag = [&](int tile_off, int kb, int s8) __attribute__((always_inline)) {
+    return *reinterpret_cast<const bf16x8*>(smem + koff[s8] + (tile_off + kb * 8192));
+  };
+  auto v_frag = [&](int tile_off, int kb, int j2, int db) __attribute__((always_inline)) {
+    const bf16x4 va = lds_read_tr(smem + voffA[db] + (tile_off + (32 * kb + 16 * j2) * 256));
+    const bf16x4 vb = lds_read_tr(smem + voffB[db] + (tile_off + (32 * kb + 16 * j2) * 256));
+    bf16x8 a;
+    a[0] = va[0]; a[1] = va[1]; a[2] = va[2]; a[3] = va[3];
+    a[4] = vb[0]; a[5] = vb[1]; a[6] = vb[2]; a[7] = vb[3];
+    return a;
+  };
 
   f32x16 oacc[4];
 #pragma unroll
@@ -130,119 +159,180 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams p) {
   float m_run = -INFINITY, l_run = 0.f;
   const float sl2 = p.scale_log2;
 
-  // per-lane pieces of the fragment addresses
-  const int g16 = lane >> 4, i0 = (lane & 15) >> 2, i1 = lane & 3;
-  // K row fragment: row 32*kb + n, column 2*s8 + hh
-  const int k_row_off = n * 256;
-  const int k_sw = ((n & 3) << 2) ^ ((n >> 2) & 3);
-  // V^T quad read: rows 16*j + 4*hh + i0 (+8), 8 bytes at d = 32*db + 16*(g16&1) + 4*i1
-  const int v_c16 = 2 * (g16 & 1) + (i1 >> 1);
-  const int v_sub = (i1 & 1) * 8;
+  // mask of a key block starting at key0 (causal diagonal / end of the key range)
+  auto mask_block = [&](f32x16& s, int key0) __attribute__((always_inline)) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e)
+      if (key0 + 8 * (e >> 2) + 4 * hh + (e & 3) > limit) s[e] = -INFINITY;
+  };
+  // running-max update for a block with row max mx (already scaled): returns the factor for older terms
+  auto update_max = [&](float mx) __attribute__((always_inline)) {
+    const float m_new = (mx > m_run + kRescaleThreshold) ? fmaxf(m_run, mx) : m_run;
+    const float alpha = fast_exp2(m_run - m_new);
+    m_run = m_new;
+    return alpha;
+  };
+// keeps a value, and therefore the instructions that produce it, at this point of the program
+#define MOBA_PIN(x) asm volatile("" : "+v"(x))
 
-  for (int it = 0; it < nkt; ++it) {
-    const int buf = it & 1;
-    const bool has_next = it + 1 < nkt;
-    const int kt = key_tile(it);
-    if (has_next) issue_tile(key_tile(it + 1), buf ^ 1);
+  // ---- prologue ----
+  issue_k(key_tile(0), 0);
+  issue_v(key_tile(0), 0);
+  if (nkt > 1) issue_k(key_tile(1), 1);
+  wait_newer4(nkt > 1);
+  scrub_v(key_tile(0), 0);
+  __syncthreads();
 
-    if (kt * TN <= t.wave_max_limit) {  // wave-uniform: skip tiles entirely above the diagonal
-      const char* ks = smem + buf * kTileBytes;
-      const char* vs = smem + (2 + buf) * kTileBytes;
-      // S^T (keys x queries), two 32-key blocks: fetch all K fragments, then two
-      // interleaved accumulation chains
-      bf16x8 ka[2][8];
-      __builtin_amdgcn_sched_barrier(0);
+  f32x16 s0, s1;   // S^T, then P^T, of the current and the next key block
+  bf16x8 pb[2];    // P^T operand of the current block: elements 0..7 and 8..15
+  {
 #pragma unroll
-      for (int s8 = 0; s8 < 8; ++s8)
+    for (int e = 0; e < 16; ++e) s0[e] = 0.f;
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-          ka[kb][s8] = *reinterpret_cast<const bf16x8*>(ks + kb * 8192 + k_row_off + (((2 * s8 + hh) ^ k_sw) << 4));
-      f32x16 sacc[2];
+    for (int s8 = 0; s8 < 8; ++s8) s0 = mfma32(k_frag(0, 0, s8), bq[s8], s0);
+    if (key_tile(0) * TN + 31 > t.wave_min_limit) mask_block(s0, key_tile(0) * TN);
+    float mx = s0[0];
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
+    for (int e = 1; e < 16; ++e) mx = fmaxf(mx, s0[e]);
+    update_max(max_xhalf(mx) * sl2);  // nothing accumulated yet: the factor is not needed
 #pragma unroll
-        for (int e = 0; e < 16; ++e) sacc[kb][e] = 0.f;
+    for (int e = 0; e < 8; ++e) {
+      const float pe = fast_exp2(s0[e] * sl2 - m_run);
+      l_run += pe;
+      pb[0][e] = (bf16)pe;
+    }
+  }
+
+  // One pipeline step on key block (tile it, block kb).  sc: its S^T with the running max decided
+  // and elements 0..7 already exponentiated into pb[0].  sn receives S^T of the next block.
+  // kn/vs: LDS byte offsets (compile-time) of the K tile of the next block and the V tile of this block.  Each of the 16 slots is one MFMA
+  // plus a share of the vector work; the pins and scheduling barriers keep that order.
+  auto step = [&](f32x16& sc, f32x16& sn, int kn, int nkb, int next_key0, auto has_next_c, bool masked, int vs,
+                  int kb) __attribute__((always_inline)) {
+    constexpr bool has_next = decltype(has_next_c)::value;
+    // ---- phase 1: S^T of the next block under exponentials 8..15 of this block ----
+    bf16x8 ka[8];
+    bf16x8 va[8];
+    float pf[8];
+    float rs = 0.f;
+    if constexpr (has_next) {
 #pragma unroll
-      for (int s8 = 0; s8 < 8; ++s8)
+      for (int i = 0; i < 4; ++i) ka[i] = k_frag(kn, nkb, i);
+    }
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb) sacc[kb] = mfma32(ka[kb][s8], bq[s8], sacc[kb]);
-      // 8 fragment reads ahead, then reads and MFMAs in step
-      __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+    for (int s8 = 0; s8 < 8; ++s8) {
+      if constexpr (has_next) {
+        if (s8 + 4 < 8) ka[s8 + 4] = k_frag(kn, nkb, s8 + 4);
+        if (s8 == 0) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+          for (int e = 0; e < 16; ++e) sn[e] = 0.f;
+        }
+        sn = mfma32(ka[s8], bq[s8], sn);
       }
-      __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+      pf[s8] = fast_exp2(sc[8 + s8] * sl2 - m_run);
+      rs += pf[s8];
+      MOBA_PIN(pf[s8]);
+      MOBA_PIN(rs);
+      if (s8 >= 6) {  // first V^T fragments of phase 2
+        va[2 * (s8 - 6)] = v_frag(vs, kb, 0, 2 * (s8 - 6));
+        va[2 * (s8 - 6) + 1] = v_frag(vs, kb, 0, 2 * (s8 - 6) + 1);
+      }
       __builtin_amdgcn_sched_barrier(0);
+    }
+    l_run += rs;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) pb[1][e] = (bf16)pf[e];
 
-      if (kt * TN + TN - 1 > t.wave_min_limit) {
+    // ---- phase 2: O^T += V^T P^T of this block under the row max and exponentials 0..7 of the next ----
+    if constexpr (has_next) {
+      if (masked) mask_block(sn, next_key0);
+    }
+    float mx = -INFINITY, alpha = 1.f, rn = 0.f;
+    float pg[8];
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
+    for (int k = 0; k < 8; ++k) {
+      const int j2 = k >> 2, db = k & 3;
+      if (k + 4 < 8) va[k + 4] = v_frag(vs, kb, 1, db);
+      oacc[db] = mfma32(va[k], pb[j2], oacc[db]);
+      if constexpr (has_next) {
+        if (k == 1) {
+          mx = fmaxf(fmaxf(sn[0], sn[1]), fmaxf(sn[2], sn[3]));
+          mx = fmaxf(mx, fmaxf(fmaxf(sn[4], sn[5]), fmaxf(sn[6], sn[7])));
+          MOBA_PIN(mx);
+        } else if (k == 2) {
+          mx = fmaxf(mx, fmaxf(fmaxf(sn[8], sn[9]), fmaxf(sn[10], sn[11])));
+          mx = fmaxf(mx, fmaxf(fmaxf(sn[12], sn[13]), fmaxf(sn[14], sn[15])));
+          MOBA_PIN(mx);
+        } else if (k == 3) {
+          alpha = update_max(max_xhalf(mx) * sl2);
+          MOBA_PIN(alpha);
+        } else if (k >= 4) {
 #pragma unroll
-          for (int e = 0; e < 16; ++e) {
-            const int key = kt * TN + 32 * kb + 8 * (e >> 2) + 4 * hh + (e & 3);
-            if (key > limit) sacc[kb][e] = -INFINITY;
+          for (int e = 2 * (k - 4); e < 2 * (k - 4) + 2; ++e) {
+            pg[e] = fast_exp2(sn[e] * sl2 - m_run);
+            rn += pg[e];
+            MOBA_PIN(pg[e]);
           }
+          MOBA_PIN(rn);
+        }
       }
-      float mx = fmaxf(sacc[0][0], sacc[1][0]);
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int e = 1; e < 16; ++e) mx = fmaxf(mx, sacc[kb][e]);
-      mx = max_xhalf(mx) * sl2;
-      // lazy running max: move it only when the tile max exceeds it by the threshold
-      if (__any(mx > m_run + kRescaleThreshold)) {
-        const float m_new = fmaxf(m_run, mx);
-        const float alpha = fast_exp2(m_run - m_new);
-        m_run = m_new;
-        l_run *= alpha;
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if constexpr (has_next) {
+      if (__any(alpha != 1.f)) {  // rare: the running max moved
 #pragma unroll
         for (int db = 0; db < 4; ++db)
 #pragma unroll
           for (int e = 0; e < 16; ++e) oacc[db][e] *= alpha;
       }
-      float rs = 0.f;
+      l_run = l_run * alpha + rn;
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const float pe = fast_exp2(sacc[kb][e] * sl2 - m_run);
-          sacc[kb][e] = pe;
-          rs += pe;
-        }
-      l_run += rs;
-      // P^T operand for the four 16-key steps
-      bf16x8 pb[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int kb = j >> 1, e0 = 8 * (j & 1);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) pb[j][e] = (bf16)sacc[kb][e0 + e];
-      }
-      // O^T += V^T P^T
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int keyA = 16 * j + 4 * hh + i0;  // keyA & 3 == i0, (keyA >> 2) & 3 == hh
-        const int keyB = keyA + 8;              // (keyB >> 2) & 3 == hh + 2
-#pragma unroll
-        for (int db = 0; db < 4; ++db) {
-          const int c16 = 4 * db + v_c16;
-          const bf16x4 va = lds_read_tr(vs + keyA * 256 + ((c16 ^ (i0 << 2) ^ hh) << 4) + v_sub);
-          const bf16x4 vb = lds_read_tr(vs + keyB * 256 + ((c16 ^ (i0 << 2) ^ (hh + 2)) << 4) + v_sub);
-          bf16x8 a;
-          a[0] = va[0]; a[1] = va[1]; a[2] = va[2]; a[3] = va[3];
-          a[4] = vb[0]; a[5] = vb[1]; a[6] = vb[2]; a[7] = vb[3];
-          oacc[db] = mfma32(a, pb[j], oacc[db]);
-        }
-      }
+      for (int e = 0; e < 8; ++e) pb[0][e] = (bf16)pg[e];
     }
-    if (has_next) {
-      wait_vmem();
-      scrub_tile(key_tile(it + 1), buf ^ 1);
+  };
+
+  // st: LDS stage of this tile (= parity of it), compile-time so that every LDS address is
+  // a per-lane register plus an immediate
+  auto tile_body = [&](int it, auto st_c, auto more_c) __attribute__((always_inline)) {
+    constexpr int st = decltype(st_c)::value;
+    constexpr bool more = decltype(more_c)::value;  // a tile follows this one
+    constexpr int kcur = st * kTileBytes, knext = (st ^ 1) * kTileBytes, vcur = (2 + st) * kTileBytes;
+    const int key0 = key_tile(it) * TN;
+    const int key0n = more ? key_tile(it + 1) * TN : 0;
+    // the mask is needed once a key block reaches past the smallest row limit of the wave
+    const bool mask_a = key0 + 63 > t.wave_min_limit;
+    const bool mask_b = more && (key0n + 31 > t.wave_min_limit);
+    if constexpr (more) issue_v(key_tile(it + 1), st ^ 1);  // V(it-1) is dead since the barrier that ended tile it-1
+
+    step(s0, s1, kcur, 1, key0 + 32, std::true_type{}, mask_a, vcur, 0);
+
+    // K(it) is dead; K(it+1) must be visible for the second half of this tile
+    if constexpr (more) wait_newer4(true);
+    __syncthreads();
+    if (it + 2 < nkt) issue_k(key_tile(it + 2), st);
+
+    step(s1, s0, knext, 0, key0n, more_c, mask_b, vcur, 1);
+
+    if constexpr (more) {
+      wait_newer4(it + 2 < nkt);
+      scrub_v(key_tile(it + 1), st ^ 1);
     }
     __syncthreads();
+  };
+  using St0 = std::integral_constant<int, 0>;
+  using St1 = std::integral_constant<int, 1>;
+  int it = 0;
+  for (; it + 2 < nkt; it += 2) {
+    tile_body(it, St0{}, std::true_type{});
+    tile_body(it + 1, St1{}, std::true_type{});
   }
+  if (it + 2 == nkt) {
+    tile_body(it, St0{}, std::true_type{});
+    tile_body(it + 1, St1{}, std::false_type{});
+  } else {
+    tile_body(it, St0{}, std::false_type{});
+  }
+#undef MOBA_PIN
 
   // ---- epilogue: normalise, write the partial ----
   const float l_tot = sum_xhalf(l_run);
