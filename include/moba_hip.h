@@ -85,21 +85,6 @@ int moba_fwd(const void* q, const void* k, const void* v, void* part_o, float* p
              const int32_t* chunk_tok, const int32_t* self_tile_prefix, void* out, float* lse, int64_t S, int H, int D,
              int K, int F, int N, int B, int64_t hist_bound, int64_t self_tiles, void* stream);
 
-/* Wide-tile variant of moba_fwd_partials: 256 query rows per workgroup, software
- * pipelined; tile_off and self_tile_prefix must be counted in moba_fwd_wide_tile_rows()-row
- * tiles.  Same results as moba_fwd_partials up to fp32 summation order. */
-int moba_fwd_wide_tile_rows(void);
-int moba_fwd_partials_wide(const void* q, const void* k, const void* v, void* part_o, float* part_lse,
-                           const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest,
-                           const int32_t* fchunk_tok, const int32_t* chunk_tok, const int32_t* self_tile_prefix,
-                           int64_t S, int H, int D, int K, int F, int N, int B, int64_t hist_bound, int64_t self_tiles,
-                           void* stream);
-
-/* Helpers on int32 device arrays: exclusive prefix sum in place of a[0..n) with the total at
- * a[n]; and the tile_off table (nseg+1 entries) of a gather list for another row-tile size. */
-void moba_scan_i32(int32_t* a, int n, void* stream);
-int moba_tile_offsets(const int32_t* seg_off, int32_t* tile_off, int nseg, int tile_rows, void* stream);
-
 /* Backward.  Replaces MixedAttention.backward, moba/moba_efficient.py:185-267, and the
  * autograd scatter of its gathered gradients.  Deterministic (no floating-point atomics).
  *   dout, q, k, v, out [S,H,D] bf16; lse [S,H] fp32 from the forward

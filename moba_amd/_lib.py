@@ -27,10 +27,6 @@ _SIGNATURES = {
     "moba_build_lists": (c_int, [c_void_p] * 9 + [c_int64] + [c_int] * 7 + [c_void_p]),
     "moba_fwd_tile_rows": (c_int, []),
     "moba_fwd_partials": (c_int, [c_void_p] * 11 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_int64, c_void_p]),
-    "moba_fwd_wide_tile_rows": (c_int, []),
-    "moba_fwd_partials_wide": (c_int, [c_void_p] * 11 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_int64, c_void_p]),
-    "moba_scan_i32": (None, [c_void_p, c_int, c_void_p]),
-    "moba_tile_offsets": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "moba_fwd_merge": (c_int, [c_void_p] * 5 + [c_int64, c_int, c_int, c_int, c_void_p]),
     "moba_fwd": (c_int, [c_void_p] * 14 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_int64, c_void_p]),
     "moba_bwd": (c_int, [c_void_p] * 19 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_int64, c_void_p]),

@@ -14,7 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(CSRC, "build")
 LIB = os.path.join(HERE, "libmoba_hip.so")
-SOURCES = ["chunk_mean.hip", "gate_topk.hip", "lists.hip", "fwd.hip", "fwd_wide.hip", "bwd.hip", "capi.hip"]
+SOURCES = ["chunk_mean.hip", "gate_topk.hip", "lists.hip", "fwd.hip", "bwd.hip", "capi.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -27,7 +27,7 @@ FLAGS = [
 
 # per-source extra flags: the attention kernels never produce NaN from finite inputs, and
 # telling the compiler so removes the canonicalisation of every MFMA result before a max
-EXTRA = {"fwd.hip": ["-fno-honor-nans"], "fwd_wide.hip": ["-fno-honor-nans"]}
+EXTRA = {"fwd.hip": ["-fno-honor-nans"]}
 
 
 def _compile(src: str, force: bool) -> str:

@@ -193,11 +193,6 @@ __global__ __launch_bounds__(256) void lists_segments_kernel(const int* __restri
 
 using namespace moba;
 
-// exclusive prefix sum of a[0..n) in place, total at a[n] (device array of n+1 ints)
-extern "C" void moba_scan_i32(int32_t* a, int n, void* stream) {
-  hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, a, n);
-}
-
 // Limits: chunks per sequence minus one (cmax) is bounded by the LDS the fill pass
 // needs, 48 bytes per candidate chunk.
 extern "C" int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, const int32_t* chunk_fb,

@@ -14,13 +14,12 @@ Stages (each also callable on its own, which is how the tests reach them):
 from __future__ import annotations
 
 import ctypes
-import os
 from typing import Optional
 
 import torch
 
 from . import _lib
-from .plan import MobaPlan, TILE_ROWS, WIDE_TILE_ROWS, make_plan
+from .plan import MobaPlan, TILE_ROWS, make_plan
 
 HEAD_DIM = 128
 
@@ -82,26 +81,7 @@ def topk_from_scores(scores: torch.Tensor, K: int) -> torch.Tensor:
     return sel
 
 
-def fwd_tile_rows(plan: MobaPlan) -> int:
-    """Row tile of the forward kernel used for this plan: the wide (256-row, software
-    pipelined) kernel pays off once a chunk holds several key tiles per row tile."""
-    forced = os.environ.get("MOBA_FWD_TILE_ROWS")
-    if forced:
-        return int(forced)
-    longest = plan.chunk_size if not plan.fallback else max(b - a for a, b in zip(plan.cu[:-1], plan.cu[1:]))
-    return WIDE_TILE_ROWS if longest >= 512 else TILE_ROWS
-
-
-def tile_offsets(seg_off: torch.Tensor, tile_rows: int) -> torch.Tensor:
-    """tile_off table of a gather list for another row-tile size."""
-    lib = _lib.load()
-    out = torch.empty_like(seg_off)
-    _lib.check(lib.moba_tile_offsets(_ptr(seg_off), _ptr(out), seg_off.numel() - 1, tile_rows, _stream(seg_off.device)),
-               "moba_tile_offsets")
-    return out
-
-
-def build_lists(sel: torch.Tensor, plan: MobaPlan, tile_rows: int = TILE_ROWS):
+def build_lists(sel: torch.Tensor, plan: MobaPlan):
     """(seg_off [F*H+1], tile_off [F*H+1], seg_dest [M]) int32 -- see csrc/lists.hip."""
     lib = _lib.load()
     S, H, K = sel.shape
@@ -114,7 +94,7 @@ def build_lists(sel: torch.Tensor, plan: MobaPlan, tile_rows: int = TILE_ROWS):
     t = plan.tables
     _lib.check(lib.moba_build_lists(_ptr(sel), _ptr(t["chunk_tok"]), _ptr(t["chunk_fb"]), _ptr(t["chunk_local"]),
                                     _ptr(t["pair_off"]), _ptr(cnt), _ptr(seg_off), _ptr(tile_off), _ptr(seg_dest),
-                                    S, H, K, plan.N, plan.F, plan.P, plan.cmax, tile_rows, _stream(dev)),
+                                    S, H, K, plan.N, plan.F, plan.P, plan.cmax, TILE_ROWS, _stream(dev)),
                "moba_build_lists")
     return seg_off, tile_off, seg_dest
 
@@ -163,8 +143,6 @@ def _forward(q, k, v, plan: MobaPlan, timer: Optional[StageTimer] = None):
     K = plan.K
     t = plan.tables
     span = (lambda name: timer.span(name, dev)) if timer is not None else (lambda name: _NoSpan())
-    rows = fwd_tile_rows(plan)
-    wide = rows == WIDE_TILE_ROWS
     if plan.fallback:
         sel = seg_off = tile_off = seg_dest = None
     else:
@@ -173,23 +151,20 @@ def _forward(q, k, v, plan: MobaPlan, timer: Optional[StageTimer] = None):
         with span("gate_topk"):
             sel = gate_topk(q, kbar, plan)
         with span("build_lists"):
-            seg_off, tile_off, seg_dest = build_lists(sel, plan, rows)
+            seg_off, tile_off, seg_dest = build_lists(sel, plan)
     part_o = torch.empty((S * H * (K + 1), D), dtype=q.dtype, device=dev)
     part_lse = torch.empty((S * H * (K + 1),), dtype=torch.float32, device=dev)
     out = torch.empty_like(q)
     lse = torch.empty((S, H), dtype=torch.float32, device=dev)
     with span("fwd_partials"):
-        fn = lib.moba_fwd_partials_wide if wide else lib.moba_fwd_partials
-        _lib.check(fn(_ptr(q), _ptr(k), _ptr(v), _ptr(part_o), _ptr(part_lse), _ptr(seg_off), _ptr(tile_off),
-                      _ptr(seg_dest), _ptr(t.get("fchunk_tok")), _ptr(t["chunk_tok"]),
-                      _ptr(t["self_tile_prefix_wide" if wide else "self_tile_prefix"]), S, H, D, K, plan.F, plan.N,
-                      plan.chunk_size, plan.hist_tile_bound(H, rows), plan.self_tiles_wide if wide else plan.self_tiles,
-                      _stream(dev)), "moba_fwd_partials")
+        _lib.check(lib.moba_fwd_partials(_ptr(q), _ptr(k), _ptr(v), _ptr(part_o), _ptr(part_lse), _ptr(seg_off),
+                                         _ptr(tile_off), _ptr(seg_dest), _ptr(t.get("fchunk_tok")),
+                                         _ptr(t["chunk_tok"]), _ptr(t["self_tile_prefix"]), S, H, D, K, plan.F, plan.N,
+                                         plan.chunk_size, plan.hist_tile_bound(H), plan.self_tiles, _stream(dev)),
+                   "moba_fwd_partials")
     with span("fwd_merge"):
         _lib.check(lib.moba_fwd_merge(_ptr(part_o), _ptr(part_lse), _ptr(sel), _ptr(out), _ptr(lse), S, H, D, K,
                                       _stream(dev)), "moba_fwd_merge")
-    if tile_off is not None and rows != TILE_ROWS:
-        tile_off = None  # the backward kernels use 128-row tiles: rebuilt on demand
     return out, lse, sel, seg_off, tile_off, seg_dest
 
 
@@ -199,8 +174,6 @@ def _backward(dout, q, k, v, out, lse, sel, seg_off, tile_off, seg_dest, plan: M
     dev = q.device
     K = plan.K
     t = plan.tables
-    if tile_off is None and seg_off is not None:
-        tile_off = tile_offsets(seg_off, TILE_ROWS)
     dq = torch.empty_like(q)
     dk = torch.empty_like(k)
     dv = torch.empty_like(v)

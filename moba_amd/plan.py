@@ -16,8 +16,7 @@ from typing import Dict, List, Tuple
 import numpy as np
 import torch
 
-TILE_ROWS = 128       # query rows per workgroup of the 128-row attention kernels (forward and backward)
-WIDE_TILE_ROWS = 256  # query rows per workgroup of the wide forward kernel
+TILE_ROWS = 128  # query rows per workgroup of the attention kernels
 
 
 @dataclass
@@ -35,14 +34,13 @@ class MobaPlan:
     P: int              # (filtered chunk, later chunk of the same sequence) pairs
     cmax: int           # max chunks per sequence minus one
     pairs_per_head: int  # selected (token, chunk) pairs per head  (M / H)
-    self_tiles: int     # 128-row tiles of the self part, per head
-    self_tiles_wide: int  # 256-row tiles of the self part, per head
+    self_tiles: int     # row tiles of the self part, per head
     flops_per_head: float
     tables: Dict[str, torch.Tensor] = field(default_factory=dict)
     host: Dict[str, np.ndarray] = field(default_factory=dict)
 
-    def hist_tile_bound(self, H: int, tile_rows: int = TILE_ROWS) -> int:
-        return (self.pairs_per_head * H) // tile_rows + self.F * H
+    def hist_tile_bound(self, H: int) -> int:
+        return (self.pairs_per_head * H) // TILE_ROWS + self.F * H
 
 
 def _host_tables(cu: np.ndarray, B: int, topk: int):
@@ -67,11 +65,9 @@ def _host_tables(cu: np.ndarray, B: int, topk: int):
     N = int(n_chunks.sum())
     tiles = (chunk_len + TILE_ROWS - 1) // TILE_ROWS
     self_tile_prefix = np.concatenate([[0], np.cumsum(tiles)])
-    tiles_w = (chunk_len + WIDE_TILE_ROWS - 1) // WIDE_TILE_ROWS
-    out = dict(chunk_tok=chunk_tok, self_tile_prefix=self_tile_prefix,
-               self_tile_prefix_wide=np.concatenate([[0], np.cumsum(tiles_w)]))
+    out = dict(chunk_tok=chunk_tok, self_tile_prefix=self_tile_prefix)
     info = dict(nseq=nseq, N=N, F=0 if fallback else F, k_eff=k_eff, fallback=fallback, K=0, P=0, cmax=0,
-                pairs_per_head=0, self_tiles=int(tiles.sum()), self_tiles_wide=int(tiles_w.sum()))
+                pairs_per_head=0, self_tiles=int(tiles.sum()))
     pairs_self = int((chunk_len.astype(np.int64) * (chunk_len + 1) // 2).sum())
     if not fallback:
         seq_fbase = np.concatenate([[0], np.cumsum(n_chunks - 1)])
@@ -121,7 +117,7 @@ def make_plan(cu_seqlens, chunk_size: int, moba_topk: int, device=None) -> MobaP
     plan = MobaPlan(cu=cu.tolist(), chunk_size=int(chunk_size), moba_topk=int(moba_topk), S=int(cu[-1]),
                     nseq=info["nseq"], N=info["N"], F=info["F"], k_eff=info["k_eff"], K=info["K"],
                     fallback=info["fallback"], P=info["P"], cmax=info["cmax"], pairs_per_head=info["pairs_per_head"],
-                    self_tiles=info["self_tiles"], self_tiles_wide=info["self_tiles_wide"], flops_per_head=info["flops_per_head_per_d"], host=host)
+                    self_tiles=info["self_tiles"], flops_per_head=info["flops_per_head_per_d"], host=host)
     if device is not None and torch.device(device).type != "cpu":
         names = list(host)
         flat = np.concatenate([host[n_].astype(np.int32) for n_ in names])
