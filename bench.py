@@ -29,6 +29,9 @@ sys.path.insert(0, ROOT)
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of moba_fwd_kernel from rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled by a copy
+# kernel of known size (profiles/moba_fwd_128k_hbm_traffic.txt); measured for the headline workload only
+FWD_KERNEL_TRAFFIC_BYTES = {"cfg4_L131072_h32_c4096_k12": 46.69e9}
 
 WORKLOADS = {
     # name: (seq lens or None, heads, kv_heads, chunk, topk, normalise, backward)
@@ -145,7 +148,7 @@ def main():
         "stage_ms": stage_ms,
         "roofline": {"kernel": "moba_fwd_kernel", "bound": "mfma", "achieved": achieved,
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
-                     "traffic": None},
+                     "traffic": FWD_KERNEL_TRAFFIC_BYTES.get(args.workload)},
     }
     if "chunk_mean" in stage_ms:
         gbs = S * H * D * 2 / (stage_ms["chunk_mean"] * 1e-3) / 1e9
