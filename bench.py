@@ -98,6 +98,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default=DEFAULT, choices=list(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--backward", action="store_true", help="also time forward + backward")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
@@ -127,6 +128,23 @@ def main():
     dt = (time.perf_counter() - t0) / args.steps
     stage_ms = {name: sum(x) / len(x) for name, x in timer.ms().items()}
 
+    # forward + backward (reported beside the forward figure for the workloads that name it)
+    fwd_bwd_ms = None
+    if WORKLOADS[args.workload][6] or args.backward:
+        g = torch.Generator(device=dev).manual_seed(1)
+        do = torch.randn(q.shape, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+        qg, kg, vg = (x.clone().requires_grad_(True) for x in (q, k, v))
+        for _ in range(max(1, args.warmup)):
+            E.moba_attn_varlen(qg, kg, vg, cu_t, max_seqlen, B, topk).backward(do)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for _ in range(args.steps):
+            qg.grad = kg.grad = vg.grad = None
+            E.moba_attn_varlen(qg, kg, vg, cu_t, max_seqlen, B, topk).backward(do)
+        torch.cuda.synchronize()
+        fwd_bwd_ms = (time.perf_counter() - t1) / args.steps * 1e3
+        del qg, kg, vg, do
+
     kern_ms = stage_ms["fwd_partials"]
     achieved = flops / (kern_ms * 1e-3) / 1e12
     result = {
@@ -150,6 +168,9 @@ def main():
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
                      "traffic": FWD_KERNEL_TRAFFIC_BYTES.get(args.workload)},
     }
+    if fwd_bwd_ms is not None:
+        # algorithmic backward work is 2.5x the forward's
+        result["fwd_bwd"] = {"ms_per_step": fwd_bwd_ms, "tflops": 3.5 * flops / (fwd_bwd_ms * 1e-3) / 1e12}
     if "chunk_mean" in stage_ms:
         gbs = S * H * D * 2 / (stage_ms["chunk_mean"] * 1e-3) / 1e9
         result["chunk_mean_hbm"] = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
