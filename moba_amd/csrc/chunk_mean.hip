@@ -28,16 +28,17 @@ __global__ __launch_bounds__(256) void chunk_mean_partial_kernel(
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.0;
   int t = t0;
-  for (; t + 4 <= t1; t += 4) {
-    bf16x8 x0 = *reinterpret_cast<const bf16x8*>(src);
-    bf16x8 x1 = *reinterpret_cast<const bf16x8*>(src + row_stride);
-    bf16x8 x2 = *reinterpret_cast<const bf16x8*>(src + 2 * row_stride);
-    bf16x8 x3 = *reinterpret_cast<const bf16x8*>(src + 3 * row_stride);
-    src += 4 * row_stride;
+  for (; t + 8 <= t1; t += 8) {
+    bf16x8 x[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) x[u] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(src + u * row_stride));
+    src += 8 * row_stride;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      // the four-term sum of bf16 values is exact in fp64 whatever the order
-      acc[e] += ((double)(float)x0[e] + (double)(float)x1[e]) + ((double)(float)x2[e] + (double)(float)x3[e]);
+      // sums of bf16 values are exact in fp64 whatever the order
+      const double a = ((double)(float)x[0][e] + (double)(float)x[1][e]) + ((double)(float)x[2][e] + (double)(float)x[3][e]);
+      const double b = ((double)(float)x[4][e] + (double)(float)x[5][e]) + ((double)(float)x[6][e] + (double)(float)x[7][e]);
+      acc[e] += a + b;
     }
   }
   for (; t < t1; ++t) {
@@ -79,8 +80,9 @@ using namespace moba;
 static int pick_nsplit(int HD8, int F, int B) {
   const int colblocks = (HD8 + 255) / 256;
   int nsplit = 1;
-  // enough workgroups to fill 256 CUs several times over, at least 32 tokens per split
-  while ((int64_t)colblocks * F * nsplit < 4096 && B / (nsplit * 2) >= 32) nsplit *= 2;
+  // enough workgroups to keep every CU's memory pipeline full (8 row loads in flight per lane),
+  // few enough that the fp64 partial sums stay a small fraction of the traffic
+  while ((int64_t)colblocks * F * nsplit < 1536 && B / (nsplit * 2) >= 64) nsplit *= 2;
   return nsplit;
 }
 

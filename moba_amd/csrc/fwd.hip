@@ -364,27 +364,41 @@ __global__ __launch_bounds__(256) void moba_merge_kernel(const bf16* __restrict_
   const int K = K1 - 1;
   const float* pl = part_lse + row * K1;
   const int* ps = sel + row * K;
+  // absent slots are redirected to slot 0 with weight 0, so every load below is
+  // unconditional and the loads of a group of four slots are in flight together
   float mx = pl[0];
-  for (int j = 0; j < K; ++j)
-    if (ps[j] >= 0) mx = fmaxf(mx, pl[1 + j]);
+  for (int j = 0; j < K; ++j) {
+    const float l = pl[1 + j];
+    mx = ps[j] >= 0 ? fmaxf(mx, l) : mx;
+  }
   float acc[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.f;
   float wsum = 0.f;
   const bf16* po = part_o + row * K1 * kHeadDim + c8 * 8;
-  for (int j = 0; j < K1; ++j) {
-    if (j > 0 && ps[j - 1] < 0) continue;
-    const float w = fast_exp2(pl[j] - mx);
-    wsum += w;
-    const bf16x8 x = *reinterpret_cast<const bf16x8*>(po + (int64_t)j * kHeadDim);
+  for (int j0 = 0; j0 < K1; j0 += 4) {
+    bf16x8 x[4];
+    float w[4];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) acc[e] += w * (float)x[e];
+    for (int u = 0; u < 4; ++u) {
+      const int j = j0 + u;
+      const bool ok = j < K1 && (j == 0 || ps[j < K1 ? j - 1 : 0] >= 0);
+      const int jj = ok ? j : 0;
+      x[u] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(po + (int64_t)jj * kHeadDim));
+      w[u] = ok ? fast_exp2(pl[jj] - mx) : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      wsum += w[u];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] += w[u] * (float)x[u][e];
+    }
   }
   const float inv = 1.f / wsum;
   bf16x8 o;
 #pragma unroll
   for (int e = 0; e < 8; ++e) o[e] = (bf16)(acc[e] * inv);
-  *reinterpret_cast<bf16x8*>(out + row * kHeadDim + c8 * 8) = o;
+  __builtin_nontemporal_store(o, reinterpret_cast<bf16x8*>(out + row * kHeadDim + c8 * 8));
   if (c8 == 0) lse[row] = (mx + fast_log2(wsum)) * 0.6931471805599453f;
 }
 
