@@ -96,10 +96,15 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default=DEFAULT, choices=list(WORKLOADS))
+    ap.add_argument("--workload", default=DEFAULT, help="one of %s, or its cfgN prefix" % ", ".join(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--backward", action="store_true", help="also time forward + backward")
     args = ap.parse_args()
+    if args.workload not in WORKLOADS:
+        match = [w for w in WORKLOADS if w.split("_")[0] == args.workload]
+        if len(match) != 1:
+            ap.error("unknown workload %r" % args.workload)
+        args.workload = match[0]
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
         sys.exit(2)

@@ -89,7 +89,7 @@ int moba_fwd(const void* q, const void* k, const void* v, void* part_o, float* p
  * autograd scatter of its gathered gradients.  Deterministic (no floating-point atomics).
  *   dout, q, k, v, out [S,H,D] bf16; lse [S,H] fp32 from the forward
  *   chunk_fid [N] int32: filtered id of each chunk, -1 for the last chunk of a sequence
- *   delta [S,H] fp32 scratch; part_dq [S*H*(K+1), D] fp32 scratch
+ *   delta [2,S,H] fp32 scratch (rowsum(dO*O), then the LSE in the log2 domain); part_dq [S*H*(K+1), D] fp32 scratch
  *   dq, dk, dv [S,H,D] bf16 out */
 int moba_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out, const float* lse,
              const int32_t* sel, const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest,

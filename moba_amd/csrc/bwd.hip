@@ -19,6 +19,8 @@
 // All matrix products use v_mfma_f32_32x32x16_bf16; transposed operands come from
 // ds_read_b64_tr_b16.  Algorithmic work: 10*D flops per attended (query, key) pair
 // (the recomputation of S and dO V^T in both kernels adds 4*D on top).
+#include <type_traits>
+
 #include "attn_common.h"
 
 namespace moba {
@@ -27,7 +29,8 @@ constexpr float kLog2e = 1.4426950408889634f;
 constexpr int TQ = 64;                                  // query rows per step of the dK/dV kernel
 constexpr int kBwdDqLds = 4 * kTileBytes;               // K[2], V[2]
 constexpr int kQStage = 2 * TQ * kHeadDim * 2 + 2 * TQ * 4;  // Q tile, dO tile, lse, delta
-constexpr int kBwdDkvLds = 2 * kQStage;
+constexpr int kDkvStages = 3;
+constexpr int kBwdDkvLds = kDkvStages * kQStage;
 
 struct BwdParams {
   const bf16* q;
@@ -36,6 +39,7 @@ struct BwdParams {
   const bf16* dout;
   const float* lse;    // [S*H] natural log
   const float* delta;  // [S*H]
+  const float* lse2;   // [S*H] lse in the log2 domain
   float* part_dq;      // [S*H*K1, D] fp32
   bf16* dk;
   bf16* dv;
@@ -43,10 +47,13 @@ struct BwdParams {
   TileTables t;
   float scale_log2;
   float scale;
+  uint32_t hk_magic;  // n / (H*K1) == (n * hk_magic) >> hk_shift for every n < 2^31
+  uint32_t hk_shift;
 };
 
 __global__ __launch_bounds__(256) void bwd_delta_kernel(const bf16* __restrict__ dout, const bf16* __restrict__ out,
-                                                        float* __restrict__ delta, int64_t rows) {
+                                                        const float* __restrict__ lse, float* __restrict__ delta,
+                                                        float* __restrict__ lse2, int64_t rows) {
   const int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
   const int c8 = threadIdx.x & 15;
   float acc = 0.f;
@@ -58,7 +65,10 @@ __global__ __launch_bounds__(256) void bwd_delta_kernel(const bf16* __restrict__
   }
 #pragma unroll
   for (int o = 8; o >= 1; o >>= 1) acc += __shfl_xor(acc, o, 64);
-  if (row < rows && c8 == 0) delta[row] = acc;
+  if (row < rows && c8 == 0) {
+    delta[row] = acc;
+    lse2[row] = lse[row] * kLog2e;
+  }
 }
 
 // ------------------------------------------------------------------------------------ dQ
@@ -314,20 +324,30 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams p) {
   const uint32_t lds_base = lds_addr(smem);
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   const int ld_rin = lane >> 4, ld_pc = lane & 15;
-  // token of row `row` (0..TQ-1) of query tile qi; rows past the end repeat the last row
-  auto row_token = [&](int qi, int row) -> int {
-    if (qi < nself) return c0 + key0 + min(qi * TQ + row, self_rows - 1);
-    const int idx = min((qi - nself) * TQ + row, list_rows - 1);
-    return p.t.seg_dest[list_base + idx] / (H * K1);
+  // Row lookups run one stage ahead of the copies: fetch_rows(qi) starts the loads of the
+  // gather-list entries of stage qi (self stages need none), issue_stage(qi) turns them into
+  // tokens and issues the copies.  Rows past the end repeat the last row.
+  int raw[5];  // rows 4*(4*i + wave) + lane/16 for i < 4 (Q and dO copies), row = lane (lse, delta)
+  auto fetch_rows = [&](int qi) __attribute__((always_inline)) {
+    if (qi < nself || qi >= ntile) return;
+    const int base = (qi - nself) * TQ;
+    const int* src = p.t.seg_dest + list_base;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) raw[i] = src[min(base + 4 * (4 * i + wave_u) + ld_rin, list_rows - 1)];
+    raw[4] = src[min(base + lane, list_rows - 1)];
   };
-  auto issue_stage = [&](int qi, int buf) {
+  auto issue_stage = [&](int qi, int buf) __attribute__((always_inline)) {
     const uint32_t qdst = lds_base + buf * kQStage;
     const uint32_t odst = qdst + TQ * kHeadDim * 2;
-    // all row lookups first, so that the copies are issued back to back
-    int toks[4];
+    int toks[5];
+    if (qi < nself) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) toks[i] = row_token(qi, 4 * (4 * i + wave_u) + ld_rin);
-    const int tok_l = row_token(qi, lane);
+      for (int i = 0; i < 4; ++i) toks[i] = c0 + key0 + min(qi * TQ + 4 * (4 * i + wave_u) + ld_rin, self_rows - 1);
+      toks[4] = c0 + key0 + min(qi * TQ + lane, self_rows - 1);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 5; ++i) toks[i] = (int)(((uint64_t)(uint32_t)raw[i] * p.hk_magic) >> p.hk_shift);
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int slab = 4 * i + wave_u;
@@ -338,7 +358,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams p) {
       async_copy16((const char*)p.dout + off, odst + slab * 1024);
     }
     if (wave_u < 2) {
-      const float* src = (wave_u == 0 ? p.lse : p.delta) + ((int64_t)tok_l * H + h);
+      const float* src = (wave_u == 0 ? p.lse2 : p.delta) + ((int64_t)toks[4] * H + h);
       async_copy4(src, qdst + 2 * TQ * kHeadDim * 2 + wave_u * (TQ * 4));
     }
   };
@@ -356,96 +376,172 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams p) {
   const int tr_c16 = 2 * (g16 & 1) + (i1 >> 1);
   const int tr_sub = (i1 & 1) * 8;
 
-  if (ntile > 0) {
-    issue_stage(0, 0);
-    wait_vmem();
-  }
-  __syncthreads();
-
-  for (int qi = 0; qi < ntile; ++qi) {
-    const int buf = qi & 1;
-    const bool has_next = qi + 1 < ntile;
-    if (has_next) issue_stage(qi + 1, buf ^ 1);
-
-    const char* qs = smem + buf * kQStage;
+  // The loop is software pipelined over blocks of 32 query rows (two per stage):
+  //   phase A of block b: the 16 MFMAs of S and dO V^T of block b+1, one per slot, each slot
+  //                       also holding the exponential of one element of block b -- MFMA and
+  //                       VALU pipes busy together;
+  //   phase B of block b: dV^T += dO^T P and dK^T += Q^T dS (16 MFMAs fed by transposed LDS
+  //                       reads), while the row fragments and softmax statistics that the
+  //                       next phase A needs are fetched from LDS.
+  // Three LDS stages and one barrier per stage: at the barrier after phase A of the first
+  // block of stage s every wave is past stage s-1, whose buffer then takes stage s+2, and the
+  // copies of stage s+1 (issued one stage earlier) have landed.
+#define MOBA_PIN(x) asm volatile("" : "+v"(x))
+  bf16x8 qa[8], oa[8];  // row fragments of the block whose S comes next
+  f32x4 l4[4], d4[4];   // log2-LSE and delta of the rows of the block whose P comes next
+  auto load_frags = [&](const char* qs, int qb) __attribute__((always_inline)) {
     const char* os = qs + TQ * kHeadDim * 2;
+#pragma unroll
+    for (int s8 = 0; s8 < 8; ++s8) {
+      const int o = qb * 8192 + row_off + (((2 * s8 + hh) ^ row_sw) << 4);
+      qa[s8] = *reinterpret_cast<const bf16x8*>(qs + o);
+      oa[s8] = *reinterpret_cast<const bf16x8*>(os + o);
+    }
+  };
+  auto load_stats = [&](const char* qs, int qb) __attribute__((always_inline)) {
     const float* lse_s = reinterpret_cast<const float*>(qs + 2 * TQ * kHeadDim * 2);
     const float* del_s = lse_s + TQ;
-    const bool is_self = qi < nself;
-    // number of real rows in this tile, and for self tiles the chunk position of row 0
-    const int rows_here = is_self ? min(TQ, self_rows - qi * TQ) : min(TQ, list_rows - (qi - nself) * TQ);
-    const int qpos0 = key0 + qi * TQ;  // only meaningful for self tiles
-    // causal masking can only bite while the tile's first row is before the wave's last key
-    const bool masked = (rows_here < TQ) || (is_self && qpos0 < key0 + wave * 32 + 31);
-
 #pragma unroll
-    for (int qb = 0; qb < 2; ++qb) {
-      // S (queries x keys) and dO V^T: lane = key, elements = queries 32*qb + 8g + 4hh + r
-      bf16x8 qa[8], oa[8];
-      __builtin_amdgcn_sched_barrier(0);
+    for (int g = 0; g < 4; ++g) {
+      l4[g] = *reinterpret_cast<const f32x4*>(lse_s + 32 * qb + 8 * g + 4 * hh);
+      d4[g] = *reinterpret_cast<const f32x4*>(del_s + 32 * qb + 8 * g + 4 * hh);
+    }
+  };
+  // S and dO V^T from qa/oa into (s_next, dp_next); P and dS of (s_cur, dp_cur) with l4/d4.
+  // Block rows are 32*qb + 8g + 4hh + r; `rows_ok` rows of the stage are real, self stages are causal.
+  auto phase_a = [&](f32x16& s_next, f32x16& dp_next, const f32x16& s_cur, const f32x16& dp_cur, auto masked_c,
+                     int qb, int rows_ok, bool is_self, int qpos0, bf16x8 (&pb)[2], bf16x8 (&dsb)[2])
+                     __attribute__((always_inline)) {
+    f32x16 zero;
 #pragma unroll
-      for (int s8 = 0; s8 < 8; ++s8) {
-        const int o = qb * 8192 + row_off + (((2 * s8 + hh) ^ row_sw) << 4);
-        qa[s8] = *reinterpret_cast<const bf16x8*>(qs + o);
-        oa[s8] = *reinterpret_cast<const bf16x8*>(os + o);
-      }
-      f32x16 sacc, dpacc;
+    for (int e = 0; e < 16; ++e) zero[e] = 0.f;
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int e = 0; e < 16; ++e) { sacc[e] = 0.f; dpacc[e] = 0.f; }
+    for (int k = 0; k < 16; k += 2) {
+      const int s8 = k >> 1;
+      float pe[2], ds[2];
 #pragma unroll
-      for (int s8 = 0; s8 < 8; ++s8) {
-        sacc = mfma32(qa[s8], bk[s8], sacc);
-        dpacc = mfma32(oa[s8], bv[s8], dpacc);
-      }
-      __builtin_amdgcn_sched_group_barrier(0x100, 16, 0);
-      __builtin_amdgcn_sched_group_barrier(0x008, 16, 0);
-      __builtin_amdgcn_sched_barrier(0);
-
-      bf16x8 pb[2], dsb[2];
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const f32x4 l4 = *reinterpret_cast<const f32x4*>(lse_s + 32 * qb + 8 * g + 4 * hh);
-        const f32x4 d4 = *reinterpret_cast<const f32x4*>(del_s + 32 * qb + 8 * g + 4 * hh);
-#pragma unroll
-        for (int rr = 0; rr < 4; ++rr) {
-          const int e = 4 * g + rr;
+      for (int u = 0; u < 2; ++u) {
+        if (u == 0) s_next = mfma32(qa[s8], bk[s8], s8 == 0 ? zero : s_next);
+        else        dp_next = mfma32(oa[s8], bv[s8], s8 == 0 ? zero : dp_next);
+        const int e = k + u, g = e >> 2, rr = e & 3;
+        pe[u] = fast_exp2(s_cur[e] * sl2 - l4[g][rr]);
+        if constexpr (decltype(masked_c)::value) {
           const int row = 32 * qb + 8 * g + 4 * hh + rr;
-          float pe = fast_exp2(sacc[e] * sl2 - l4[rr] * kLog2e);
-          if (masked) {
-            const bool ok = (row < rows_here) && (!is_self || qpos0 + row >= mykey);
-            pe = ok ? pe : 0.f;
-          }
-          pb[e >> 3][e & 7] = (bf16)pe;
-          dsb[e >> 3][e & 7] = (bf16)(pe * (dpacc[e] - d4[rr]));
+          const bool ok = (row < rows_ok) && (!is_self || qpos0 + row >= mykey);
+          pe[u] = ok ? pe[u] : 0.f;
         }
+        ds[u] = pe[u] * (dp_cur[e] - d4[g][rr]);
+        MOBA_PIN(pe[u]);
+        MOBA_PIN(ds[u]);
+        __builtin_amdgcn_sched_barrier(0);
       }
-      // dV^T += dO^T P and dK^T += Q^T dS  (contraction over the 32 queries, two steps of 16)
+      pb[k >> 3][k & 7] = (bf16)pe[0];
+      pb[k >> 3][(k & 7) + 1] = (bf16)pe[1];
+      dsb[k >> 3][k & 7] = (bf16)ds[0];
+      dsb[k >> 3][(k & 7) + 1] = (bf16)ds[1];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  // accumulate block (qs, qb); then fetch the fragments of (qs_f, qb_f) and the statistics of (qs_s, qb_s)
+  auto phase_b = [&](const char* qs, int qb, const bf16x8 (&pb)[2], const bf16x8 (&dsb)[2], const char* qs_f, int qb_f,
+                     const char* qs_s, int qb_s) __attribute__((always_inline)) {
+    const char* os = qs + TQ * kHeadDim * 2;
 #pragma unroll
-      for (int j2 = 0; j2 < 2; ++j2) {
-        const int rowA = 32 * qb + 16 * j2 + 4 * hh + i0;
-        const int rowB = rowA + 8;
+    for (int j2 = 0; j2 < 2; ++j2) {
+      const int rowA = 32 * qb + 16 * j2 + 4 * hh + i0;
+      const int rowB = rowA + 8;
 #pragma unroll
-        for (int db = 0; db < 4; ++db) {
-          const int c16 = 4 * db + tr_c16;
-          const int offA = rowA * 256 + ((c16 ^ (i0 << 2) ^ hh) << 4) + tr_sub;
-          const int offB = rowB * 256 + ((c16 ^ (i0 << 2) ^ (hh + 2)) << 4) + tr_sub;
-          const bf16x4 oa4 = lds_read_tr(os + offA);
-          const bf16x4 ob4 = lds_read_tr(os + offB);
-          const bf16x4 qa4 = lds_read_tr(qs + offA);
-          const bf16x4 qb4 = lds_read_tr(qs + offB);
-          bf16x8 ao, aq;
-          ao[0] = oa4[0]; ao[1] = oa4[1]; ao[2] = oa4[2]; ao[3] = oa4[3];
-          ao[4] = ob4[0]; ao[5] = ob4[1]; ao[6] = ob4[2]; ao[7] = ob4[3];
-          aq[0] = qa4[0]; aq[1] = qa4[1]; aq[2] = qa4[2]; aq[3] = qa4[3];
-          aq[4] = qb4[0]; aq[5] = qb4[1]; aq[6] = qb4[2]; aq[7] = qb4[3];
-          dvacc[db] = mfma32(ao, pb[j2], dvacc[db]);
-          dkacc[db] = mfma32(aq, dsb[j2], dkacc[db]);
-        }
+      for (int db = 0; db < 4; ++db) {
+        const int c16 = 4 * db + tr_c16;
+        const int offA = rowA * 256 + ((c16 ^ (i0 << 2) ^ hh) << 4) + tr_sub;
+        const int offB = rowB * 256 + ((c16 ^ (i0 << 2) ^ (hh + 2)) << 4) + tr_sub;
+        const bf16x4 oa4 = lds_read_tr(os + offA);
+        const bf16x4 ob4 = lds_read_tr(os + offB);
+        const bf16x4 qa4 = lds_read_tr(qs + offA);
+        const bf16x4 qb4 = lds_read_tr(qs + offB);
+        bf16x8 ao, aq;
+        ao[0] = oa4[0]; ao[1] = oa4[1]; ao[2] = oa4[2]; ao[3] = oa4[3];
+        ao[4] = ob4[0]; ao[5] = ob4[1]; ao[6] = ob4[2]; ao[7] = ob4[3];
+        aq[0] = qa4[0]; aq[1] = qa4[1]; aq[2] = qa4[2]; aq[3] = qa4[3];
+        aq[4] = qb4[0]; aq[5] = qb4[1]; aq[6] = qb4[2]; aq[7] = qb4[3];
+        dvacc[db] = mfma32(ao, pb[j2], dvacc[db]);
+        dkacc[db] = mfma32(aq, dsb[j2], dkacc[db]);
       }
     }
+    load_stats(qs_s, qb_s);
+    load_frags(qs_f, qb_f);
+    // 8 transposed reads ahead, then four reads per pair of MFMAs; the prefetches ride behind
+    __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+#pragma unroll
+    for (int i = 0; i < 6; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+#pragma unroll
+  for (int i = 0; i < 5; ++i) raw[i] = 0;
+  fetch_rows(0);
+  issue_stage(0, 0);
+  fetch_rows(1);
+  wait_vmem();
+  __syncthreads();
+  if (ntile > 1) issue_stage(1, 1);
+  fetch_rows(2);
+
+  // S of block 0 (a phase A whose softmax half works on zeros and is discarded)
+  f32x16 sA, dA, sB, dB;
+  {
+    bf16x8 pb[2], dsb[2];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) { sB[e] = 0.f; dB[e] = 0.f; }
+#pragma unroll
+    for (int g = 0; g < 4; ++g) { l4[g] = f32x4{0.f, 0.f, 0.f, 0.f}; d4[g] = l4[g]; }
+    load_frags(smem, 0);
+    phase_a(sA, dA, sB, dB, std::false_type{}, 0, 0, false, 0, pb, dsb);
+    load_stats(smem, 0);
+    load_frags(smem, 1);
+  }
+  int buf = 0;
+  for (int qi = 0; qi < ntile; ++qi) {
+    const char* qs = smem + buf * kQStage;
+    const int buf1 = buf == 2 ? 0 : buf + 1;
+    const int buf2 = buf1 == 2 ? 0 : buf1 + 1;
+    const bool has_next = qi + 1 < ntile;
+    const bool is_self = qi < nself;
+    // number of real rows in this stage, and for self stages the chunk position of row 0
+    const int rows_here = is_self ? min(TQ, self_rows - qi * TQ) : min(TQ, list_rows - (qi - nself) * TQ);
+    const int qpos0 = key0 + qi * TQ;  // only meaningful for self stages
+    // causal masking can only bite while the stage's first row is before the wave's last key
+    const bool masked = (rows_here < TQ) || (is_self && qpos0 < key0 + wave * 32 + 31);
+    // the block after the last one is the last one again: its S is computed and dropped
+    const char* qs_next = has_next ? smem + buf1 * kQStage : qs;
+    bf16x8 pb[2], dsb[2];
+
+    if (masked) phase_a(sB, dB, sA, dA, std::true_type{}, 0, rows_here, is_self, qpos0, pb, dsb);
+    else        phase_a(sB, dB, sA, dA, std::false_type{}, 0, rows_here, is_self, qpos0, pb, dsb);
+
     if (has_next) wait_vmem();
     __syncthreads();
+    if (qi + 2 < ntile) issue_stage(qi + 2, buf2);
+    fetch_rows(qi + 3);
+
+    phase_b(qs, 0, pb, dsb, qs_next, 0, qs, 1);
+    if (masked) phase_a(sA, dA, sB, dB, std::true_type{}, 1, rows_here, is_self, qpos0, pb, dsb);
+    else        phase_a(sA, dA, sB, dB, std::false_type{}, 1, rows_here, is_self, qpos0, pb, dsb);
+    phase_b(qs, 1, pb, dsb, qs_next, 1, qs_next, 0);
+    buf = buf1;
   }
+#undef MOBA_PIN
 
   if (key_valid) {
     const int64_t off = ((int64_t)(c0 + mykey) * H + h) * kHeadDim;
@@ -492,7 +588,7 @@ extern "C" int moba_bwd(const void* dout, const void* q, const void* k, const vo
 
   BwdParams p;
   p.q = (const bf16*)q; p.k = (const bf16*)k; p.v = (const bf16*)v; p.dout = (const bf16*)dout;
-  p.lse = lse; p.delta = delta; p.part_dq = part_dq; p.dk = (bf16*)dk; p.dv = (bf16*)dv;
+  p.lse = lse; p.delta = delta; p.lse2 = delta + S * H; p.part_dq = part_dq; p.dk = (bf16*)dk; p.dv = (bf16*)dv;
   p.chunk_fid = chunk_fid;
   p.t.seg_off = seg_off; p.t.tile_off = tile_off; p.t.seg_dest = seg_dest; p.t.fchunk_tok = fchunk_tok;
   p.t.chunk_tok = chunk_tok; p.t.self_tile_prefix = self_tile_prefix;
@@ -501,6 +597,13 @@ extern "C" int moba_bwd(const void* dout, const void* q, const void* k, const vo
   p.t.self_total = (int)(self_tiles * H);
   p.scale = (float)(1.0 / sqrt((double)D));
   p.scale_log2 = (float)(1.4426950408889634 / sqrt((double)D));
+  // division by H*K1 as a multiplication: with s = 31 + ceil(log2 d) and m = floor(2^s / d) + 1 the
+  // error m*d - 2^s is at most d <= 2^(s-31), so n*m >> s is the exact quotient for n < 2^31; m < 2^32
+  const uint64_t hk = (uint64_t)H * (K + 1);
+  uint32_t lg = 0;
+  while ((1ull << lg) < hk) ++lg;
+  p.hk_shift = 31 + lg;
+  p.hk_magic = (uint32_t)((1ull << p.hk_shift) / hk + 1);
 
   hipStream_t st = (hipStream_t)stream;
   static bool attr_set = false;
@@ -514,7 +617,7 @@ extern "C" int moba_bwd(const void* dout, const void* q, const void* k, const vo
   }
   const int64_t rows = S * H;
   hipLaunchKernelGGL(bwd_delta_kernel, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st, (const bf16*)dout,
-                     (const bf16*)out, delta, rows);
+                     (const bf16*)out, lse, delta, delta + S * H, rows);
   hipLaunchKernelGGL(bwd_dq_kernel, dim3((unsigned)grid_q), dim3(256), kBwdDqLds, st, p);
   hipLaunchKernelGGL(bwd_dq_reduce_kernel, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st,
                      (const float*)part_dq, sel, (bf16*)dq, rows, K + 1, p.scale);

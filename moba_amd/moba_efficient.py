@@ -177,7 +177,7 @@ def _backward(dout, q, k, v, out, lse, sel, seg_off, tile_off, seg_dest, plan: M
     dq = torch.empty_like(q)
     dk = torch.empty_like(k)
     dv = torch.empty_like(v)
-    delta = torch.empty((S, H), dtype=torch.float32, device=dev)
+    delta = torch.empty((2, S, H), dtype=torch.float32, device=dev)
     part_dq = torch.empty((S * H * (K + 1), D), dtype=torch.float32, device=dev)
     _lib.check(lib.moba_bwd(_ptr(dout), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(sel), _ptr(seg_off),
                             _ptr(tile_off), _ptr(seg_dest), _ptr(t.get("fchunk_tok")), _ptr(t["chunk_tok"]),
