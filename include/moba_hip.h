@@ -6,7 +6,9 @@
  * pointers unless stated otherwise; tensors are contiguous; `stream` is a hipStream_t.
  * The library allocates nothing, frees nothing, and never synchronises the device:
  * every launch is enqueued on `stream`.  Return value: 0, or a negative code that
- * moba_strerror() explains.  bf16 data, head_dim 128.
+ * moba_strerror() explains.  head_dim 128; q, k, v and everything derived from them are
+ * bf16 (dtype = MOBA_DTYPE_BF16) or fp16 (dtype = MOBA_DTYPE_F16, the dtype of the reference's
+ * example, examples/llama.py:26); below, "elem" stands for that type.
  *
  * Shapes use: S packed tokens, H heads, D head_dim, B chunk size, N chunks,
  * F filtered chunks (chunks that are not the last of their sequence), K selected
@@ -23,18 +25,20 @@
 extern "C" {
 #endif
 
+enum { MOBA_DTYPE_BF16 = 0, MOBA_DTYPE_F16 = 1 };
+
 int moba_version(void);
 const char* moba_strerror(int code);
 
 /* Key chunk-mean.  Replaces moba/moba_efficient.py:326-340 (index_select of the
  * filtered chunks, .mean(dim=1) on bf16, .float()).
- *   k          [S,H,D] bf16
+ *   k          [S,H,D] elem
  *   fchunk_tok [F] int32, first token of each filtered chunk
- *   kbar       [F,H,D] bf16 out
+ *   kbar       [F,H,D] elem out (the mean rounded once to the element type)
  *   workspace  moba_chunk_mean_workspace_bytes() bytes, 8-byte aligned */
 size_t moba_chunk_mean_workspace_bytes(int H, int D, int F, int B);
 int moba_chunk_mean(const void* k, const int32_t* fchunk_tok, void* kbar, void* workspace, int64_t S, int H, int D,
-                    int F, int B, void* stream);
+                    int F, int B, int dtype, void* stream);
 
 /* Gate scores + causal top-k.  Replaces moba/moba_efficient.py:341-371 (fp32 einsum,
  * -inf mask, torch.topk, dropping -inf picks).
@@ -44,7 +48,7 @@ int moba_chunk_mean(const void* k, const int32_t* fchunk_tok, void* kbar, void* 
  *              score of every valid candidate (debug / test output), may be NULL
  * K <= 64. */
 int moba_gate_topk(const void* q, const void* kbar, const int32_t* cu_seqlens, const int32_t* seq_fbase, int32_t* sel,
-                   float* scores_out, int64_t S, int H, int D, int nseq, int F, int B, int K, void* stream);
+                   float* scores_out, int64_t S, int H, int D, int nseq, int F, int B, int K, int dtype, void* stream);
 
 /* The selection step of moba/moba_efficient.py:365-371 alone, on caller-supplied
  * scores [S,H,F] fp32 (-inf = not a candidate).  Same routine as moba_gate_topk. */
@@ -68,34 +72,35 @@ int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, const int32_t
 /* Attention.  Replaces MixedAttention.forward, moba/moba_efficient.py:69-183 (two
  * flash-attn varlen forwards and the LSE merge), and with K = 0 and one chunk per
  * sequence the full-causal case of moba/moba_efficient.py:318-321.
- *   part_o [S*H*(K+1), D] bf16 and part_lse [S*H*(K+1)] fp32: per-slot partial results
+ *   part_o [S*H*(K+1), D] elem and part_lse [S*H*(K+1)] fp32: per-slot partial results
  *   self_tile_prefix [N+1] int32: prefix sum of ceil(chunk_len / moba_fwd_tile_rows())
- *   out [S,H,D] bf16, lse [S,H] fp32 (natural log)
+ *   out [S,H,D] elem, lse [S,H] fp32 (natural log)
  *   hist_bound: upper bound on the number of history tiles, e.g. M/tile_rows + F*H
  *   self_tiles: self_tile_prefix[N] */
 int moba_fwd_tile_rows(void);
 int moba_fwd_partials(const void* q, const void* k, const void* v, void* part_o, float* part_lse,
                       const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest,
                       const int32_t* fchunk_tok, const int32_t* chunk_tok, const int32_t* self_tile_prefix, int64_t S,
-                      int H, int D, int K, int F, int N, int B, int64_t hist_bound, int64_t self_tiles, void* stream);
+                      int H, int D, int K, int F, int N, int B, int64_t hist_bound, int64_t self_tiles, int dtype,
+                      void* stream);
 int moba_fwd_merge(const void* part_o, const float* part_lse, const int32_t* sel, void* out, float* lse, int64_t S,
-                   int H, int D, int K, void* stream);
+                   int H, int D, int K, int dtype, void* stream);
 int moba_fwd(const void* q, const void* k, const void* v, void* part_o, float* part_lse, const int32_t* sel,
              const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest, const int32_t* fchunk_tok,
              const int32_t* chunk_tok, const int32_t* self_tile_prefix, void* out, float* lse, int64_t S, int H, int D,
-             int K, int F, int N, int B, int64_t hist_bound, int64_t self_tiles, void* stream);
+             int K, int F, int N, int B, int64_t hist_bound, int64_t self_tiles, int dtype, void* stream);
 
 /* Backward.  Replaces MixedAttention.backward, moba/moba_efficient.py:185-267, and the
  * autograd scatter of its gathered gradients.  Deterministic (no floating-point atomics).
- *   dout, q, k, v, out [S,H,D] bf16; lse [S,H] fp32 from the forward
+ *   dout, q, k, v, out [S,H,D] elem; lse [S,H] fp32 from the forward
  *   chunk_fid [N] int32: filtered id of each chunk, -1 for the last chunk of a sequence
  *   delta [2,S,H] fp32 scratch (rowsum(dO*O), then the LSE in the log2 domain); part_dq [S*H*(K+1), D] fp32 scratch
- *   dq, dk, dv [S,H,D] bf16 out */
+ *   dq, dk, dv [S,H,D] elem out */
 int moba_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out, const float* lse,
              const int32_t* sel, const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest,
              const int32_t* fchunk_tok, const int32_t* chunk_tok, const int32_t* self_tile_prefix,
              const int32_t* chunk_fid, float* delta, float* part_dq, void* dq, void* dk, void* dv, int64_t S, int H,
-             int D, int K, int F, int N, int B, int64_t hist_bound, int64_t self_tiles, void* stream);
+             int D, int K, int F, int N, int B, int64_t hist_bound, int64_t self_tiles, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

@@ -112,8 +112,18 @@ __device__ __forceinline__ float sum_xhalf(float x) {
 __device__ __forceinline__ int sw_col16(int row, int c16) { return c16 ^ ((row & 3) << 2) ^ ((row >> 2) & 3); }
 __device__ __forceinline__ int tile_off16(int row, int c16) { return row * 256 + (sw_col16(row, c16) << 4); }
 
-__device__ __forceinline__ bf16x4 lds_read_tr(const char* p) {
-  return __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) bf16x4*)(p));
+__device__ __forceinline__ void lds_read_tr(const char* p, bf16x4& out) {
+  out = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) bf16x4*)(p));
+}
+__device__ __forceinline__ void lds_read_tr(const char* p, f16x4& out) {
+  typedef __attribute__((ext_vector_type(4))) short i16x4;
+  out = __builtin_bit_cast(f16x4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4*)(p)));
+}
+template <class V4>
+__device__ __forceinline__ V4 lds_read_tr(const char* p) {
+  V4 r;
+  lds_read_tr(p, r);
+  return r;
 }
 
 // asynchronous 16-byte copy global -> LDS: lane i of the wave fills lds_wave_base + 16*i.

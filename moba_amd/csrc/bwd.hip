@@ -32,17 +32,18 @@ constexpr int kQStage = 2 * TQ * kHeadDim * 2 + 2 * TQ * 4;  // Q tile, dO tile,
 constexpr int kDkvStages = 3;
 constexpr int kBwdDkvLds = kDkvStages * kQStage;
 
+template <class E>
 struct BwdParams {
-  const bf16* q;
-  const bf16* k;
-  const bf16* v;
-  const bf16* dout;
+  const typename E::elem* q;
+  const typename E::elem* k;
+  const typename E::elem* v;
+  const typename E::elem* dout;
   const float* lse;    // [S*H] natural log
   const float* delta;  // [S*H]
   const float* lse2;   // [S*H] lse in the log2 domain
   float* part_dq;      // [S*H*K1, D] fp32
-  bf16* dk;
-  bf16* dv;
+  typename E::elem* dk;
+  typename E::elem* dv;
   const int* chunk_fid;  // [N] filtered id of a chunk, -1 for the last chunk of a sequence
   TileTables t;
   float scale_log2;
@@ -51,15 +52,18 @@ struct BwdParams {
   uint32_t hk_shift;
 };
 
-__global__ __launch_bounds__(256) void bwd_delta_kernel(const bf16* __restrict__ dout, const bf16* __restrict__ out,
+template <class E>
+__global__ __launch_bounds__(256) void bwd_delta_kernel(const typename E::elem* __restrict__ dout,
+                                                        const typename E::elem* __restrict__ out,
                                                         const float* __restrict__ lse, float* __restrict__ delta,
                                                         float* __restrict__ lse2, int64_t rows) {
+  MOBA_ELEM_TYPES(E)
   const int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
   const int c8 = threadIdx.x & 15;
   float acc = 0.f;
   if (row < rows) {
-    const bf16x8 a = *reinterpret_cast<const bf16x8*>(dout + row * kHeadDim + c8 * 8);
-    const bf16x8 b = *reinterpret_cast<const bf16x8*>(out + row * kHeadDim + c8 * 8);
+    const elem8 a = *reinterpret_cast<const elem8*>(dout + row * kHeadDim + c8 * 8);
+    const elem8 b = *reinterpret_cast<const elem8*>(out + row * kHeadDim + c8 * 8);
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc += (float)a[e] * (float)b[e];
   }
@@ -72,7 +76,9 @@ __global__ __launch_bounds__(256) void bwd_delta_kernel(const bf16* __restrict__
 }
 
 // ------------------------------------------------------------------------------------ dQ
-__global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
+template <class E>
+__global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams<E> p) {
+  MOBA_ELEM_TYPES(E)
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int n = lane & 31, hh = lane >> 5;
@@ -84,13 +90,13 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
   const int h = t.h, nkeys = t.nkeys, kv_tok0 = t.kv_tok0, limit = t.limit;
   const bool row_valid = r < t.row_count;
 
-  bf16x8 bq[8], bdo[8];
+  elem8 bq[8], bdo[8];
   {
     const int64_t off = ((int64_t)t.tok * H + h) * kHeadDim + 8 * hh;
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
-      bq[ks] = *reinterpret_cast<const bf16x8*>(p.q + off + 16 * ks);
-      bdo[ks] = *reinterpret_cast<const bf16x8*>(p.dout + off + 16 * ks);
+      bq[ks] = *reinterpret_cast<const elem8*>(p.q + off + 16 * ks);
+      bdo[ks] = *reinterpret_cast<const elem8*>(p.dout + off + 16 * ks);
     }
   }
   const float lse2 = p.lse[(int64_t)t.tok * H + h] * kLog2e;
@@ -165,13 +171,13 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb) {
         // S^T and (dO V^T)^T for 32 keys x 32 queries: two independent MFMA chains
-        bf16x8 ka[8], va[8];
+        elem8 ka[8], va[8];
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int s8 = 0; s8 < 8; ++s8) {
           const int o = kb * 8192 + row_off + (((2 * s8 + hh) ^ row_sw) << 4);
-          ka[s8] = *reinterpret_cast<const bf16x8*>(ks + o);
-          va[s8] = *reinterpret_cast<const bf16x8*>(vs + o);
+          ka[s8] = *reinterpret_cast<const elem8*>(ks + o);
+          va[s8] = *reinterpret_cast<const elem8*>(vs + o);
         }
         f32x16 sacc, dpacc;
 #pragma unroll
@@ -197,11 +203,11 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
             if (key > limit) sacc[e] = -INFINITY;
           }
         }
-        bf16x8 dsb[2];
+        elem8 dsb[2];
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
           const float pe = fast_exp2(sacc[e] * sl2 - lse2);
-          dsb[e >> 3][e & 7] = (bf16)(pe * (dpacc[e] - dl));
+          dsb[e >> 3][e & 7] = (elem)(pe * (dpacc[e] - dl));
         }
         // dQ^T += K^T dS^T
 #pragma unroll
@@ -212,9 +218,9 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
 #pragma unroll
           for (int db = 0; db < 4; ++db) {
             const int c16 = 4 * db + tr_c16;
-            const bf16x4 xa = lds_read_tr(ks + keyA * 256 + ((c16 ^ (i0 << 2) ^ hh) << 4) + tr_sub);
-            const bf16x4 xb = lds_read_tr(ks + keyB * 256 + ((c16 ^ (i0 << 2) ^ (hh + 2)) << 4) + tr_sub);
-            bf16x8 a;
+            const elem4 xa = lds_read_tr<elem4>(ks + keyA * 256 + ((c16 ^ (i0 << 2) ^ hh) << 4) + tr_sub);
+            const elem4 xb = lds_read_tr<elem4>(ks + keyB * 256 + ((c16 ^ (i0 << 2) ^ (hh + 2)) << 4) + tr_sub);
+            elem8 a;
             a[0] = xa[0]; a[1] = xa[1]; a[2] = xa[2]; a[3] = xa[3];
             a[4] = xb[0]; a[5] = xb[1]; a[6] = xb[2]; a[7] = xb[3];
             dqacc[db] = mfma32(a, dsb[j2], dqacc[db]);
@@ -244,9 +250,12 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams p) {
 }
 
 // dq[row] = scale * sum over the row's valid slots of part_dq; 16 lanes per row
+template <class E>
 __global__ __launch_bounds__(256) void bwd_dq_reduce_kernel(const float* __restrict__ part_dq,
-                                                            const int* __restrict__ sel, bf16* __restrict__ dq,
-                                                            int64_t rows, int K1, float scale) {
+                                                            const int* __restrict__ sel,
+                                                            typename E::elem* __restrict__ dq, int64_t rows, int K1,
+                                                            float scale) {
+  MOBA_ELEM_TYPES(E)
   const int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
   if (row >= rows) return;
   const int c8 = threadIdx.x & 15;
@@ -263,14 +272,16 @@ __global__ __launch_bounds__(256) void bwd_dq_reduce_kernel(const float* __restr
 #pragma unroll
     for (int e = 0; e < 4; ++e) { acc[e] += a[e]; acc[4 + e] += b[e]; }
   }
-  bf16x8 o;
+  elem8 o;
 #pragma unroll
-  for (int e = 0; e < 8; ++e) o[e] = (bf16)(acc[e] * scale);
-  *reinterpret_cast<bf16x8*>(dq + row * kHeadDim + c8 * 8) = o;
+  for (int e = 0; e < 8; ++e) o[e] = (elem)(acc[e] * scale);
+  *reinterpret_cast<elem8*>(dq + row * kHeadDim + c8 * 8) = o;
 }
 
 // ------------------------------------------------------------------------------------ dK, dV
-__global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams p) {
+template <class E>
+__global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
+  MOBA_ELEM_TYPES(E)
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int n = lane & 31, hh = lane >> 5;
@@ -310,13 +321,13 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams p) {
   const int ntile = nself + nhist;
 
   // ---- K^T and V^T operands of this lane's key: [16*ks + 8*hh .. +7] ----
-  bf16x8 bk[8], bv[8];
+  elem8 bk[8], bv[8];
   {
     const int64_t off = ((int64_t)(c0 + min(mykey, len - 1)) * H + h) * kHeadDim + 8 * hh;
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
-      bk[ks] = *reinterpret_cast<const bf16x8*>(p.k + off + 16 * ks);
-      bv[ks] = *reinterpret_cast<const bf16x8*>(p.v + off + 16 * ks);
+      bk[ks] = *reinterpret_cast<const elem8*>(p.k + off + 16 * ks);
+      bv[ks] = *reinterpret_cast<const elem8*>(p.v + off + 16 * ks);
     }
   }
 
@@ -387,15 +398,15 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams p) {
   // block of stage s every wave is past stage s-1, whose buffer then takes stage s+2, and the
   // copies of stage s+1 (issued one stage earlier) have landed.
 #define MOBA_PIN(x) asm volatile("" : "+v"(x))
-  bf16x8 qa[8], oa[8];  // row fragments of the block whose S comes next
+  elem8 qa[8], oa[8];  // row fragments of the block whose S comes next
   f32x4 l4[4], d4[4];   // log2-LSE and delta of the rows of the block whose P comes next
   auto load_frags = [&](const char* qs, int qb) __attribute__((always_inline)) {
     const char* os = qs + TQ * kHeadDim * 2;
 #pragma unroll
     for (int s8 = 0; s8 < 8; ++s8) {
       const int o = qb * 8192 + row_off + (((2 * s8 + hh) ^ row_sw) << 4);
-      qa[s8] = *reinterpret_cast<const bf16x8*>(qs + o);
-      oa[s8] = *reinterpret_cast<const bf16x8*>(os + o);
+      qa[s8] = *reinterpret_cast<const elem8*>(qs + o);
+      oa[s8] = *reinterpret_cast<const elem8*>(os + o);
     }
   };
   auto load_stats = [&](const char* qs, int qb) __attribute__((always_inline)) {
@@ -410,7 +421,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams p) {
   // S and dO V^T from qa/oa into (s_next, dp_next); P and dS of (s_cur, dp_cur) with l4/d4.
   // Block rows are 32*qb + 8g + 4hh + r; `rows_ok` rows of the stage are real, self stages are causal.
   auto phase_a = [&](f32x16& s_next, f32x16& dp_next, const f32x16& s_cur, const f32x16& dp_cur, auto masked_c,
-                     int qb, int rows_ok, bool is_self, int qpos0, bf16x8 (&pb)[2], bf16x8 (&dsb)[2])
+                     int qb, int rows_ok, bool is_self, int qpos0, elem8 (&pb)[2], elem8 (&dsb)[2])
                      __attribute__((always_inline)) {
     f32x16 zero;
 #pragma unroll
@@ -436,15 +447,15 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams p) {
         MOBA_PIN(ds[u]);
         __builtin_amdgcn_sched_barrier(0);
       }
-      pb[k >> 3][k & 7] = (bf16)pe[0];
-      pb[k >> 3][(k & 7) + 1] = (bf16)pe[1];
-      dsb[k >> 3][k & 7] = (bf16)ds[0];
-      dsb[k >> 3][(k & 7) + 1] = (bf16)ds[1];
+      pb[k >> 3][k & 7] = (elem)pe[0];
+      pb[k >> 3][(k & 7) + 1] = (elem)pe[1];
+      dsb[k >> 3][k & 7] = (elem)ds[0];
+      dsb[k >> 3][(k & 7) + 1] = (elem)ds[1];
     }
     __builtin_amdgcn_sched_barrier(0);
   };
   // accumulate block (qs, qb); then fetch the fragments of (qs_f, qb_f) and the statistics of (qs_s, qb_s)
-  auto phase_b = [&](const char* qs, int qb, const bf16x8 (&pb)[2], const bf16x8 (&dsb)[2], const char* qs_f, int qb_f,
+  auto phase_b = [&](const char* qs, int qb, const elem8 (&pb)[2], const elem8 (&dsb)[2], const char* qs_f, int qb_f,
                      const char* qs_s, int qb_s) __attribute__((always_inline)) {
     const char* os = qs + TQ * kHeadDim * 2;
 #pragma unroll
@@ -456,11 +467,11 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams p) {
         const int c16 = 4 * db + tr_c16;
         const int offA = rowA * 256 + ((c16 ^ (i0 << 2) ^ hh) << 4) + tr_sub;
         const int offB = rowB * 256 + ((c16 ^ (i0 << 2) ^ (hh + 2)) << 4) + tr_sub;
-        const bf16x4 oa4 = lds_read_tr(os + offA);
-        const bf16x4 ob4 = lds_read_tr(os + offB);
-        const bf16x4 qa4 = lds_read_tr(qs + offA);
-        const bf16x4 qb4 = lds_read_tr(qs + offB);
-        bf16x8 ao, aq;
+        const elem4 oa4 = lds_read_tr<elem4>(os + offA);
+        const elem4 ob4 = lds_read_tr<elem4>(os + offB);
+        const elem4 qa4 = lds_read_tr<elem4>(qs + offA);
+        const elem4 qb4 = lds_read_tr<elem4>(qs + offB);
+        elem8 ao, aq;
         ao[0] = oa4[0]; ao[1] = oa4[1]; ao[2] = oa4[2]; ao[3] = oa4[3];
         ao[4] = ob4[0]; ao[5] = ob4[1]; ao[6] = ob4[2]; ao[7] = ob4[3];
         aq[0] = qa4[0]; aq[1] = qa4[1]; aq[2] = qa4[2]; aq[3] = qa4[3];
@@ -501,7 +512,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams p) {
   // S of block 0 (a phase A whose softmax half works on zeros and is discarded)
   f32x16 sA, dA, sB, dB;
   {
-    bf16x8 pb[2], dsb[2];
+    elem8 pb[2], dsb[2];
 #pragma unroll
     for (int e = 0; e < 16; ++e) { sB[e] = 0.f; dB[e] = 0.f; }
 #pragma unroll
@@ -525,7 +536,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams p) {
     const bool masked = (rows_here < TQ) || (is_self && qpos0 < key0 + wave * 32 + 31);
     // the block after the last one is the last one again: its S is computed and dropped
     const char* qs_next = has_next ? smem + buf1 * kQStage : qs;
-    bf16x8 pb[2], dsb[2];
+    elem8 pb[2], dsb[2];
 
     if (masked) phase_a(sB, dB, sA, dA, std::true_type{}, 0, rows_here, is_self, qpos0, pb, dsb);
     else        phase_a(sB, dB, sA, dA, std::false_type{}, 0, rows_here, is_self, qpos0, pb, dsb);
@@ -550,10 +561,10 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams p) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         u32x2 wk, wv;
-        wk[0] = pack_bf16(dkacc[db][4 * g + 0] * p.scale, dkacc[db][4 * g + 1] * p.scale);
-        wk[1] = pack_bf16(dkacc[db][4 * g + 2] * p.scale, dkacc[db][4 * g + 3] * p.scale);
-        wv[0] = pack_bf16(dvacc[db][4 * g + 0], dvacc[db][4 * g + 1]);
-        wv[1] = pack_bf16(dvacc[db][4 * g + 2], dvacc[db][4 * g + 3]);
+        wk[0] = pack2<E>(dkacc[db][4 * g + 0] * p.scale, dkacc[db][4 * g + 1] * p.scale);
+        wk[1] = pack2<E>(dkacc[db][4 * g + 2] * p.scale, dkacc[db][4 * g + 3] * p.scale);
+        wv[0] = pack2<E>(dvacc[db][4 * g + 0], dvacc[db][4 * g + 1]);
+        wv[1] = pack2<E>(dvacc[db][4 * g + 2], dvacc[db][4 * g + 3]);
         *reinterpret_cast<u32x2*>(p.dk + off + 32 * db + 8 * g + 4 * hh) = wk;
         *reinterpret_cast<u32x2*>(p.dv + off + 32 * db + 8 * g + 4 * hh) = wv;
       }
@@ -564,37 +575,17 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams p) {
 
 using namespace moba;
 
-extern "C" int moba_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out,
-                        const float* lse, const int32_t* sel, const int32_t* seg_off, const int32_t* tile_off,
-                        const int32_t* seg_dest, const int32_t* fchunk_tok, const int32_t* chunk_tok,
-                        const int32_t* self_tile_prefix, const int32_t* chunk_fid, float* delta, float* part_dq,
-                        void* dq, void* dk, void* dv, int64_t S, int H, int D, int K, int F, int N, int B,
-                        int64_t hist_bound, int64_t self_tiles, void* stream) {
-  if (!dout || !q || !k || !v || !out || !lse || !chunk_tok || !self_tile_prefix || !delta || !part_dq || !dq ||
-      !dk || !dv)
-    return MOBA_ERR_ARG;
-  if (K > 0 && (!sel || !seg_off || !tile_off || !seg_dest || !fchunk_tok || !chunk_fid)) return MOBA_ERR_ARG;
-  if (D != kHeadDim) return MOBA_ERR_UNSUPPORTED;
-  if (S <= 0 || H <= 0 || K < 0 || F < 0 || N <= 0 || B <= 0 || hist_bound < 0 || self_tiles <= 0) return MOBA_ERR_ARG;
-  const void* ptrs[] = {dout, q, k, v, out, part_dq, dq, dk, dv};
-  for (const void* x : ptrs)
-    if ((uintptr_t)x & 15) return MOBA_ERR_ARG;
-  if ((int64_t)S * H * (K + 1) >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
-  const int64_t per = 8 * kXcdBlock;
-  const int64_t total_q = (K > 0 ? hist_bound : 0) + self_tiles * H;
-  const int64_t grid_q = (total_q + per - 1) / per * per;
-  const int64_t grid_kv = (self_tiles * H + per - 1) / per * per;
-  if (grid_q >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
-
-  BwdParams p;
-  p.q = (const bf16*)q; p.k = (const bf16*)k; p.v = (const bf16*)v; p.dout = (const bf16*)dout;
-  p.lse = lse; p.delta = delta; p.lse2 = delta + S * H; p.part_dq = part_dq; p.dk = (bf16*)dk; p.dv = (bf16*)dv;
+template <class E>
+static int launch_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out, const float* lse,
+                      const int32_t* sel, const int32_t* chunk_fid, float* delta, float* part_dq, void* dq, void* dk,
+                      void* dv, const TileTables& t, int64_t S, int H, int D, int K, int64_t grid_q, int64_t grid_kv,
+                      hipStream_t st) {
+  typedef typename E::elem elem;
+  BwdParams<E> p;
+  p.q = (const elem*)q; p.k = (const elem*)k; p.v = (const elem*)v; p.dout = (const elem*)dout;
+  p.lse = lse; p.delta = delta; p.lse2 = delta + S * H; p.part_dq = part_dq; p.dk = (elem*)dk; p.dv = (elem*)dv;
   p.chunk_fid = chunk_fid;
-  p.t.seg_off = seg_off; p.t.tile_off = tile_off; p.t.seg_dest = seg_dest; p.t.fchunk_tok = fchunk_tok;
-  p.t.chunk_tok = chunk_tok; p.t.self_tile_prefix = self_tile_prefix;
-  p.t.S = (int)S; p.t.H = H; p.t.K1 = K + 1; p.t.F = (K > 0) ? F : 0; p.t.N = N; p.t.B = B;
-  p.t.hist_bound = (K > 0) ? (int)hist_bound : 0;
-  p.t.self_total = (int)(self_tiles * H);
+  p.t = t;
   p.scale = (float)(1.0 / sqrt((double)D));
   p.scale_log2 = (float)(1.4426950408889634 / sqrt((double)D));
   // division by H*K1 as a multiplication: with s = 31 + ceil(log2 d) and m = floor(2^s / d) + 1 the
@@ -605,22 +596,56 @@ extern "C" int moba_bwd(const void* dout, const void* q, const void* k, const vo
   p.hk_shift = 31 + lg;
   p.hk_magic = (uint32_t)((1ull << p.hk_shift) / hk + 1);
 
-  hipStream_t st = (hipStream_t)stream;
-  static bool attr_set = false;
+  static bool attr_set = false;  // one flag per element type
   if (!attr_set) {
-    if (hipFuncSetAttribute((const void*)bwd_dq_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdDqLds) !=
+    if (hipFuncSetAttribute((const void*)bwd_dq_kernel<E>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdDqLds) !=
             hipSuccess ||
-        hipFuncSetAttribute((const void*)bwd_dkv_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdDkvLds) !=
+        hipFuncSetAttribute((const void*)bwd_dkv_kernel<E>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdDkvLds) !=
             hipSuccess)
       return MOBA_ERR_LAUNCH;
     attr_set = true;
   }
   const int64_t rows = S * H;
-  hipLaunchKernelGGL(bwd_delta_kernel, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st, (const bf16*)dout,
-                     (const bf16*)out, lse, delta, delta + S * H, rows);
-  hipLaunchKernelGGL(bwd_dq_kernel, dim3((unsigned)grid_q), dim3(256), kBwdDqLds, st, p);
-  hipLaunchKernelGGL(bwd_dq_reduce_kernel, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st,
-                     (const float*)part_dq, sel, (bf16*)dq, rows, K + 1, p.scale);
-  hipLaunchKernelGGL(bwd_dkv_kernel, dim3((unsigned)grid_kv), dim3(256), kBwdDkvLds, st, p);
+  hipLaunchKernelGGL(bwd_delta_kernel<E>, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st, (const elem*)dout,
+                     (const elem*)out, lse, delta, delta + S * H, rows);
+  hipLaunchKernelGGL(bwd_dq_kernel<E>, dim3((unsigned)grid_q), dim3(256), kBwdDqLds, st, p);
+  hipLaunchKernelGGL(bwd_dq_reduce_kernel<E>, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st,
+                     (const float*)part_dq, sel, (elem*)dq, rows, K + 1, p.scale);
+  hipLaunchKernelGGL(bwd_dkv_kernel<E>, dim3((unsigned)grid_kv), dim3(256), kBwdDkvLds, st, p);
   return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
+}
+
+extern "C" int moba_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out,
+                        const float* lse, const int32_t* sel, const int32_t* seg_off, const int32_t* tile_off,
+                        const int32_t* seg_dest, const int32_t* fchunk_tok, const int32_t* chunk_tok,
+                        const int32_t* self_tile_prefix, const int32_t* chunk_fid, float* delta, float* part_dq,
+                        void* dq, void* dk, void* dv, int64_t S, int H, int D, int K, int F, int N, int B,
+                        int64_t hist_bound, int64_t self_tiles, int dtype, void* stream) {
+  if (!dout || !q || !k || !v || !out || !lse || !chunk_tok || !self_tile_prefix || !delta || !part_dq || !dq ||
+      !dk || !dv)
+    return MOBA_ERR_ARG;
+  if (K > 0 && (!sel || !seg_off || !tile_off || !seg_dest || !fchunk_tok || !chunk_fid)) return MOBA_ERR_ARG;
+  if (D != kHeadDim || (dtype != MOBA_DTYPE_BF16 && dtype != MOBA_DTYPE_F16)) return MOBA_ERR_UNSUPPORTED;
+  if (S <= 0 || H <= 0 || K < 0 || F < 0 || N <= 0 || B <= 0 || hist_bound < 0 || self_tiles <= 0) return MOBA_ERR_ARG;
+  const void* ptrs[] = {dout, q, k, v, out, part_dq, dq, dk, dv};
+  for (const void* x : ptrs)
+    if ((uintptr_t)x & 15) return MOBA_ERR_ARG;
+  if ((int64_t)S * H * (K + 1) >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
+  const int64_t per = 8 * kXcdBlock;
+  const int64_t total_q = (K > 0 ? hist_bound : 0) + self_tiles * H;
+  const int64_t grid_q = (total_q + per - 1) / per * per;
+  const int64_t grid_kv = (self_tiles * H + per - 1) / per * per;
+  if (grid_q >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
+  TileTables t;
+  t.seg_off = seg_off; t.tile_off = tile_off; t.seg_dest = seg_dest; t.fchunk_tok = fchunk_tok;
+  t.chunk_tok = chunk_tok; t.self_tile_prefix = self_tile_prefix;
+  t.S = (int)S; t.H = H; t.K1 = K + 1; t.F = (K > 0) ? F : 0; t.N = N; t.B = B;
+  t.hist_bound = (K > 0) ? (int)hist_bound : 0;
+  t.self_total = (int)(self_tiles * H);
+  hipStream_t st = (hipStream_t)stream;
+  return dtype == MOBA_DTYPE_F16
+             ? launch_bwd<F16>(dout, q, k, v, out, lse, sel, chunk_fid, delta, part_dq, dq, dk, dv, t, S, H, D, K,
+                               grid_q, grid_kv, st)
+             : launch_bwd<Bf16>(dout, q, k, v, out, lse, sel, chunk_fid, delta, part_dq, dq, dk, dv, t, S, H, D, K,
+                                grid_q, grid_kv, st);
 }

@@ -1,10 +1,11 @@
-// Key chunk-mean: kbar[f, h, :] = bf16( mean over the B tokens of filtered chunk f of K[., h, :] ).
+// Key chunk-mean: kbar[f, h, :] = round( mean over the B tokens of filtered chunk f of K[., h, :] ),
+// rounded once to the element type (bf16 or fp16).
 //
 // HBM-bound: K is read exactly once with 16-byte loads (a wave covers 1 KiB of
 // one token row); the algorithmic traffic is S*H*D*2 bytes.  Accumulation is
-// in fp64: the sum of a chunk of bf16 values is then exact, so the result
+// in fp64: the sum of a chunk of 16-bit float values is then exact, so the result
 // does not depend on how the chunk is split over workgroups, and the rounded
-// mean is reproducible bit for bit (fp64 -> fp32 -> bf16, round to nearest even).
+// mean is reproducible bit for bit (fp64 -> fp32 -> element type, round to nearest even).
 //
 // Stage 1: grid (column blocks, token splits, F); each thread owns 8 adjacent
 //          columns of the [H*D] token row and sums its token split.
@@ -13,9 +14,11 @@
 
 namespace moba {
 
+template <class E>
 __global__ __launch_bounds__(256) void chunk_mean_partial_kernel(
-    const bf16* __restrict__ k, const int* __restrict__ fchunk_tok, double* __restrict__ partial,
+    const typename E::elem* __restrict__ k, const int* __restrict__ fchunk_tok, double* __restrict__ partial,
     int HD8 /* H*D/8 */, int B, int nsplit, int tok_per_split) {
+  MOBA_ELEM_TYPES(E)
   const int col = blockIdx.x * 256 + threadIdx.x;
   if (col >= HD8) return;
   const int split = blockIdx.y;
@@ -23,26 +26,26 @@ __global__ __launch_bounds__(256) void chunk_mean_partial_kernel(
   const int t0 = split * tok_per_split;
   const int t1 = min(B, t0 + tok_per_split);
   const int64_t row_stride = (int64_t)HD8 * 8;
-  const bf16* src = k + ((int64_t)fchunk_tok[f] + t0) * row_stride + (int64_t)col * 8;
+  const elem* src = k + ((int64_t)fchunk_tok[f] + t0) * row_stride + (int64_t)col * 8;
   double acc[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.0;
   int t = t0;
   for (; t + 8 <= t1; t += 8) {
-    bf16x8 x[8];
+    elem8 x[8];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) x[u] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(src + u * row_stride));
+    for (int u = 0; u < 8; ++u) x[u] = __builtin_nontemporal_load(reinterpret_cast<const elem8*>(src + u * row_stride));
     src += 8 * row_stride;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      // sums of bf16 values are exact in fp64 whatever the order
+      // sums of 16-bit float values are exact in fp64 whatever the order
       const double a = ((double)(float)x[0][e] + (double)(float)x[1][e]) + ((double)(float)x[2][e] + (double)(float)x[3][e]);
       const double b = ((double)(float)x[4][e] + (double)(float)x[5][e]) + ((double)(float)x[6][e] + (double)(float)x[7][e]);
       acc[e] += a + b;
     }
   }
   for (; t < t1; ++t) {
-    bf16x8 x0 = *reinterpret_cast<const bf16x8*>(src);
+    elem8 x0 = *reinterpret_cast<const elem8*>(src);
     src += row_stride;
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[e] += (double)(float)x0[e];
@@ -52,8 +55,10 @@ __global__ __launch_bounds__(256) void chunk_mean_partial_kernel(
   for (int e = 0; e < 8; ++e) dst[e] = acc[e];
 }
 
+template <class E>
 __global__ __launch_bounds__(256) void chunk_mean_finish_kernel(
-    const double* __restrict__ partial, bf16* __restrict__ kbar, int HD8, int B, int nsplit, int F) {
+    const double* __restrict__ partial, typename E::elem* __restrict__ kbar, int HD8, int B, int nsplit, int F) {
+  MOBA_ELEM_TYPES(E)
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;  // over F * HD8
   if (idx >= (int64_t)F * HD8) return;
   const int f = (int)(idx / HD8);
@@ -66,11 +71,11 @@ __global__ __launch_bounds__(256) void chunk_mean_finish_kernel(
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[e] += src[e];
   }
-  bf16x8 o;
+  elem8 o;
   const double inv = (double)B;
 #pragma unroll
-  for (int e = 0; e < 8; ++e) o[e] = (bf16)(float)(acc[e] / inv);
-  *reinterpret_cast<bf16x8*>(kbar + idx * 8) = o;
+  for (int e = 0; e < 8; ++e) o[e] = (elem)(float)(acc[e] / inv);
+  *reinterpret_cast<elem8*>(kbar + idx * 8) = o;
 }
 
 }  // namespace moba
@@ -93,8 +98,9 @@ extern "C" size_t moba_chunk_mean_workspace_bytes(int H, int D, int F, int B) {
 }
 
 extern "C" int moba_chunk_mean(const void* k, const int32_t* fchunk_tok, void* kbar, void* workspace,
-                               int64_t S, int H, int D, int F, int B, void* stream) {
+                               int64_t S, int H, int D, int F, int B, int dtype, void* stream) {
   if (F == 0) return MOBA_OK;
+  if (dtype != MOBA_DTYPE_BF16 && dtype != MOBA_DTYPE_F16) return MOBA_ERR_UNSUPPORTED;
   if (!k || !fchunk_tok || !kbar || !workspace || S <= 0 || H <= 0 || D <= 0 || F < 0 || B <= 0) return MOBA_ERR_ARG;
   if ((H * D) % 8 != 0 || ((uintptr_t)k & 15) || ((uintptr_t)kbar & 15) || ((uintptr_t)workspace & 7)) return MOBA_ERR_ARG;
   const int HD8 = H * D / 8;
@@ -102,10 +108,18 @@ extern "C" int moba_chunk_mean(const void* k, const int32_t* fchunk_tok, void* k
   const int tps = (B + nsplit - 1) / nsplit;
   hipStream_t st = (hipStream_t)stream;
   dim3 grid((HD8 + 255) / 256, nsplit, F);
-  hipLaunchKernelGGL(chunk_mean_partial_kernel, grid, dim3(256), 0, st, (const bf16*)k, fchunk_tok,
-                     (double*)workspace, HD8, B, nsplit, tps);
   const int64_t n = (int64_t)F * HD8;
-  hipLaunchKernelGGL(chunk_mean_finish_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
-                     (const double*)workspace, (bf16*)kbar, HD8, B, nsplit, F);
+  const dim3 fgrid((unsigned)((n + 255) / 256));
+  if (dtype == MOBA_DTYPE_F16) {
+    hipLaunchKernelGGL(chunk_mean_partial_kernel<F16>, grid, dim3(256), 0, st, (const f16*)k, fchunk_tok,
+                       (double*)workspace, HD8, B, nsplit, tps);
+    hipLaunchKernelGGL(chunk_mean_finish_kernel<F16>, fgrid, dim3(256), 0, st, (const double*)workspace, (f16*)kbar,
+                       HD8, B, nsplit, F);
+  } else {
+    hipLaunchKernelGGL(chunk_mean_partial_kernel<Bf16>, grid, dim3(256), 0, st, (const bf16*)k, fchunk_tok,
+                       (double*)workspace, HD8, B, nsplit, tps);
+    hipLaunchKernelGGL(chunk_mean_finish_kernel<Bf16>, fgrid, dim3(256), 0, st, (const double*)workspace,
+                       (bf16*)kbar, HD8, B, nsplit, F);
+  }
   return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
 }

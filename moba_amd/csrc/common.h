@@ -9,10 +9,35 @@ typedef __bf16 bf16;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef _Float16 f16;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(4))) _Float16 f16x4;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+
+// Element types of q, k, v: every kernel is a template over one of these and names the
+// types elem, elem2, elem4, elem8 inside its body (MOBA_ELEM_TYPES).
+struct Bf16 {
+  typedef bf16 elem;
+  typedef bf16x2 elem2;
+  typedef bf16x4 elem4;
+  typedef bf16x8 elem8;
+};
+struct F16 {
+  typedef f16 elem;
+  typedef f16x2 elem2;
+  typedef f16x4 elem4;
+  typedef f16x8 elem8;
+};
+#define MOBA_ELEM_TYPES(E)            \
+  using elem = typename E::elem;      \
+  using elem2 = typename E::elem2;    \
+  using elem4 = typename E::elem4;    \
+  using elem8 = typename E::elem8;
+enum : int { MOBA_DTYPE_BF16 = 0, MOBA_DTYPE_F16 = 1 };
 
 constexpr int kHeadDim = 128;  // the MFMA kernels are specialised for D = 128
 constexpr int kWave = 64;
@@ -32,6 +57,9 @@ enum : int {
 __device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
 }
+__device__ __forceinline__ f32x16 mfma32(f16x8 a, f16x8 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+}
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
@@ -39,11 +67,13 @@ __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_lo
 // value held by the lane 32 positions away (the other half of the wave)
 __device__ __forceinline__ float xhalf(float x) { return __shfl_xor(x, 32, 64); }
 
-__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
-  bf16x2 p;
-  p[0] = (bf16)lo;
-  p[1] = (bf16)hi;
-  return *reinterpret_cast<uint32_t*>(&p);
+// two floats rounded (to nearest even) to the element type, packed into 32 bits
+template <class E>
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+  typename E::elem2 p;
+  p[0] = (typename E::elem)lo;
+  p[1] = (typename E::elem)hi;
+  return __builtin_bit_cast(uint32_t, p);
 }
 
 // largest i in [0, n) with a[i] <= x, for ascending a with a[0] <= x

@@ -22,11 +22,12 @@ namespace moba {
 
 constexpr int kFwdLds = 4 * kTileBytes;  // K[2], V[2]
 
+template <class E>
 struct FwdParams {
-  const bf16* q;
-  const bf16* k;
-  const bf16* v;
-  bf16* part_o;     // [S*H*K1, D]
+  const typename E::elem* q;
+  const typename E::elem* k;
+  const typename E::elem* v;
+  typename E::elem* part_o;  // [S*H*K1, D]
   float* part_lse;  // [S*H*K1], log2 domain
   TileTables t;
   float scale_log2;  // D^-0.5 * log2(e)
@@ -40,7 +41,9 @@ constexpr float kRescaleThreshold = 8.f;  // log2 units: the running max may lag
 // so the vector work of one block executes under the MFMAs of its neighbours, and the
 // fragment reads from LDS run a few MFMAs ahead.  K and V tiles (64 keys) are double
 // buffered separately: K(t+1) must be resident half a tile before V(t+1).
-__global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams p) {
+template <class E>
+__global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) {
+  MOBA_ELEM_TYPES(E)
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int n = lane & 31, hh = lane >> 5;
@@ -53,11 +56,11 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams p) {
   const bool row_valid = r < t.row_count;
 
   // ---- Q^T operand: lane (n, hh) holds q[tok][16*ks + 8*hh .. +7] ----
-  bf16x8 bq[8];
+  elem8 bq[8];
   {
-    const bf16* src = p.q + ((int64_t)t.tok * H + h) * kHeadDim + 8 * hh;
+    const elem* src = p.q + ((int64_t)t.tok * H + h) * kHeadDim + 8 * hh;
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) bq[ks] = *reinterpret_cast<const bf16x8*>(src + 16 * ks);
+    for (int ks = 0; ks < 8; ++ks) bq[ks] = *reinterpret_cast<const elem8*>(src + 16 * ks);
   }
 
   // ---- K/V tile loader: global -> LDS without passing through registers.
@@ -140,12 +143,12 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams p) {
     }
   }
   auto k_frag = [&](int tile_off, int kb, int s8) __attribute__((always_inline)) {
-    return *reinterpret_cast<const bf16x8*>(smem + koff[s8] + (tile_off + kb * 8192));
+    return *reinterpret_cast<const elem8*>(smem + koff[s8] + (tile_off + kb * 8192));
   };
   auto v_frag = [&](int tile_off, int kb, int j2, int db) __attribute__((always_inline)) {
-    const bf16x4 va = lds_read_tr(smem + voffA[db] + (tile_off + (32 * kb + 16 * j2) * 256));
-    const bf16x4 vb = lds_read_tr(smem + voffB[db] + (tile_off + (32 * kb + 16 * j2) * 256));
-    bf16x8 a;
+    const elem4 va = lds_read_tr<elem4>(smem + voffA[db] + (tile_off + (32 * kb + 16 * j2) * 256));
+    const elem4 vb = lds_read_tr<elem4>(smem + voffB[db] + (tile_off + (32 * kb + 16 * j2) * 256));
+    elem8 a;
     a[0] = va[0]; a[1] = va[1]; a[2] = va[2]; a[3] = va[3];
     a[4] = vb[0]; a[5] = vb[1]; a[6] = vb[2]; a[7] = vb[3];
     return a;
@@ -184,7 +187,7 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams p) {
   __syncthreads();
 
   f32x16 s0, s1;   // S^T, then P^T, of the current and the next key block
-  bf16x8 pb[2];    // P^T operand of the current block: elements 0..7 and 8..15
+  elem8 pb[2];    // P^T operand of the current block: elements 0..7 and 8..15
   {
 #pragma unroll
     for (int e = 0; e < 16; ++e) s0[e] = 0.f;
@@ -199,7 +202,7 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams p) {
     for (int e = 0; e < 8; ++e) {
       const float pe = fast_exp2(s0[e] * sl2 - m_run);
       l_run += pe;
-      pb[0][e] = (bf16)pe;
+      pb[0][e] = (elem)pe;
     }
   }
 
@@ -211,8 +214,8 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams p) {
                   int kb) __attribute__((always_inline)) {
     constexpr bool has_next = decltype(has_next_c)::value;
     // ---- phase 1: S^T of the next block under exponentials 8..15 of this block ----
-    bf16x8 ka[8];
-    bf16x8 va[8];
+    elem8 ka[8];
+    elem8 va[8];
     float pf[8];
     float rs = 0.f;
     if constexpr (has_next) {
@@ -241,7 +244,7 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams p) {
     }
     l_run += rs;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) pb[1][e] = (bf16)pf[e];
+    for (int e = 0; e < 8; ++e) pb[1][e] = (elem)pf[e];
 
     // ---- phase 2: O^T += V^T P^T of this block under the row max and exponentials 0..7 of the next ----
     if constexpr (has_next) {
@@ -287,7 +290,7 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams p) {
       }
       l_run = l_run * alpha + rn;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) pb[0][e] = (bf16)pg[e];
+      for (int e = 0; e < 8; ++e) pb[0][e] = (elem)pg[e];
     }
   };
 
@@ -338,14 +341,14 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams p) {
   const float l_tot = sum_xhalf(l_run);
   const float inv = 1.f / l_tot;
   if (row_valid) {
-    bf16* dst = p.part_o + (int64_t)t.dest * kHeadDim;
+    elem* dst = p.part_o + (int64_t)t.dest * kHeadDim;
 #pragma unroll
     for (int db = 0; db < 4; ++db)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         u32x2 w;
-        w[0] = pack_bf16(oacc[db][4 * g + 0] * inv, oacc[db][4 * g + 1] * inv);
-        w[1] = pack_bf16(oacc[db][4 * g + 2] * inv, oacc[db][4 * g + 3] * inv);
+        w[0] = pack2<E>(oacc[db][4 * g + 0] * inv, oacc[db][4 * g + 1] * inv);
+        w[1] = pack2<E>(oacc[db][4 * g + 2] * inv, oacc[db][4 * g + 3] * inv);
         *reinterpret_cast<u32x2*>(dst + 32 * db + 8 * g + 4 * hh) = w;
       }
     if (hh == 0) p.part_lse[t.dest] = m_run + fast_log2(l_tot);
@@ -354,10 +357,12 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams p) {
 
 // Combine the K1 slots of each (token, head): slot 0 is the self part, slot 1+j the
 // j-th selected history chunk (present iff sel[row, j] >= 0).  16 lanes per row.
-__global__ __launch_bounds__(256) void moba_merge_kernel(const bf16* __restrict__ part_o,
+template <class E>
+__global__ __launch_bounds__(256) void moba_merge_kernel(const typename E::elem* __restrict__ part_o,
                                                          const float* __restrict__ part_lse,
-                                                         const int* __restrict__ sel, bf16* __restrict__ out,
+                                                         const int* __restrict__ sel, typename E::elem* __restrict__ out,
                                                          float* __restrict__ lse, int64_t rows, int K1) {
+  MOBA_ELEM_TYPES(E)
   const int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
   if (row >= rows) return;
   const int c8 = threadIdx.x & 15;
@@ -375,16 +380,16 @@ __global__ __launch_bounds__(256) void moba_merge_kernel(const bf16* __restrict_
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.f;
   float wsum = 0.f;
-  const bf16* po = part_o + row * K1 * kHeadDim + c8 * 8;
+  const elem* po = part_o + row * K1 * kHeadDim + c8 * 8;
   for (int j0 = 0; j0 < K1; j0 += 4) {
-    bf16x8 x[4];
+    elem8 x[4];
     float w[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int j = j0 + u;
       const bool ok = j < K1 && (j == 0 || ps[j < K1 ? j - 1 : 0] >= 0);
       const int jj = ok ? j : 0;
-      x[u] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(po + (int64_t)jj * kHeadDim));
+      x[u] = __builtin_nontemporal_load(reinterpret_cast<const elem8*>(po + (int64_t)jj * kHeadDim));
       w[u] = ok ? fast_exp2(pl[jj] - mx) : 0.f;
     }
 #pragma unroll
@@ -395,10 +400,10 @@ __global__ __launch_bounds__(256) void moba_merge_kernel(const bf16* __restrict_
     }
   }
   const float inv = 1.f / wsum;
-  bf16x8 o;
+  elem8 o;
 #pragma unroll
-  for (int e = 0; e < 8; ++e) o[e] = (bf16)(acc[e] * inv);
-  __builtin_nontemporal_store(o, reinterpret_cast<bf16x8*>(out + row * kHeadDim + c8 * 8));
+  for (int e = 0; e < 8; ++e) o[e] = (elem)(acc[e] * inv);
+  __builtin_nontemporal_store(o, reinterpret_cast<elem8*>(out + row * kHeadDim + c8 * 8));
   if (c8 == 0) lse[row] = (mx + fast_log2(wsum)) * 0.6931471805599453f;
 }
 
@@ -408,50 +413,64 @@ using namespace moba;
 
 extern "C" int moba_fwd_tile_rows(void) { return TM; }
 
+template <class E>
+static int launch_partials(const void* q, const void* k, const void* v, void* part_o, float* part_lse,
+                           const TileTables& t, int D, int64_t grid, hipStream_t st) {
+  FwdParams<E> p;
+  p.q = (const typename E::elem*)q; p.k = (const typename E::elem*)k; p.v = (const typename E::elem*)v;
+  p.part_o = (typename E::elem*)part_o; p.part_lse = part_lse;
+  p.t = t;
+  p.scale_log2 = (float)(1.4426950408889634 / sqrt((double)D));
+  static bool attr_set = false;  // one flag per element type
+  if (!attr_set) {
+    if (hipFuncSetAttribute((const void*)moba_fwd_kernel<E>, hipFuncAttributeMaxDynamicSharedMemorySize, kFwdLds) !=
+        hipSuccess)
+      return MOBA_ERR_LAUNCH;
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(moba_fwd_kernel<E>, dim3((unsigned)grid), dim3(256), kFwdLds, st, p);
+  return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
+}
+
 // hist_bound: any upper bound on the number of history tiles (floor(M/128) + F*H is one).
 extern "C" int moba_fwd_partials(const void* q, const void* k, const void* v, void* part_o, float* part_lse,
                                  const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest,
                                  const int32_t* fchunk_tok, const int32_t* chunk_tok,
                                  const int32_t* self_tile_prefix, int64_t S, int H, int D, int K, int F, int N, int B,
-                                 int64_t hist_bound, int64_t self_tiles, void* stream) {
+                                 int64_t hist_bound, int64_t self_tiles, int dtype, void* stream) {
   if (!q || !k || !v || !part_o || !part_lse || !chunk_tok || !self_tile_prefix) return MOBA_ERR_ARG;
   if (K > 0 && (!seg_off || !tile_off || !seg_dest || !fchunk_tok)) return MOBA_ERR_ARG;
-  if (D != kHeadDim) return MOBA_ERR_UNSUPPORTED;
+  if (D != kHeadDim || (dtype != MOBA_DTYPE_BF16 && dtype != MOBA_DTYPE_F16)) return MOBA_ERR_UNSUPPORTED;
   if (S <= 0 || H <= 0 || K < 0 || F < 0 || N <= 0 || B <= 0 || hist_bound < 0 || self_tiles <= 0) return MOBA_ERR_ARG;
   if (((uintptr_t)q & 15) || ((uintptr_t)k & 15) || ((uintptr_t)v & 15) || ((uintptr_t)part_o & 15)) return MOBA_ERR_ARG;
   if ((int64_t)S * H * (K + 1) >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
   const int64_t total = (K > 0 ? hist_bound : 0) + self_tiles * H;
   const int64_t grid = (total + 8 * kXcdBlock - 1) / (8 * kXcdBlock) * (8 * kXcdBlock);
   if (grid >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
-  FwdParams p;
-  p.q = (const bf16*)q; p.k = (const bf16*)k; p.v = (const bf16*)v;
-  p.part_o = (bf16*)part_o; p.part_lse = part_lse;
-  p.t.seg_off = seg_off; p.t.tile_off = tile_off; p.t.seg_dest = seg_dest; p.t.fchunk_tok = fchunk_tok;
-  p.t.chunk_tok = chunk_tok; p.t.self_tile_prefix = self_tile_prefix;
-  p.t.S = (int)S; p.t.H = H; p.t.K1 = K + 1; p.t.F = (K > 0) ? F : 0; p.t.N = N; p.t.B = B;
-  p.t.hist_bound = (K > 0) ? (int)hist_bound : 0;
-  p.t.self_total = (int)(self_tiles * H);
-  p.scale_log2 = (float)(1.4426950408889634 / sqrt((double)D));
+  TileTables t;
+  t.seg_off = seg_off; t.tile_off = tile_off; t.seg_dest = seg_dest; t.fchunk_tok = fchunk_tok;
+  t.chunk_tok = chunk_tok; t.self_tile_prefix = self_tile_prefix;
+  t.S = (int)S; t.H = H; t.K1 = K + 1; t.F = (K > 0) ? F : 0; t.N = N; t.B = B;
+  t.hist_bound = (K > 0) ? (int)hist_bound : 0;
+  t.self_total = (int)(self_tiles * H);
   hipStream_t st = (hipStream_t)stream;
-  static bool attr_set = false;
-  if (!attr_set) {
-    if (hipFuncSetAttribute((const void*)moba_fwd_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kFwdLds) !=
-        hipSuccess)
-      return MOBA_ERR_LAUNCH;
-    attr_set = true;
-  }
-  hipLaunchKernelGGL(moba_fwd_kernel, dim3((unsigned)grid), dim3(256), kFwdLds, st, p);
-  return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
+  return dtype == MOBA_DTYPE_F16 ? launch_partials<F16>(q, k, v, part_o, part_lse, t, D, grid, st)
+                                 : launch_partials<Bf16>(q, k, v, part_o, part_lse, t, D, grid, st);
 }
 
 extern "C" int moba_fwd_merge(const void* part_o, const float* part_lse, const int32_t* sel, void* out, float* lse,
-                              int64_t S, int H, int D, int K, void* stream) {
+                              int64_t S, int H, int D, int K, int dtype, void* stream) {
   if (!part_o || !part_lse || !out || !lse || (K > 0 && !sel)) return MOBA_ERR_ARG;
-  if (D != kHeadDim) return MOBA_ERR_UNSUPPORTED;
+  if (D != kHeadDim || (dtype != MOBA_DTYPE_BF16 && dtype != MOBA_DTYPE_F16)) return MOBA_ERR_UNSUPPORTED;
   if (S <= 0 || H <= 0 || K < 0 || ((uintptr_t)part_o & 15) || ((uintptr_t)out & 15)) return MOBA_ERR_ARG;
   const int64_t rows = S * H;
-  hipLaunchKernelGGL(moba_merge_kernel, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, (hipStream_t)stream,
-                     (const bf16*)part_o, part_lse, sel, (bf16*)out, lse, rows, K + 1);
+  const dim3 grid((unsigned)((rows + 15) / 16));
+  if (dtype == MOBA_DTYPE_F16)
+    hipLaunchKernelGGL(moba_merge_kernel<F16>, grid, dim3(256), 0, (hipStream_t)stream, (const f16*)part_o, part_lse,
+                       sel, (f16*)out, lse, rows, K + 1);
+  else
+    hipLaunchKernelGGL(moba_merge_kernel<Bf16>, grid, dim3(256), 0, (hipStream_t)stream, (const bf16*)part_o,
+                       part_lse, sel, (bf16*)out, lse, rows, K + 1);
   return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
 }
 
@@ -460,9 +479,9 @@ extern "C" int moba_fwd(const void* q, const void* k, const void* v, void* part_
                         const int32_t* sel, const int32_t* seg_off, const int32_t* tile_off,
                         const int32_t* seg_dest, const int32_t* fchunk_tok, const int32_t* chunk_tok,
                         const int32_t* self_tile_prefix, void* out, float* lse, int64_t S, int H, int D, int K,
-                        int F, int N, int B, int64_t hist_bound, int64_t self_tiles, void* stream) {
+                        int F, int N, int B, int64_t hist_bound, int64_t self_tiles, int dtype, void* stream) {
   int rc = moba_fwd_partials(q, k, v, part_o, part_lse, seg_off, tile_off, seg_dest, fchunk_tok, chunk_tok,
-                             self_tile_prefix, S, H, D, K, F, N, B, hist_bound, self_tiles, stream);
+                             self_tile_prefix, S, H, D, K, F, N, B, hist_bound, self_tiles, dtype, stream);
   if (rc != MOBA_OK) return rc;
-  return moba_fwd_merge(part_o, part_lse, sel, out, lse, S, H, D, K, stream);
+  return moba_fwd_merge(part_o, part_lse, sel, out, lse, S, H, D, K, dtype, stream);
 }

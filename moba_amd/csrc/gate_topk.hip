@@ -51,11 +51,12 @@ __device__ __forceinline__ int find_seq(const int* __restrict__ cu, int nseq, in
   return upper_row(cu, nseq, s);
 }
 
-template <int KMAX>
+template <class E, int KMAX>
 __global__ __launch_bounds__(256) void gate_topk_kernel(
-    const bf16* __restrict__ q, const bf16* __restrict__ kbar, const int* __restrict__ cu_seqlens,
+    const typename E::elem* __restrict__ q, const typename E::elem* __restrict__ kbar, const int* __restrict__ cu_seqlens,
     const int* __restrict__ seq_fbase, int* __restrict__ sel, float* __restrict__ scores_out,
     int S, int H, int nseq, int F, int B, int K) {
+  MOBA_ELEM_TYPES(E)
   __shared__ float sc[4][64][33];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int n = lane & 31, hh = lane >> 5;
@@ -86,21 +87,21 @@ __global__ __launch_bounds__(256) void gate_topk_kernel(
 
   if (fhi > 0) {  // wave-uniform (and block-uniform)
     // Q^T operand: lane (n, hh) holds q[token n (+32)][16*ks + 8*hh .. +7]
-    bf16x8 bq[2][8];
+    elem8 bq[2][8];
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) {
       const int tok = min(tok0 + 32 * qb + n, S - 1);
-      const bf16* src = q + ((int64_t)tok * H + hc) * kHeadDim + 8 * hh;
+      const elem* src = q + ((int64_t)tok * H + hc) * kHeadDim + 8 * hh;
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks) bq[qb][ks] = *reinterpret_cast<const bf16x8*>(src + 16 * ks);
+      for (int ks = 0; ks < 8; ++ks) bq[qb][ks] = *reinterpret_cast<const elem8*>(src + 16 * ks);
     }
     for (int f0 = flo; f0 < fhi; f0 += 32) {
       const int fr = min(f0 + n, F - 1);
-      const bf16* src = kbar + ((int64_t)fr * H + hc) * kHeadDim + 8 * hh;
+      const elem* src = kbar + ((int64_t)fr * H + hc) * kHeadDim + 8 * hh;
       f32x16 acc0 = {0}, acc1 = {0};
 #pragma unroll
       for (int ks = 0; ks < 8; ++ks) {
-        const bf16x8 a = *reinterpret_cast<const bf16x8*>(src + 16 * ks);
+        const elem8 a = *reinterpret_cast<const elem8*>(src + 16 * ks);
         acc0 = mfma32(a, bq[0][ks], acc0);
         acc1 = mfma32(a, bq[1][ks], acc1);
       }
@@ -165,16 +166,21 @@ using namespace moba;
 
 extern "C" int moba_gate_topk(const void* q, const void* kbar, const int32_t* cu_seqlens, const int32_t* seq_fbase,
                               int32_t* sel, float* scores_out, int64_t S, int H, int D, int nseq, int F, int B,
-                              int K, void* stream) {
+                              int K, int dtype, void* stream) {
   if (!q || !kbar || !cu_seqlens || !seq_fbase || !sel) return MOBA_ERR_ARG;
+  if (dtype != MOBA_DTYPE_BF16 && dtype != MOBA_DTYPE_F16) return MOBA_ERR_UNSUPPORTED;
   if (S <= 0 || S > 0x7fffffff - 64 || H <= 0 || nseq <= 0 || F <= 0 || B <= 0 || K <= 0) return MOBA_ERR_ARG;
   if (D != kHeadDim) return MOBA_ERR_UNSUPPORTED;
   if (((uintptr_t)q & 15) || ((uintptr_t)kbar & 15)) return MOBA_ERR_ARG;
   dim3 grid((unsigned)((S + 63) / 64), (unsigned)((H + 3) / 4));
   hipStream_t st = (hipStream_t)stream;
-#define CALL(KM)                                                                                              \
-  hipLaunchKernelGGL(gate_topk_kernel<KM>, grid, dim3(256), 0, st, (const bf16*)q, (const bf16*)kbar, cu_seqlens, \
-                     seq_fbase, sel, scores_out, (int)S, H, nseq, F, B, K)
+#define CALL(KM)                                                                                               \
+  if (dtype == MOBA_DTYPE_F16)                                                                                 \
+    hipLaunchKernelGGL((gate_topk_kernel<F16, KM>), grid, dim3(256), 0, st, (const f16*)q, (const f16*)kbar,   \
+                       cu_seqlens, seq_fbase, sel, scores_out, (int)S, H, nseq, F, B, K);                      \
+  else                                                                                                         \
+    hipLaunchKernelGGL((gate_topk_kernel<Bf16, KM>), grid, dim3(256), 0, st, (const bf16*)q, (const bf16*)kbar, \
+                       cu_seqlens, seq_fbase, sel, scores_out, (int)S, H, nseq, F, B, K)
   MOBA_DISPATCH_K(K, CALL)
 #undef CALL
   return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;

@@ -32,11 +32,19 @@ def _stream(device) -> ctypes.c_void_p:
     return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 
+def _dtype_code(t: torch.Tensor) -> int:
+    if t.dtype == torch.bfloat16:
+        return _lib.DTYPE_BF16
+    if t.dtype == torch.float16:
+        return _lib.DTYPE_F16
+    raise TypeError("moba_attn_varlen supports bfloat16 and float16 q, k, v")
+
+
 def _check_qkv(q, k, v):
     if not (q.is_cuda and k.is_cuda and v.is_cuda):
         raise RuntimeError("moba_attn_varlen needs tensors on an AMD GPU (there is no CPU path)")
-    if q.dtype != torch.bfloat16 or k.dtype != q.dtype or v.dtype != q.dtype:
-        raise TypeError("moba_attn_varlen supports bfloat16 q, k, v")
+    if q.dtype not in (torch.bfloat16, torch.float16) or k.dtype != q.dtype or v.dtype != q.dtype:
+        raise TypeError("moba_attn_varlen supports bfloat16 and float16 q, k, v (all three of the same dtype)")
     if q.dim() != 3 or q.shape != k.shape or q.shape != v.shape:
         raise ValueError("q, k, v must all be [seqlen, heads, head_dim] with the same number of heads")
     if q.shape[2] != HEAD_DIM:
@@ -45,14 +53,14 @@ def _check_qkv(q, k, v):
 
 # ----------------------------------------------------------------------------- stages
 def chunk_mean(k: torch.Tensor, plan: MobaPlan) -> torch.Tensor:
-    """kbar [F, H, D] bf16: mean of K over every filtered chunk (exact sum, rounded once)."""
+    """kbar [F, H, D] in k's dtype: mean of K over every filtered chunk (exact sum, rounded once)."""
     lib = _lib.load()
     S, H, D = k.shape
     kbar = torch.empty((plan.F, H, D), dtype=k.dtype, device=k.device)
     nbytes = lib.moba_chunk_mean_workspace_bytes(H, D, plan.F, plan.chunk_size)
     ws = torch.empty(nbytes // 8, dtype=torch.float64, device=k.device)
     _lib.check(lib.moba_chunk_mean(_ptr(k), _ptr(plan.tables["fchunk_tok"]), _ptr(kbar), _ptr(ws), S, H, D, plan.F,
-                                   plan.chunk_size, _stream(k.device)), "moba_chunk_mean")
+                                   plan.chunk_size, _dtype_code(k), _stream(k.device)), "moba_chunk_mean")
     return kbar
 
 
@@ -66,7 +74,7 @@ def gate_topk(q: torch.Tensor, kbar: torch.Tensor, plan: MobaPlan, return_scores
         scores = torch.full((S, H, plan.F), float("-inf"), dtype=torch.float32, device=q.device)
     _lib.check(lib.moba_gate_topk(_ptr(q), _ptr(kbar), _ptr(plan.tables["cu_seqlens"]), _ptr(plan.tables["seq_fbase"]),
                                   _ptr(sel), _ptr(scores), S, H, D, plan.nseq, plan.F, plan.chunk_size, plan.K,
-                                  _stream(q.device)), "moba_gate_topk")
+                                  _dtype_code(q), _stream(q.device)), "moba_gate_topk")
     return (sel, scores) if return_scores else sel
 
 
@@ -160,11 +168,11 @@ def _forward(q, k, v, plan: MobaPlan, timer: Optional[StageTimer] = None):
         _lib.check(lib.moba_fwd_partials(_ptr(q), _ptr(k), _ptr(v), _ptr(part_o), _ptr(part_lse), _ptr(seg_off),
                                          _ptr(tile_off), _ptr(seg_dest), _ptr(t.get("fchunk_tok")),
                                          _ptr(t["chunk_tok"]), _ptr(t["self_tile_prefix"]), S, H, D, K, plan.F, plan.N,
-                                         plan.chunk_size, plan.hist_tile_bound(H), plan.self_tiles, _stream(dev)),
-                   "moba_fwd_partials")
+                                         plan.chunk_size, plan.hist_tile_bound(H), plan.self_tiles, _dtype_code(q),
+                                         _stream(dev)), "moba_fwd_partials")
     with span("fwd_merge"):
         _lib.check(lib.moba_fwd_merge(_ptr(part_o), _ptr(part_lse), _ptr(sel), _ptr(out), _ptr(lse), S, H, D, K,
-                                      _stream(dev)), "moba_fwd_merge")
+                                      _dtype_code(q), _stream(dev)), "moba_fwd_merge")
     return out, lse, sel, seg_off, tile_off, seg_dest
 
 
@@ -184,7 +192,7 @@ def _backward(dout, q, k, v, out, lse, sel, seg_off, tile_off, seg_dest, plan: M
                             _ptr(t["self_tile_prefix"]), _ptr(t.get("chunk_fid")),
                             _ptr(delta), _ptr(part_dq), _ptr(dq), _ptr(dk), _ptr(dv),
                             S, H, D, K, plan.F, plan.N, plan.chunk_size, plan.hist_tile_bound(H), plan.self_tiles,
-                            _stream(dev)), "moba_bwd")
+                            _dtype_code(q), _stream(dev)), "moba_bwd")
     return dq, dk, dv
 
 
@@ -220,7 +228,7 @@ def moba_attn_varlen(
     """Mixture-of-block attention over a packed batch.
 
     Args (as moba/moba_efficient.py:270-297):
-        q, k, v: [seqlen, heads, head_dim] bf16, same number of heads
+        q, k, v: [seqlen, heads, head_dim] bf16 or fp16, same number of heads
         cu_seqlens: int32 cumulative sequence lengths, starting at 0 and ending at seqlen
         max_seqlen: longest sequence (accepted for signature compatibility; sizes come from cu_seqlens)
         moba_chunk_size, moba_topk: block size and number of attended blocks (the current one included)

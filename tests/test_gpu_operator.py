@@ -19,11 +19,11 @@ MAX_ABS, MEAN_ABS = 2e-2, 2e-3
 REF_MAX_ABS, REF_MEAN_ABS = 4e-2, 4e-4
 
 
-def run_case(batch, seqlen, heads, B, topk, seed=0, check_grad=True):
+def run_case(batch, seqlen, heads, B, topk, seed=0, check_grad=True, dtype=torch.bfloat16):
     from moba_amd import moba_efficient as E
     from moba_amd.plan import make_plan
 
-    q, k, v, do, cu, mx = make_case(batch, seqlen, heads, seed=seed)
+    q, k, v, do, cu, mx = make_case(batch, seqlen, heads, seed=seed, dtype=dtype)
     dev = torch.device("cuda")
     cu_t = torch.tensor(cu, dtype=torch.int32, device=dev)
     qg, kg, vg = (x.to(dev).requires_grad_(True) for x in (q, k, v))
@@ -54,7 +54,7 @@ def run_case(batch, seqlen, heads, B, topk, seed=0, check_grad=True):
     err = (out.detach().cpu().float() - ref.detach()).abs()
     assert err.max() < MAX_ABS and err.mean() < MEAN_ABS, ("out", err.max().item(), err.mean().item())
     # the reference test compares two bf16 outputs (moba_naive returns o.type_as(q)): round the oracle likewise
-    err16 = (out.detach().cpu().float() - ref.detach().to(torch.bfloat16).float()).abs()
+    err16 = (out.detach().cpu().float() - ref.detach().to(dtype).float()).abs()
     assert err16.max() < REF_MAX_ABS and err16.mean() < REF_MEAN_ABS, ("out16", err16.max().item(), err16.mean().item())
     if check_grad:
         ref.backward(do.float())
@@ -92,6 +92,19 @@ def test_reference_grid(chunk):
 ])
 def test_edge_shapes(batch, seqlen, heads, B, topk):
     run_case(batch, seqlen, heads, B, topk, seed=7)
+
+
+@pytest.mark.parametrize("batch,seqlen,heads,B,topk", [
+    (1, 1024, 2, 128, 3),
+    (4, 2048, 4, 256, 4),
+    (7, 2048, 8, 128, 2),
+    (3, 1500, 3, 100, 3),
+    (1, 2048, 2, 128, 1),
+    (2, 4096, 2, 64, 12),
+])
+def test_float16(batch, seqlen, heads, B, topk):
+    """fp16 inputs (the dtype of the reference's example script), same bounds as bf16."""
+    run_case(batch, seqlen, heads, B, topk, seed=11, dtype=torch.float16)
 
 
 def test_one_token_sequences():
