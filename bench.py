@@ -44,7 +44,7 @@ WORKLOADS = {
 DEFAULT = "cfg4_L131072_h32_c4096_k12"
 
 
-def make_inputs(name, device):
+def make_inputs(name, device, gqa=False):
     lens, H, Hkv, B, topk, normalise, _ = WORKLOADS[name]
     if lens is None:
         rng = random.Random(0)
@@ -61,7 +61,7 @@ def make_inputs(name, device):
     q = draw(H)
     k = draw(Hkv)
     v = draw(Hkv)
-    if Hkv != H:  # the wrapper's repeat_kv (moba/wrapper.py:59-61), outside the timed region
+    if Hkv != H and not gqa:  # the wrapper's repeat_kv (moba/wrapper.py:59-61), outside the timed region
         k = torch.repeat_interleave(k, H // Hkv, dim=1).contiguous()
         v = torch.repeat_interleave(v, H // Hkv, dim=1).contiguous()
     cu = [0]
@@ -99,6 +99,9 @@ def main():
     ap.add_argument("--workload", default=DEFAULT, help="one of %s, or its cfgN prefix" % ", ".join(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--backward", action="store_true", help="also time forward + backward")
+    ap.add_argument("--gqa", action="store_true",
+                    help="keep the key/value heads unexpanded (grouped-query operator) instead of the reference "
+                         "wrapper's repeat_kv; not the headline configuration")
     args = ap.parse_args()
     if args.workload not in WORKLOADS:
         match = [w for w in WORKLOADS if w.split("_")[0] == args.workload]
@@ -116,19 +119,19 @@ def main():
     from moba_amd.plan import make_plan
 
     dev = torch.device("cuda:0")
-    q, k, v, cu, max_seqlen, B, topk = make_inputs(args.workload, dev)
+    q, k, v, cu, max_seqlen, B, topk = make_inputs(args.workload, dev, args.gqa)
     S, H, D = q.shape
     cu_t = torch.tensor(cu, dtype=torch.int32, device=dev)
     plan = make_plan(cu_t, B, topk)
     flops = plan.flops_per_head * D * H
 
     for _ in range(args.warmup):
-        E.moba_attn_varlen(q, k, v, cu_t, max_seqlen, B, topk)
+        E.moba_attn_varlen_with_lse(q, k, v, cu_t, max_seqlen, B, topk, gqa=args.gqa)
     torch.cuda.synchronize()
     timer = E.StageTimer()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        E.moba_attn_varlen_with_lse(q, k, v, cu_t, max_seqlen, B, topk, timer=timer)
+        E.moba_attn_varlen_with_lse(q, k, v, cu_t, max_seqlen, B, topk, timer=timer, gqa=args.gqa)
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / args.steps
     stage_ms = {name: sum(x) / len(x) for name, x in timer.ms().items()}
@@ -139,13 +142,14 @@ def main():
         g = torch.Generator(device=dev).manual_seed(1)
         do = torch.randn(q.shape, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
         qg, kg, vg = (x.clone().requires_grad_(True) for x in (q, k, v))
+        op = E.moba_attn_varlen_gqa if args.gqa else E.moba_attn_varlen
         for _ in range(max(1, args.warmup)):
-            E.moba_attn_varlen(qg, kg, vg, cu_t, max_seqlen, B, topk).backward(do)
+            op(qg, kg, vg, cu_t, max_seqlen, B, topk).backward(do)
         torch.cuda.synchronize()
         t1 = time.perf_counter()
         for _ in range(args.steps):
             qg.grad = kg.grad = vg.grad = None
-            E.moba_attn_varlen(qg, kg, vg, cu_t, max_seqlen, B, topk).backward(do)
+            op(qg, kg, vg, cu_t, max_seqlen, B, topk).backward(do)
         torch.cuda.synchronize()
         fwd_bwd_ms = (time.perf_counter() - t1) / args.steps * 1e3
         del qg, kg, vg, do
@@ -165,7 +169,7 @@ def main():
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "synthetic",
-        "config": {"workload": args.workload, "tokens": S, "heads": H, "head_dim": D, "chunk": B, "topk": topk,
+        "config": {"workload": args.workload, "tokens": S, "heads": H, "kv_heads": k.shape[1], "head_dim": D, "chunk": B, "topk": topk,
                    "sequences": len(cu) - 1, "fwd_flops": flops},
         "pct_mfma_peak_whole_op": 100.0 * flops / dt / 1e12 / MFMA_BF16_PEAK_TFLOPS,
         "stage_ms": stage_ms,
@@ -177,11 +181,13 @@ def main():
         # algorithmic backward work is 2.5x the forward's
         result["fwd_bwd"] = {"ms_per_step": fwd_bwd_ms, "tflops": 3.5 * flops / (fwd_bwd_ms * 1e-3) / 1e12}
     if "chunk_mean" in stage_ms:
-        gbs = S * H * D * 2 / (stage_ms["chunk_mean"] * 1e-3) / 1e9
+        gbs = k.numel() * 2 / (stage_ms["chunk_mean"] * 1e-3) / 1e9
         result["chunk_mean_hbm"] = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                     "frac": gbs / HBM_PEAK_GBS}
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(q, k, v, B, topk)
+        rep = H // k.shape[1]
+        result["cpu_baseline"] = cpu_baseline(q, k[:, ::1] if rep == 1 else torch.repeat_interleave(k[:, :1], 4, dim=1),
+                                              v[:, ::1] if rep == 1 else torch.repeat_interleave(v[:, :1], 4, dim=1), B, topk)
     print(json.dumps(result))
 
 

@@ -10,7 +10,9 @@
  * bf16 (dtype = MOBA_DTYPE_BF16) or fp16 (dtype = MOBA_DTYPE_F16, the dtype of the reference's
  * example, examples/llama.py:26); below, "elem" stands for that type.
  *
- * Shapes use: S packed tokens, H heads, D head_dim, B chunk size, N chunks,
+ * Shapes use: S packed tokens, H query heads, Hkv key/value heads (H is a multiple of Hkv;
+ * query head h reads key/value head h / (H/Hkv); the reference operator has H == Hkv and
+ * its wrapper repeats the key/value heads first, moba/wrapper.py:59-61), D head_dim, B chunk size, N chunks,
  * F filtered chunks (chunks that are not the last of their sequence), K selected
  * history chunks per (token, head), M = number of selected (token, head, chunk)
  * triples, P = number of (filtered chunk, later chunk of the same sequence) pairs.
@@ -32,7 +34,7 @@ const char* moba_strerror(int code);
 
 /* Key chunk-mean.  Replaces moba/moba_efficient.py:326-340 (index_select of the
  * filtered chunks, .mean(dim=1) on bf16, .float()).
- *   k          [S,H,D] elem
+ *   k          [S,H,D] elem (H here is the number of key/value heads)
  *   fchunk_tok [F] int32, first token of each filtered chunk
  *   kbar       [F,H,D] elem out (the mean rounded once to the element type)
  *   workspace  moba_chunk_mean_workspace_bytes() bytes, 8-byte aligned */
@@ -48,7 +50,8 @@ int moba_chunk_mean(const void* k, const int32_t* fchunk_tok, void* kbar, void* 
  *              score of every valid candidate (debug / test output), may be NULL
  * K <= 64. */
 int moba_gate_topk(const void* q, const void* kbar, const int32_t* cu_seqlens, const int32_t* seq_fbase, int32_t* sel,
-                   float* scores_out, int64_t S, int H, int D, int nseq, int F, int B, int K, int dtype, void* stream);
+                   float* scores_out, int64_t S, int H, int Hkv, int D, int nseq, int F, int B, int K, int dtype,
+                   void* stream);
 
 /* The selection step of moba/moba_efficient.py:365-371 alone, on caller-supplied
  * scores [S,H,F] fp32 (-inf = not a candidate).  Same routine as moba_gate_topk. */
@@ -81,26 +84,27 @@ int moba_fwd_tile_rows(void);
 int moba_fwd_partials(const void* q, const void* k, const void* v, void* part_o, float* part_lse,
                       const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest,
                       const int32_t* fchunk_tok, const int32_t* chunk_tok, const int32_t* self_tile_prefix, int64_t S,
-                      int H, int D, int K, int F, int N, int B, int64_t hist_bound, int64_t self_tiles, int dtype,
-                      void* stream);
+                      int H, int Hkv, int D, int K, int F, int N, int B, int64_t hist_bound, int64_t self_tiles,
+                      int dtype, void* stream);
 int moba_fwd_merge(const void* part_o, const float* part_lse, const int32_t* sel, void* out, float* lse, int64_t S,
                    int H, int D, int K, int dtype, void* stream);
 int moba_fwd(const void* q, const void* k, const void* v, void* part_o, float* part_lse, const int32_t* sel,
              const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest, const int32_t* fchunk_tok,
-             const int32_t* chunk_tok, const int32_t* self_tile_prefix, void* out, float* lse, int64_t S, int H, int D,
-             int K, int F, int N, int B, int64_t hist_bound, int64_t self_tiles, int dtype, void* stream);
+             const int32_t* chunk_tok, const int32_t* self_tile_prefix, void* out, float* lse, int64_t S, int H, int Hkv,
+             int D, int K, int F, int N, int B, int64_t hist_bound, int64_t self_tiles, int dtype, void* stream);
 
 /* Backward.  Replaces MixedAttention.backward, moba/moba_efficient.py:185-267, and the
  * autograd scatter of its gathered gradients.  Deterministic (no floating-point atomics).
- *   dout, q, k, v, out [S,H,D] elem; lse [S,H] fp32 from the forward
+ *   dout, q, out, dq [S,H,D] elem; k, v, dk, dv [S,Hkv,D] elem; lse [S,H] fp32 from the forward
  *   chunk_fid [N] int32: filtered id of each chunk, -1 for the last chunk of a sequence
  *   delta [2,S,H] fp32 scratch (rowsum(dO*O), then the LSE in the log2 domain); part_dq [S*H*(K+1), D] fp32 scratch
- *   dq, dk, dv [S,H,D] elem out */
+ *   dq, dk, dv: out; dk and dv of a key/value head sum over its query heads */
 int moba_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out, const float* lse,
              const int32_t* sel, const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest,
              const int32_t* fchunk_tok, const int32_t* chunk_tok, const int32_t* self_tile_prefix,
              const int32_t* chunk_fid, float* delta, float* part_dq, void* dq, void* dk, void* dv, int64_t S, int H,
-             int D, int K, int F, int N, int B, int64_t hist_bound, int64_t self_tiles, int dtype, void* stream);
+             int Hkv, int D, int K, int F, int N, int B, int64_t hist_bound, int64_t self_tiles, int dtype,
+             void* stream);
 
 #ifdef __cplusplus
 }

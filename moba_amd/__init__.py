@@ -4,10 +4,10 @@
 from functools import partial
 
 from .config import MoBAConfig
-from .moba_efficient import moba_attn_varlen
+from .moba_efficient import moba_attn_varlen, moba_attn_varlen_gqa
 from .wrapper import moba_layer
 
-__all__ = ["MoBAConfig", "register_moba", "moba_attn_varlen", "moba_layer"]
+__all__ = ["MoBAConfig", "register_moba", "moba_attn_varlen", "moba_attn_varlen_gqa", "moba_layer"]
 
 
 def register_moba(cfg: MoBAConfig):

@@ -20,6 +20,7 @@ struct TileTables {
   const int* chunk_tok;         // [N+1] first token of every chunk
   const int* self_tile_prefix;  // [N+1] prefix sum of row tiles per chunk
   int S, H, K1, F, N, B;
+  int Hkv, rep;                 // key/value heads and query heads per key/value head (H = Hkv * rep)
   int hist_bound;               // logical tile ids below it are history tiles
   int self_total;               // self_tile_prefix[N] * H
 };

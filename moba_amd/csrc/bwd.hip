@@ -102,7 +102,8 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams<E> p) {
   const float lse2 = p.lse[(int64_t)t.tok * H + h] * kLog2e;
   const float dl = p.delta[(int64_t)t.tok * H + h];
 
-  const int64_t row_bytes = (int64_t)H * kHeadDim * 2;
+  const int hkv = h / p.t.rep;                                // key/value head of this query head
+  const int64_t row_bytes = (int64_t)p.t.Hkv * kHeadDim * 2;   // of a K or V token row
   const uint32_t lds_base = lds_addr(smem);
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   const int ld_kin = lane >> 4, ld_pc = lane & 15;
@@ -118,7 +119,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams<E> p) {
       const int c16 = sw_col16(key, ld_pc);
       int64_t tk = kv_tok0 + key0 + key;
       if (!full) tk = min(tk, (int64_t)p.t.S - 1);
-      const int64_t off = tk * row_bytes + h * (kHeadDim * 2) + c16 * 16;
+      const int64_t off = tk * row_bytes + hkv * (kHeadDim * 2) + c16 * 16;
       async_copy16((const char*)p.k + off, kdst + slab * 1024);
       async_copy16((const char*)p.v + off, vdst + slab * 1024);
     }
@@ -285,21 +286,21 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int n = lane & 31, hh = lane >> 5;
-  const int H = p.t.H, K1 = p.t.K1;
+  const int H = p.t.H, K1 = p.t.K1, Hkv = p.t.Hkv, rep = p.t.rep;
 
-  // ---- which 128-key tile: same enumeration as the forward's self tiles ----
+  // ---- which 128-key tile of which key/value head: the forward's self-tile enumeration over Hkv heads ----
   const int st = logical_tile_id();
-  if (st >= p.t.self_total) return;
+  if (st >= p.t.self_total / rep) return;
   int lo = 0, hi = p.t.N;
   while (hi - lo > 1) {
     const int mid = (lo + hi) >> 1;
-    if (p.t.self_tile_prefix[mid] * H <= st) lo = mid; else hi = mid;
+    if (p.t.self_tile_prefix[mid] * Hkv <= st) lo = mid; else hi = mid;
   }
   const int c = lo;
-  const int rem = st - p.t.self_tile_prefix[c] * H;
+  const int rem = st - p.t.self_tile_prefix[c] * Hkv;
   const int nt = p.t.self_tile_prefix[c + 1] - p.t.self_tile_prefix[c];
-  const int h = rem / nt;
-  const int tin = rem - h * nt;
+  const int hkv = rem / nt;
+  const int tin = rem - hkv * nt;
   const int c0 = p.t.chunk_tok[c];
   const int len = p.t.chunk_tok[c + 1] - c0;
   const int key0 = tin * TM;
@@ -309,21 +310,24 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
   // ---- the rows that attend these keys: causal rows of the chunk, then the gather list ----
   const int self_rows = len - key0;              // chunk positions key0 .. len-1
   const int nself = (self_rows + TQ - 1) / TQ;
-  int list_base = 0, list_rows = 0;
-  {
-    const int f = (p.chunk_fid && K1 > 1) ? p.chunk_fid[c] : -1;
-    if (f >= 0) {
-      list_base = p.t.seg_off[f * H + h];
-      list_rows = p.t.seg_off[f * H + h + 1] - list_base;
+  const int fid = (p.chunk_fid && K1 > 1) ? p.chunk_fid[c] : -1;
+  // the query heads of this key/value head are walked one after the other; per head:
+  int h = hkv * rep, list_base = 0, list_rows = 0, ntile = nself;
+  auto select_head = [&](int hq) __attribute__((always_inline)) {
+    h = hq;
+    list_base = 0;
+    list_rows = 0;
+    if (fid >= 0) {
+      list_base = p.t.seg_off[fid * H + hq];
+      list_rows = p.t.seg_off[fid * H + hq + 1] - list_base;
     }
-  }
-  const int nhist = (list_rows + TQ - 1) / TQ;
-  const int ntile = nself + nhist;
+    ntile = nself + (list_rows + TQ - 1) / TQ;
+  };
 
   // ---- K^T and V^T operands of this lane's key: [16*ks + 8*hh .. +7] ----
   elem8 bk[8], bv[8];
   {
-    const int64_t off = ((int64_t)(c0 + min(mykey, len - 1)) * H + h) * kHeadDim + 8 * hh;
+    const int64_t off = ((int64_t)(c0 + min(mykey, len - 1)) * Hkv + hkv) * kHeadDim + 8 * hh;
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
       bk[ks] = *reinterpret_cast<const elem8*>(p.k + off + 16 * ks);
@@ -499,6 +503,9 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
     __builtin_amdgcn_sched_barrier(0);
   };
 
+  for (int hq = hkv * rep; hq < (hkv + 1) * rep; ++hq) {
+  select_head(hq);
+  __syncthreads();  // every wave is done with the LDS stages of the previous head
 #pragma unroll
   for (int i = 0; i < 5; ++i) raw[i] = 0;
   fetch_rows(0);
@@ -552,10 +559,11 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
     phase_b(qs, 1, pb, dsb, qs_next, 1, qs_next, 0);
     buf = buf1;
   }
+  }  // query heads
 #undef MOBA_PIN
 
   if (key_valid) {
-    const int64_t off = ((int64_t)(c0 + mykey) * H + h) * kHeadDim;
+    const int64_t off = ((int64_t)(c0 + mykey) * Hkv + hkv) * kHeadDim;
 #pragma unroll
     for (int db = 0; db < 4; ++db)
 #pragma unroll
@@ -619,7 +627,7 @@ extern "C" int moba_bwd(const void* dout, const void* q, const void* k, const vo
                         const float* lse, const int32_t* sel, const int32_t* seg_off, const int32_t* tile_off,
                         const int32_t* seg_dest, const int32_t* fchunk_tok, const int32_t* chunk_tok,
                         const int32_t* self_tile_prefix, const int32_t* chunk_fid, float* delta, float* part_dq,
-                        void* dq, void* dk, void* dv, int64_t S, int H, int D, int K, int F, int N, int B,
+                        void* dq, void* dk, void* dv, int64_t S, int H, int Hkv, int D, int K, int F, int N, int B,
                         int64_t hist_bound, int64_t self_tiles, int dtype, void* stream) {
   if (!dout || !q || !k || !v || !out || !lse || !chunk_tok || !self_tile_prefix || !delta || !part_dq || !dq ||
       !dk || !dv)
@@ -627,6 +635,7 @@ extern "C" int moba_bwd(const void* dout, const void* q, const void* k, const vo
   if (K > 0 && (!sel || !seg_off || !tile_off || !seg_dest || !fchunk_tok || !chunk_fid)) return MOBA_ERR_ARG;
   if (D != kHeadDim || (dtype != MOBA_DTYPE_BF16 && dtype != MOBA_DTYPE_F16)) return MOBA_ERR_UNSUPPORTED;
   if (S <= 0 || H <= 0 || K < 0 || F < 0 || N <= 0 || B <= 0 || hist_bound < 0 || self_tiles <= 0) return MOBA_ERR_ARG;
+  if (Hkv <= 0 || H % Hkv != 0) return MOBA_ERR_ARG;
   const void* ptrs[] = {dout, q, k, v, out, part_dq, dq, dk, dv};
   for (const void* x : ptrs)
     if ((uintptr_t)x & 15) return MOBA_ERR_ARG;
@@ -634,12 +643,13 @@ extern "C" int moba_bwd(const void* dout, const void* q, const void* k, const vo
   const int64_t per = 8 * kXcdBlock;
   const int64_t total_q = (K > 0 ? hist_bound : 0) + self_tiles * H;
   const int64_t grid_q = (total_q + per - 1) / per * per;
-  const int64_t grid_kv = (self_tiles * H + per - 1) / per * per;
+  const int64_t grid_kv = (self_tiles * Hkv + per - 1) / per * per;
   if (grid_q >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
   TileTables t;
   t.seg_off = seg_off; t.tile_off = tile_off; t.seg_dest = seg_dest; t.fchunk_tok = fchunk_tok;
   t.chunk_tok = chunk_tok; t.self_tile_prefix = self_tile_prefix;
   t.S = (int)S; t.H = H; t.K1 = K + 1; t.F = (K > 0) ? F : 0; t.N = N; t.B = B;
+  t.Hkv = Hkv; t.rep = H / Hkv;
   t.hist_bound = (K > 0) ? (int)hist_bound : 0;
   t.self_total = (int)(self_tiles * H);
   hipStream_t st = (hipStream_t)stream;

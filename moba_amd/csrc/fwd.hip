@@ -67,7 +67,8 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
   // A wave copy fills 1 KiB = 4 keys x 16 columns of 16 bytes; wave w issues slabs
   // w, w+4, w+8, w+12.  Lane i lands at slab + 16*i, so the lane picks the global column
   // whose swizzled LDS position is i.  LDS: K stages at 0 and 16 KiB, V stages at 32 and 48 KiB.
-  const int64_t row_bytes = (int64_t)H * kHeadDim * 2;
+  const int hkv = h / p.t.rep;                                   // key/value head of this query head
+  const int64_t row_bytes = (int64_t)p.t.Hkv * kHeadDim * 2;      // of a K or V token row
   const uint32_t lds_base = lds_addr(smem);
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   const int ld_kin = lane >> 4;  // key within the slab
@@ -78,8 +79,8 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
     const int key = 4 * (4 * i + wave_u) + ld_kin;
     ld_off[i] = (uint32_t)(key * row_bytes + sw_col16(key, ld_pc) * 16);  // the swizzle is an involution
   }
-  const char* k_head = (const char*)p.k + (int64_t)kv_tok0 * row_bytes + h * (kHeadDim * 2);
-  const char* v_head = (const char*)p.v + (int64_t)kv_tok0 * row_bytes + h * (kHeadDim * 2);
+  const char* k_head = (const char*)p.k + (int64_t)kv_tok0 * row_bytes + hkv * (kHeadDim * 2);
+  const char* v_head = (const char*)p.v + (int64_t)kv_tok0 * row_bytes + hkv * (kHeadDim * 2);
   auto issue = [&](const char* head, const char* tensor, int kt, uint32_t dst) __attribute__((always_inline)) {
     const int key0 = kt * TN;
     const bool full = (key0 + TN <= nkeys) && (kv_tok0 + key0 + TN <= p.t.S);
@@ -93,7 +94,7 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
         const int slab = 4 * i + wave_u;
         const int key = 4 * slab + ld_kin;
         const int64_t tk = min((int64_t)kv_tok0 + key0 + key, (int64_t)p.t.S - 1);
-        async_copy16(tensor + tk * row_bytes + h * (kHeadDim * 2) + sw_col16(key, ld_pc) * 16, dst + slab * 1024);
+        async_copy16(tensor + tk * row_bytes + hkv * (kHeadDim * 2) + sw_col16(key, ld_pc) * 16, dst + slab * 1024);
       }
     }
   };
@@ -436,9 +437,10 @@ static int launch_partials(const void* q, const void* k, const void* v, void* pa
 extern "C" int moba_fwd_partials(const void* q, const void* k, const void* v, void* part_o, float* part_lse,
                                  const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest,
                                  const int32_t* fchunk_tok, const int32_t* chunk_tok,
-                                 const int32_t* self_tile_prefix, int64_t S, int H, int D, int K, int F, int N, int B,
-                                 int64_t hist_bound, int64_t self_tiles, int dtype, void* stream) {
+                                 const int32_t* self_tile_prefix, int64_t S, int H, int Hkv, int D, int K, int F,
+                                 int N, int B, int64_t hist_bound, int64_t self_tiles, int dtype, void* stream) {
   if (!q || !k || !v || !part_o || !part_lse || !chunk_tok || !self_tile_prefix) return MOBA_ERR_ARG;
+  if (Hkv <= 0 || H % Hkv != 0) return MOBA_ERR_ARG;
   if (K > 0 && (!seg_off || !tile_off || !seg_dest || !fchunk_tok)) return MOBA_ERR_ARG;
   if (D != kHeadDim || (dtype != MOBA_DTYPE_BF16 && dtype != MOBA_DTYPE_F16)) return MOBA_ERR_UNSUPPORTED;
   if (S <= 0 || H <= 0 || K < 0 || F < 0 || N <= 0 || B <= 0 || hist_bound < 0 || self_tiles <= 0) return MOBA_ERR_ARG;
@@ -451,6 +453,7 @@ extern "C" int moba_fwd_partials(const void* q, const void* k, const void* v, vo
   t.seg_off = seg_off; t.tile_off = tile_off; t.seg_dest = seg_dest; t.fchunk_tok = fchunk_tok;
   t.chunk_tok = chunk_tok; t.self_tile_prefix = self_tile_prefix;
   t.S = (int)S; t.H = H; t.K1 = K + 1; t.F = (K > 0) ? F : 0; t.N = N; t.B = B;
+  t.Hkv = Hkv; t.rep = H / Hkv;
   t.hist_bound = (K > 0) ? (int)hist_bound : 0;
   t.self_total = (int)(self_tiles * H);
   hipStream_t st = (hipStream_t)stream;
@@ -478,10 +481,11 @@ extern "C" int moba_fwd_merge(const void* part_o, const float* part_lse, const i
 extern "C" int moba_fwd(const void* q, const void* k, const void* v, void* part_o, float* part_lse,
                         const int32_t* sel, const int32_t* seg_off, const int32_t* tile_off,
                         const int32_t* seg_dest, const int32_t* fchunk_tok, const int32_t* chunk_tok,
-                        const int32_t* self_tile_prefix, void* out, float* lse, int64_t S, int H, int D, int K,
-                        int F, int N, int B, int64_t hist_bound, int64_t self_tiles, int dtype, void* stream) {
+                        const int32_t* self_tile_prefix, void* out, float* lse, int64_t S, int H, int Hkv, int D,
+                        int K, int F, int N, int B, int64_t hist_bound, int64_t self_tiles, int dtype,
+                        void* stream) {
   int rc = moba_fwd_partials(q, k, v, part_o, part_lse, seg_off, tile_off, seg_dest, fchunk_tok, chunk_tok,
-                             self_tile_prefix, S, H, D, K, F, N, B, hist_bound, self_tiles, dtype, stream);
+                             self_tile_prefix, S, H, Hkv, D, K, F, N, B, hist_bound, self_tiles, dtype, stream);
   if (rc != MOBA_OK) return rc;
   return moba_fwd_merge(part_o, part_lse, sel, out, lse, S, H, D, K, dtype, stream);
 }

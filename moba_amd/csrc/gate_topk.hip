@@ -55,7 +55,7 @@ template <class E, int KMAX>
 __global__ __launch_bounds__(256) void gate_topk_kernel(
     const typename E::elem* __restrict__ q, const typename E::elem* __restrict__ kbar, const int* __restrict__ cu_seqlens,
     const int* __restrict__ seq_fbase, int* __restrict__ sel, float* __restrict__ scores_out,
-    int S, int H, int nseq, int F, int B, int K) {
+    int S, int H, int Hkv, int nseq, int F, int B, int K) {
   MOBA_ELEM_TYPES(E)
   __shared__ float sc[4][64][33];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -97,7 +97,7 @@ __global__ __launch_bounds__(256) void gate_topk_kernel(
     }
     for (int f0 = flo; f0 < fhi; f0 += 32) {
       const int fr = min(f0 + n, F - 1);
-      const elem* src = kbar + ((int64_t)fr * H + hc) * kHeadDim + 8 * hh;
+      const elem* src = kbar + ((int64_t)fr * Hkv + hc / (H / Hkv)) * kHeadDim + 8 * hh;
       f32x16 acc0 = {0}, acc1 = {0};
 #pragma unroll
       for (int ks = 0; ks < 8; ++ks) {
@@ -165,9 +165,10 @@ using namespace moba;
   else return MOBA_ERR_LIMIT;
 
 extern "C" int moba_gate_topk(const void* q, const void* kbar, const int32_t* cu_seqlens, const int32_t* seq_fbase,
-                              int32_t* sel, float* scores_out, int64_t S, int H, int D, int nseq, int F, int B,
-                              int K, int dtype, void* stream) {
+                              int32_t* sel, float* scores_out, int64_t S, int H, int Hkv, int D, int nseq, int F,
+                              int B, int K, int dtype, void* stream) {
   if (!q || !kbar || !cu_seqlens || !seq_fbase || !sel) return MOBA_ERR_ARG;
+  if (Hkv <= 0 || H % Hkv != 0) return MOBA_ERR_ARG;
   if (dtype != MOBA_DTYPE_BF16 && dtype != MOBA_DTYPE_F16) return MOBA_ERR_UNSUPPORTED;
   if (S <= 0 || S > 0x7fffffff - 64 || H <= 0 || nseq <= 0 || F <= 0 || B <= 0 || K <= 0) return MOBA_ERR_ARG;
   if (D != kHeadDim) return MOBA_ERR_UNSUPPORTED;
@@ -177,10 +178,10 @@ extern "C" int moba_gate_topk(const void* q, const void* kbar, const int32_t* cu
 #define CALL(KM)                                                                                               \
   if (dtype == MOBA_DTYPE_F16)                                                                                 \
     hipLaunchKernelGGL((gate_topk_kernel<F16, KM>), grid, dim3(256), 0, st, (const f16*)q, (const f16*)kbar,   \
-                       cu_seqlens, seq_fbase, sel, scores_out, (int)S, H, nseq, F, B, K);                      \
+                       cu_seqlens, seq_fbase, sel, scores_out, (int)S, H, Hkv, nseq, F, B, K);                      \
   else                                                                                                         \
     hipLaunchKernelGGL((gate_topk_kernel<Bf16, KM>), grid, dim3(256), 0, st, (const bf16*)q, (const bf16*)kbar, \
-                       cu_seqlens, seq_fbase, sel, scores_out, (int)S, H, nseq, F, B, K)
+                       cu_seqlens, seq_fbase, sel, scores_out, (int)S, H, Hkv, nseq, F, B, K)
   MOBA_DISPATCH_K(K, CALL)
 #undef CALL
   return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;

@@ -40,12 +40,17 @@ def _dtype_code(t: torch.Tensor) -> int:
     raise TypeError("moba_attn_varlen supports bfloat16 and float16 q, k, v")
 
 
-def _check_qkv(q, k, v):
+def _check_qkv(q, k, v, gqa=False):
     if not (q.is_cuda and k.is_cuda and v.is_cuda):
         raise RuntimeError("moba_attn_varlen needs tensors on an AMD GPU (there is no CPU path)")
     if q.dtype not in (torch.bfloat16, torch.float16) or k.dtype != q.dtype or v.dtype != q.dtype:
         raise TypeError("moba_attn_varlen supports bfloat16 and float16 q, k, v (all three of the same dtype)")
-    if q.dim() != 3 or q.shape != k.shape or q.shape != v.shape:
+    if q.dim() != 3 or k.shape != v.shape or k.dim() != 3 or q.shape[0] != k.shape[0] or q.shape[2] != k.shape[2]:
+        raise ValueError("q must be [seqlen, heads, head_dim] and k, v [seqlen, kv_heads, head_dim]")
+    if gqa:
+        if k.shape[1] == 0 or q.shape[1] % k.shape[1] != 0:
+            raise ValueError("the number of query heads must be a multiple of the number of key/value heads")
+    elif q.shape != k.shape:
         raise ValueError("q, k, v must all be [seqlen, heads, head_dim] with the same number of heads")
     if q.shape[2] != HEAD_DIM:
         raise ValueError(f"head_dim must be {HEAD_DIM}")
@@ -65,15 +70,17 @@ def chunk_mean(k: torch.Tensor, plan: MobaPlan) -> torch.Tensor:
 
 
 def gate_topk(q: torch.Tensor, kbar: torch.Tensor, plan: MobaPlan, return_scores: bool = False):
-    """sel [S, H, K] int32: selected filtered-chunk ids per (token, head), -1 padded."""
+    """sel [S, H, K] int32: selected filtered-chunk ids per (token, head), -1 padded.
+    kbar may have fewer heads than q (grouped-query attention)."""
     lib = _lib.load()
     S, H, D = q.shape
+    Hkv = kbar.shape[1]
     sel = torch.empty((S, H, plan.K), dtype=torch.int32, device=q.device)
     scores = None
     if return_scores:
         scores = torch.full((S, H, plan.F), float("-inf"), dtype=torch.float32, device=q.device)
     _lib.check(lib.moba_gate_topk(_ptr(q), _ptr(kbar), _ptr(plan.tables["cu_seqlens"]), _ptr(plan.tables["seq_fbase"]),
-                                  _ptr(sel), _ptr(scores), S, H, D, plan.nseq, plan.F, plan.chunk_size, plan.K,
+                                  _ptr(sel), _ptr(scores), S, H, Hkv, D, plan.nseq, plan.F, plan.chunk_size, plan.K,
                                   _dtype_code(q), _stream(q.device)), "moba_gate_topk")
     return (sel, scores) if return_scores else sel
 
@@ -167,7 +174,8 @@ def _forward(q, k, v, plan: MobaPlan, timer: Optional[StageTimer] = None):
     with span("fwd_partials"):
         _lib.check(lib.moba_fwd_partials(_ptr(q), _ptr(k), _ptr(v), _ptr(part_o), _ptr(part_lse), _ptr(seg_off),
                                          _ptr(tile_off), _ptr(seg_dest), _ptr(t.get("fchunk_tok")),
-                                         _ptr(t["chunk_tok"]), _ptr(t["self_tile_prefix"]), S, H, D, K, plan.F, plan.N,
+                                         _ptr(t["chunk_tok"]), _ptr(t["self_tile_prefix"]), S, H, k.shape[1], D, K, plan.F,
+                                         plan.N,
                                          plan.chunk_size, plan.hist_tile_bound(H), plan.self_tiles, _dtype_code(q),
                                          _stream(dev)), "moba_fwd_partials")
     with span("fwd_merge"):
@@ -191,7 +199,8 @@ def _backward(dout, q, k, v, out, lse, sel, seg_off, tile_off, seg_dest, plan: M
                             _ptr(tile_off), _ptr(seg_dest), _ptr(t.get("fchunk_tok")), _ptr(t["chunk_tok"]),
                             _ptr(t["self_tile_prefix"]), _ptr(t.get("chunk_fid")),
                             _ptr(delta), _ptr(part_dq), _ptr(dq), _ptr(dk), _ptr(dv),
-                            S, H, D, K, plan.F, plan.N, plan.chunk_size, plan.hist_tile_bound(H), plan.self_tiles,
+                            S, H, k.shape[1], D, K, plan.F, plan.N, plan.chunk_size, plan.hist_tile_bound(H),
+                            plan.self_tiles,
                             _dtype_code(q), _stream(dev)), "moba_bwd")
     return dq, dk, dv
 
@@ -238,10 +247,23 @@ def moba_attn_varlen(
     return moba_attn_varlen_with_lse(q, k, v, cu_seqlens, max_seqlen, moba_chunk_size, moba_topk)[0]
 
 
-def moba_attn_varlen_with_lse(q, k, v, cu_seqlens, max_seqlen, moba_chunk_size, moba_topk, timer=None):
+def moba_attn_varlen_gqa(q, k, v, cu_seqlens, max_seqlen, moba_chunk_size, moba_topk):
+    """``moba_attn_varlen`` with grouped-query attention inside the operator: k, v are
+    [seqlen, kv_heads, head_dim] and query head h reads key/value head h // (heads // kv_heads),
+    as ``repeat_interleave`` on the head axis would give (moba/wrapper.py:59-61), without the
+    copies.  The chunk representatives are computed once per key/value head; dk, dv are summed
+    over the query heads of a group.  No counterpart in the reference operator."""
+    return moba_attn_varlen_with_lse(q, k, v, cu_seqlens, max_seqlen, moba_chunk_size, moba_topk, gqa=True)[0]
+
+
+# lets moba_layer skip the key/value head expansion when it drives this operator
+moba_attn_varlen.grouped_query_impl = moba_attn_varlen_gqa
+
+
+def moba_attn_varlen_with_lse(q, k, v, cu_seqlens, max_seqlen, moba_chunk_size, moba_topk, timer=None, gqa=False):
     """As ``moba_attn_varlen`` but also returns the natural-log LSE [seqlen, heads] fp32.
-    ``timer`` (a StageTimer) collects per-stage device times."""
-    _check_qkv(q, k, v)
+    ``timer`` (a StageTimer) collects per-stage device times; ``gqa`` allows fewer key/value heads."""
+    _check_qkv(q, k, v, gqa)
     plan = make_plan(cu_seqlens, moba_chunk_size, moba_topk, device=q.device)
     if plan.S != q.shape[0]:
         raise ValueError(f"cu_seqlens ends at {plan.S} but q has {q.shape[0]} tokens")

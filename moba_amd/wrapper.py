@@ -1,7 +1,8 @@
 """transformers attention-interface adapter, mirroring moba/wrapper.py:29-84.
 
 Prefill (q_len == kv_len) converts the HF layout [batch, heads, seq, dim] to the packed
-varlen layout, expands KV heads to the query heads and calls the MoBA operator.
+varlen layout and calls the MoBA operator (KV heads are expanded to the query heads first
+unless the operator handles grouped-query attention itself).
 Decode (q_len != kv_len) is full causal attention over the KV cache, as in the
 reference (moba/wrapper.py:76-82), done with PyTorch's scaled_dot_product_attention.
 """
@@ -55,8 +56,14 @@ def moba_layer(
         v = hf_to_fa(value)
         rep = q_heads // kv_heads
         if rep > 1:
-            k = torch.repeat_interleave(k, rep, dim=1)
-            v = torch.repeat_interleave(v, rep, dim=1)
+            # an implementation that indexes key/value heads itself (the HIP operator) takes them as they are;
+            # others get the expanded copies, as in the reference (moba/wrapper.py:59-61)
+            grouped = getattr(moba_impl, "grouped_query_impl", None)
+            if grouped is not None:
+                moba_impl = grouped
+            else:
+                k = torch.repeat_interleave(k, rep, dim=1)
+                v = torch.repeat_interleave(v, rep, dim=1)
         cu_seqlens = torch.arange(0, (batch + 1) * kv_len, kv_len, dtype=torch.int32, device=query.device)
         out = moba_impl(
             q=q,

@@ -107,6 +107,40 @@ def test_float16(batch, seqlen, heads, B, topk):
     run_case(batch, seqlen, heads, B, topk, seed=11, dtype=torch.float16)
 
 
+@pytest.mark.parametrize("batch,seqlen,heads,kv_heads,B,topk,dtype", [
+    (1, 1024, 4, 1, 128, 3, torch.bfloat16),
+    (3, 2048, 8, 2, 256, 3, torch.bfloat16),
+    (2, 1500, 6, 3, 100, 4, torch.bfloat16),
+    (4, 2048, 8, 2, 128, 2, torch.float16),
+    (1, 2048, 4, 2, 128, 1, torch.bfloat16),     # fallback: full causal attention
+])
+def test_grouped_query(batch, seqlen, heads, kv_heads, B, topk, dtype):
+    """k, v with fewer heads: same result (bit for bit in the forward) as expanding them with
+    repeat_interleave first (moba/wrapper.py:59-61); dk, dv equal the sums over each group within rounding."""
+    from moba_amd import moba_attn_varlen, moba_attn_varlen_gqa
+    rep = heads // kv_heads
+    q, _, _, do, cu, mx = make_case(batch, seqlen, heads, seed=5, dtype=dtype)
+    _, k, v, _, _, _ = make_case(batch, seqlen, kv_heads, seed=6, dtype=dtype)
+    cu_t = torch.tensor(cu, dtype=torch.int32, device="cuda")
+    qa, ka, va = (x.cuda().requires_grad_(True) for x in (q, k, v))
+    out_a = moba_attn_varlen_gqa(qa, ka, va, cu_t, mx, B, topk)
+    out_a.backward(do.cuda())
+    qb = q.cuda().requires_grad_(True)
+    kb = torch.repeat_interleave(k.cuda(), rep, dim=1).requires_grad_(True)
+    vb = torch.repeat_interleave(v.cuda(), rep, dim=1).requires_grad_(True)
+    out_b = moba_attn_varlen(qb, kb, vb, cu_t, mx, B, topk)
+    out_b.backward(do.cuda())
+    assert torch.equal(out_a, out_b)
+    assert torch.equal(qa.grad, qb.grad)
+    for ga, gb in ((ka.grad, kb.grad), (va.grad, vb.grad)):
+        want = gb.float().view(seqlen, kv_heads, rep, 128).sum(2)
+        err = (ga.float() - want).abs()
+        assert err.max() <= 2e-2 * want.abs().max().clamp_min(1.0), err.max().item()
+        assert err.mean() <= 4e-3 * want.abs().mean() + 1e-6, (err.mean().item(), want.abs().mean().item())
+    with pytest.raises(ValueError):
+        moba_attn_varlen(qa, ka, va, cu_t, mx, B, topk)       # the 7-argument operator keeps the reference's contract
+
+
 def test_one_token_sequences():
     from moba_amd import moba_efficient as E
     g = torch.Generator().manual_seed(3)
