@@ -67,31 +67,35 @@ int moba_topk_from_scores(const float* scores, int32_t* sel, int64_t S, int H, i
  *   seg_off  [F*H+1] out, list start of segment (f,h);  tile_off [F*H+1] out, prefix
  *            sum of ceil(rows/tile_rows);  seg_dest [M] out, entries
  *            (token*H + h)*(K+1) + 1 + slot
- * cmax = most chunks in a sequence minus one. */
+ *   tile_seg [hist_bound] out: segment f*H + h of every history tile id, -1 past the last tile
+ * cmax = most chunks in a sequence minus one; hist_bound as in moba_fwd_partials. */
 int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, const int32_t* chunk_fb, const int32_t* chunk_local,
                      const int32_t* pair_off, int32_t* cnt, int32_t* seg_off, int32_t* tile_off, int32_t* seg_dest,
-                     int64_t S, int H, int K, int N, int F, int P, int cmax, int tile_rows, void* stream);
+                     int32_t* tile_seg, int64_t S, int H, int K, int N, int F, int P, int cmax, int tile_rows,
+                     int64_t hist_bound, void* stream);
 
 /* Attention.  Replaces MixedAttention.forward, moba/moba_efficient.py:69-183 (two
  * flash-attn varlen forwards and the LSE merge), and with K = 0 and one chunk per
  * sequence the full-causal case of moba/moba_efficient.py:318-321.
  *   part_o [S*H*(K+1), D] elem and part_lse [S*H*(K+1)] fp32: per-slot partial results
  *   self_tile_prefix [N+1] int32: prefix sum of ceil(chunk_len / moba_fwd_tile_rows())
+ *   self_tile_chunk [self_tile_prefix[N]] int32: the chunk of each of those tiles
+ *   tile_seg: from moba_build_lists (may be NULL when K = 0)
  *   out [S,H,D] elem, lse [S,H] fp32 (natural log)
  *   hist_bound: upper bound on the number of history tiles, e.g. M/tile_rows + F*H
  *   self_tiles: self_tile_prefix[N] */
 int moba_fwd_tile_rows(void);
 int moba_fwd_partials(const void* q, const void* k, const void* v, void* part_o, float* part_lse,
                       const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest,
-                      const int32_t* fchunk_tok, const int32_t* chunk_tok, const int32_t* self_tile_prefix, int64_t S,
-                      int H, int Hkv, int D, int K, int F, int N, int B, int64_t hist_bound, int64_t self_tiles,
+                      const int32_t* fchunk_tok, const int32_t* chunk_tok, const int32_t* self_tile_prefix,
+                      const int32_t* tile_seg, const int32_t* self_tile_chunk, int64_t S, int H, int Hkv, int D, int K, int F, int N, int B, int64_t hist_bound, int64_t self_tiles,
                       int dtype, void* stream);
 int moba_fwd_merge(const void* part_o, const float* part_lse, const int32_t* sel, void* out, float* lse, int64_t S,
                    int H, int D, int K, int dtype, void* stream);
 int moba_fwd(const void* q, const void* k, const void* v, void* part_o, float* part_lse, const int32_t* sel,
              const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest, const int32_t* fchunk_tok,
-             const int32_t* chunk_tok, const int32_t* self_tile_prefix, void* out, float* lse, int64_t S, int H, int Hkv,
-             int D, int K, int F, int N, int B, int64_t hist_bound, int64_t self_tiles, int dtype, void* stream);
+             const int32_t* chunk_tok, const int32_t* self_tile_prefix, const int32_t* tile_seg,
+             const int32_t* self_tile_chunk, void* out, float* lse, int64_t S, int H, int Hkv, int D, int K, int F, int N, int B, int64_t hist_bound, int64_t self_tiles, int dtype, void* stream);
 
 /* Backward.  Replaces MixedAttention.backward, moba/moba_efficient.py:185-267, and the
  * autograd scatter of its gathered gradients.  Deterministic (no floating-point atomics).
@@ -102,7 +106,7 @@ int moba_fwd(const void* q, const void* k, const void* v, void* part_o, float* p
 int moba_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out, const float* lse,
              const int32_t* sel, const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest,
              const int32_t* fchunk_tok, const int32_t* chunk_tok, const int32_t* self_tile_prefix,
-             const int32_t* chunk_fid, float* delta, float* part_dq, void* dq, void* dk, void* dv, int64_t S, int H,
+             const int32_t* tile_seg, const int32_t* self_tile_chunk, const int32_t* chunk_fid, float* delta, float* part_dq, void* dq, void* dk, void* dv, int64_t S, int H,
              int Hkv, int D, int K, int F, int N, int B, int64_t hist_bound, int64_t self_tiles, int dtype,
              void* stream);
 

@@ -25,14 +25,14 @@ _SIGNATURES = {
     "moba_gate_topk": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "moba_topk_from_scores": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_void_p]),
-    "moba_build_lists": (c_int, [c_void_p] * 9 + [c_int64] + [c_int] * 7 + [c_void_p]),
+    "moba_build_lists": (c_int, [c_void_p] * 10 + [c_int64] + [c_int] * 7 + [c_int64, c_void_p]),
     "moba_fwd_tile_rows": (c_int, []),
-    "moba_fwd_partials": (c_int, [c_void_p] * 11 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int64,
+    "moba_fwd_partials": (c_int, [c_void_p] * 13 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int64,
                                                    c_int64, c_int, c_void_p]),
     "moba_fwd_merge": (c_int, [c_void_p] * 5 + [c_int64, c_int, c_int, c_int, c_int, c_void_p]),
-    "moba_fwd": (c_int, [c_void_p] * 14 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_int64,
+    "moba_fwd": (c_int, [c_void_p] * 16 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_int64,
                                           c_int, c_void_p]),
-    "moba_bwd": (c_int, [c_void_p] * 19 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_int64,
+    "moba_bwd": (c_int, [c_void_p] * 21 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_int64,
                                           c_int, c_void_p]),
 }
 OPTIONAL = set()

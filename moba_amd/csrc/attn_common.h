@@ -19,6 +19,8 @@ struct TileTables {
   const int* fchunk_tok;        // [F] first token of filtered chunk f
   const int* chunk_tok;         // [N+1] first token of every chunk
   const int* self_tile_prefix;  // [N+1] prefix sum of row tiles per chunk
+  const int* tile_seg;          // [hist_bound] segment (f*H + h) of every history tile, -1 past the last one
+  const int* self_tile_chunk;   // [self_tile_prefix[N]] chunk of every per-head self tile
   int S, H, K1, F, N, B;
   int Hkv, rep;                 // key/value heads and query heads per key/value head (H = Hkv * rep)
   int hist_bound;               // logical tile ids below it are history tiles
@@ -49,9 +51,8 @@ __device__ __forceinline__ int logical_tile_id() {
 __device__ __forceinline__ bool decode_tile(const TileTables& p, int logical, int wave, int r, Tile& t) {
   const int H = p.H;
   if (logical < p.hist_bound) {
-    const int FH = p.F * H;
-    if (FH == 0 || logical >= p.tile_off[FH]) return false;
-    const int seg = upper_row(p.tile_off, FH, logical);
+    const int seg = p.tile_seg[logical];   // one lookup instead of a search in tile_off
+    if (seg < 0) return false;
     const int tile = logical - p.tile_off[seg];
     const int f = seg / H;
     t.h = seg - f * H;
@@ -69,12 +70,7 @@ __device__ __forceinline__ bool decode_tile(const TileTables& p, int logical, in
   }
   const int st = logical - p.hist_bound;
   if (st >= p.self_total) return false;
-  int lo = 0, hi = p.N;  // chunk c with self_tile_prefix[c]*H <= st
-  while (hi - lo > 1) {
-    const int mid = (lo + hi) >> 1;
-    if (p.self_tile_prefix[mid] * H <= st) lo = mid; else hi = mid;
-  }
-  const int c = lo;
+  const int c = p.self_tile_chunk[st / H];  // self_tile_prefix[c]*H <= st < self_tile_prefix[c+1]*H
   const int rem = st - p.self_tile_prefix[c] * H;
   const int nt = p.self_tile_prefix[c + 1] - p.self_tile_prefix[c];
   t.h = rem / nt;

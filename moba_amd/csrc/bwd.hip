@@ -291,12 +291,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
   // ---- which 128-key tile of which key/value head: the forward's self-tile enumeration over Hkv heads ----
   const int st = logical_tile_id();
   if (st >= p.t.self_total / rep) return;
-  int lo = 0, hi = p.t.N;
-  while (hi - lo > 1) {
-    const int mid = (lo + hi) >> 1;
-    if (p.t.self_tile_prefix[mid] * Hkv <= st) lo = mid; else hi = mid;
-  }
-  const int c = lo;
+  const int c = p.t.self_tile_chunk[st / Hkv];
   const int rem = st - p.t.self_tile_prefix[c] * Hkv;
   const int nt = p.t.self_tile_prefix[c + 1] - p.t.self_tile_prefix[c];
   const int hkv = rem / nt;
@@ -626,13 +621,15 @@ static int launch_bwd(const void* dout, const void* q, const void* k, const void
 extern "C" int moba_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out,
                         const float* lse, const int32_t* sel, const int32_t* seg_off, const int32_t* tile_off,
                         const int32_t* seg_dest, const int32_t* fchunk_tok, const int32_t* chunk_tok,
-                        const int32_t* self_tile_prefix, const int32_t* chunk_fid, float* delta, float* part_dq,
+                        const int32_t* self_tile_prefix, const int32_t* tile_seg, const int32_t* self_tile_chunk,
+                        const int32_t* chunk_fid, float* delta, float* part_dq,
                         void* dq, void* dk, void* dv, int64_t S, int H, int Hkv, int D, int K, int F, int N, int B,
                         int64_t hist_bound, int64_t self_tiles, int dtype, void* stream) {
-  if (!dout || !q || !k || !v || !out || !lse || !chunk_tok || !self_tile_prefix || !delta || !part_dq || !dq ||
-      !dk || !dv)
+  if (!dout || !q || !k || !v || !out || !lse || !chunk_tok || !self_tile_prefix || !self_tile_chunk || !delta ||
+      !part_dq || !dq || !dk || !dv)
     return MOBA_ERR_ARG;
-  if (K > 0 && (!sel || !seg_off || !tile_off || !seg_dest || !fchunk_tok || !chunk_fid)) return MOBA_ERR_ARG;
+  if (K > 0 && (!sel || !seg_off || !tile_off || !seg_dest || !fchunk_tok || !chunk_fid || !tile_seg))
+    return MOBA_ERR_ARG;
   if (D != kHeadDim || (dtype != MOBA_DTYPE_BF16 && dtype != MOBA_DTYPE_F16)) return MOBA_ERR_UNSUPPORTED;
   if (S <= 0 || H <= 0 || K < 0 || F < 0 || N <= 0 || B <= 0 || hist_bound < 0 || self_tiles <= 0) return MOBA_ERR_ARG;
   if (Hkv <= 0 || H % Hkv != 0) return MOBA_ERR_ARG;
@@ -648,6 +645,7 @@ extern "C" int moba_bwd(const void* dout, const void* q, const void* k, const vo
   TileTables t;
   t.seg_off = seg_off; t.tile_off = tile_off; t.seg_dest = seg_dest; t.fchunk_tok = fchunk_tok;
   t.chunk_tok = chunk_tok; t.self_tile_prefix = self_tile_prefix;
+  t.tile_seg = tile_seg; t.self_tile_chunk = self_tile_chunk;
   t.S = (int)S; t.H = H; t.K1 = K + 1; t.F = (K > 0) ? F : 0; t.N = N; t.B = B;
   t.Hkv = Hkv; t.rep = H / Hkv;
   t.hist_bound = (K > 0) ? (int)hist_bound : 0;

@@ -437,11 +437,12 @@ static int launch_partials(const void* q, const void* k, const void* v, void* pa
 extern "C" int moba_fwd_partials(const void* q, const void* k, const void* v, void* part_o, float* part_lse,
                                  const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest,
                                  const int32_t* fchunk_tok, const int32_t* chunk_tok,
-                                 const int32_t* self_tile_prefix, int64_t S, int H, int Hkv, int D, int K, int F,
+                                 const int32_t* self_tile_prefix, const int32_t* tile_seg,
+                                 const int32_t* self_tile_chunk, int64_t S, int H, int Hkv, int D, int K, int F,
                                  int N, int B, int64_t hist_bound, int64_t self_tiles, int dtype, void* stream) {
-  if (!q || !k || !v || !part_o || !part_lse || !chunk_tok || !self_tile_prefix) return MOBA_ERR_ARG;
+  if (!q || !k || !v || !part_o || !part_lse || !chunk_tok || !self_tile_prefix || !self_tile_chunk) return MOBA_ERR_ARG;
   if (Hkv <= 0 || H % Hkv != 0) return MOBA_ERR_ARG;
-  if (K > 0 && (!seg_off || !tile_off || !seg_dest || !fchunk_tok)) return MOBA_ERR_ARG;
+  if (K > 0 && (!seg_off || !tile_off || !seg_dest || !fchunk_tok || !tile_seg)) return MOBA_ERR_ARG;
   if (D != kHeadDim || (dtype != MOBA_DTYPE_BF16 && dtype != MOBA_DTYPE_F16)) return MOBA_ERR_UNSUPPORTED;
   if (S <= 0 || H <= 0 || K < 0 || F < 0 || N <= 0 || B <= 0 || hist_bound < 0 || self_tiles <= 0) return MOBA_ERR_ARG;
   if (((uintptr_t)q & 15) || ((uintptr_t)k & 15) || ((uintptr_t)v & 15) || ((uintptr_t)part_o & 15)) return MOBA_ERR_ARG;
@@ -452,6 +453,7 @@ extern "C" int moba_fwd_partials(const void* q, const void* k, const void* v, vo
   TileTables t;
   t.seg_off = seg_off; t.tile_off = tile_off; t.seg_dest = seg_dest; t.fchunk_tok = fchunk_tok;
   t.chunk_tok = chunk_tok; t.self_tile_prefix = self_tile_prefix;
+  t.tile_seg = tile_seg; t.self_tile_chunk = self_tile_chunk;
   t.S = (int)S; t.H = H; t.K1 = K + 1; t.F = (K > 0) ? F : 0; t.N = N; t.B = B;
   t.Hkv = Hkv; t.rep = H / Hkv;
   t.hist_bound = (K > 0) ? (int)hist_bound : 0;
@@ -481,11 +483,12 @@ extern "C" int moba_fwd_merge(const void* part_o, const float* part_lse, const i
 extern "C" int moba_fwd(const void* q, const void* k, const void* v, void* part_o, float* part_lse,
                         const int32_t* sel, const int32_t* seg_off, const int32_t* tile_off,
                         const int32_t* seg_dest, const int32_t* fchunk_tok, const int32_t* chunk_tok,
-                        const int32_t* self_tile_prefix, void* out, float* lse, int64_t S, int H, int Hkv, int D,
-                        int K, int F, int N, int B, int64_t hist_bound, int64_t self_tiles, int dtype,
-                        void* stream) {
+                        const int32_t* self_tile_prefix, const int32_t* tile_seg, const int32_t* self_tile_chunk,
+                        void* out, float* lse, int64_t S, int H, int Hkv, int D, int K, int F, int N, int B,
+                        int64_t hist_bound, int64_t self_tiles, int dtype, void* stream) {
   int rc = moba_fwd_partials(q, k, v, part_o, part_lse, seg_off, tile_off, seg_dest, fchunk_tok, chunk_tok,
-                             self_tile_prefix, S, H, Hkv, D, K, F, N, B, hist_bound, self_tiles, dtype, stream);
+                             self_tile_prefix, tile_seg, self_tile_chunk, S, H, Hkv, D, K, F, N, B, hist_bound,
+                             self_tiles, dtype, stream);
   if (rc != MOBA_OK) return rc;
   return moba_fwd_merge(part_o, part_lse, sel, out, lse, S, H, D, K, dtype, stream);
 }

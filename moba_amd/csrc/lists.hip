@@ -189,6 +189,15 @@ __global__ __launch_bounds__(256) void lists_segments_kernel(const int* __restri
   tile_off[fh] = (end - start + tile_rows - 1) / tile_rows;
 }
 
+// segment of every history tile id below `bound` (-1 past the last tile): the attention
+// kernels then find their tile with one load instead of a search in tile_off
+__global__ __launch_bounds__(256) void lists_tile_seg_kernel(const int* __restrict__ tile_off,
+                                                             int* __restrict__ tile_seg, int FH, int bound) {
+  const int t = blockIdx.x * 256 + threadIdx.x;
+  if (t >= bound) return;
+  tile_seg[t] = t < tile_off[FH] ? upper_row(tile_off, FH, t) : -1;
+}
+
 }  // namespace moba
 
 using namespace moba;
@@ -197,10 +206,13 @@ using namespace moba;
 // needs, 48 bytes per candidate chunk.
 extern "C" int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, const int32_t* chunk_fb,
                                 const int32_t* chunk_local, const int32_t* pair_off, int32_t* cnt,
-                                int32_t* seg_off, int32_t* tile_off, int32_t* seg_dest, int64_t S, int H, int K,
-                                int N, int F, int P, int cmax, int tile_rows, void* stream) {
-  if (!sel || !chunk_tok || !chunk_fb || !chunk_local || !pair_off || !cnt || !seg_off || !tile_off || !seg_dest)
+                                int32_t* seg_off, int32_t* tile_off, int32_t* seg_dest, int32_t* tile_seg,
+                                int64_t S, int H, int K, int N, int F, int P, int cmax, int tile_rows,
+                                int64_t hist_bound, void* stream) {
+  if (!sel || !chunk_tok || !chunk_fb || !chunk_local || !pair_off || !cnt || !seg_off || !tile_off || !seg_dest ||
+      !tile_seg)
     return MOBA_ERR_ARG;
+  if (hist_bound <= 0 || hist_bound >= 0x7fffffffLL) return MOBA_ERR_ARG;
   if (S <= 0 || H <= 0 || K <= 0 || N <= 0 || F <= 0 || P <= 0 || cmax <= 0 || tile_rows <= 0) return MOBA_ERR_ARG;
   if ((int64_t)S * H * (K + 1) >= 0x7fffffffLL || (int64_t)P * H >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
   if (H > 65535 || (size_t)cmax * 48 > 160 * 1024) return MOBA_ERR_LIMIT;
@@ -214,5 +226,7 @@ extern "C" int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, co
   hipLaunchKernelGGL(lists_segments_kernel, dim3((F * H + 1 + 255) / 256), dim3(256), 0, st, (const int*)cnt,
                      pair_off, seg_off, tile_off, F, H, tile_rows);
   hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(1024), 0, st, tile_off, F * H);
+  hipLaunchKernelGGL(lists_tile_seg_kernel, dim3((unsigned)((hist_bound + 255) / 256)), dim3(256), 0, st,
+                     (const int*)tile_off, tile_seg, F * H, (int)hist_bound);
   return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
 }

@@ -97,7 +97,7 @@ def topk_from_scores(scores: torch.Tensor, K: int) -> torch.Tensor:
 
 
 def build_lists(sel: torch.Tensor, plan: MobaPlan):
-    """(seg_off [F*H+1], tile_off [F*H+1], seg_dest [M]) int32 -- see csrc/lists.hip."""
+    """(seg_off [F*H+1], tile_off [F*H+1], seg_dest [M], tile_seg [tile bound]) int32 -- see csrc/lists.hip."""
     lib = _lib.load()
     S, H, K = sel.shape
     dev = sel.device
@@ -106,12 +106,14 @@ def build_lists(sel: torch.Tensor, plan: MobaPlan):
     seg_off = torch.empty(plan.F * H + 1, dtype=torch.int32, device=dev)
     tile_off = torch.empty(plan.F * H + 1, dtype=torch.int32, device=dev)
     seg_dest = torch.empty(max(M, 1), dtype=torch.int32, device=dev)
+    bound = plan.hist_tile_bound(H)
+    tile_seg = torch.empty(bound, dtype=torch.int32, device=dev)
     t = plan.tables
     _lib.check(lib.moba_build_lists(_ptr(sel), _ptr(t["chunk_tok"]), _ptr(t["chunk_fb"]), _ptr(t["chunk_local"]),
                                     _ptr(t["pair_off"]), _ptr(cnt), _ptr(seg_off), _ptr(tile_off), _ptr(seg_dest),
-                                    S, H, K, plan.N, plan.F, plan.P, plan.cmax, TILE_ROWS, _stream(dev)),
-               "moba_build_lists")
-    return seg_off, tile_off, seg_dest
+                                    _ptr(tile_seg), S, H, K, plan.N, plan.F, plan.P, plan.cmax, TILE_ROWS, bound,
+                                    _stream(dev)), "moba_build_lists")
+    return seg_off, tile_off, seg_dest, tile_seg
 
 
 class StageTimer:
@@ -159,14 +161,14 @@ def _forward(q, k, v, plan: MobaPlan, timer: Optional[StageTimer] = None):
     t = plan.tables
     span = (lambda name: timer.span(name, dev)) if timer is not None else (lambda name: _NoSpan())
     if plan.fallback:
-        sel = seg_off = tile_off = seg_dest = None
+        sel = seg_off = tile_off = seg_dest = tile_seg = None
     else:
         with span("chunk_mean"):
             kbar = chunk_mean(k, plan)
         with span("gate_topk"):
             sel = gate_topk(q, kbar, plan)
         with span("build_lists"):
-            seg_off, tile_off, seg_dest = build_lists(sel, plan)
+            seg_off, tile_off, seg_dest, tile_seg = build_lists(sel, plan)
     part_o = torch.empty((S * H * (K + 1), D), dtype=q.dtype, device=dev)
     part_lse = torch.empty((S * H * (K + 1),), dtype=torch.float32, device=dev)
     out = torch.empty_like(q)
@@ -174,17 +176,18 @@ def _forward(q, k, v, plan: MobaPlan, timer: Optional[StageTimer] = None):
     with span("fwd_partials"):
         _lib.check(lib.moba_fwd_partials(_ptr(q), _ptr(k), _ptr(v), _ptr(part_o), _ptr(part_lse), _ptr(seg_off),
                                          _ptr(tile_off), _ptr(seg_dest), _ptr(t.get("fchunk_tok")),
-                                         _ptr(t["chunk_tok"]), _ptr(t["self_tile_prefix"]), S, H, k.shape[1], D, K, plan.F,
+                                         _ptr(t["chunk_tok"]), _ptr(t["self_tile_prefix"]), _ptr(tile_seg),
+                                         _ptr(t["self_tile_chunk"]), S, H, k.shape[1], D, K, plan.F,
                                          plan.N,
                                          plan.chunk_size, plan.hist_tile_bound(H), plan.self_tiles, _dtype_code(q),
                                          _stream(dev)), "moba_fwd_partials")
     with span("fwd_merge"):
         _lib.check(lib.moba_fwd_merge(_ptr(part_o), _ptr(part_lse), _ptr(sel), _ptr(out), _ptr(lse), S, H, D, K,
                                       _dtype_code(q), _stream(dev)), "moba_fwd_merge")
-    return out, lse, sel, seg_off, tile_off, seg_dest
+    return out, lse, sel, seg_off, tile_off, seg_dest, tile_seg
 
 
-def _backward(dout, q, k, v, out, lse, sel, seg_off, tile_off, seg_dest, plan: MobaPlan):
+def _backward(dout, q, k, v, out, lse, sel, seg_off, tile_off, seg_dest, tile_seg, plan: MobaPlan):
     lib = _lib.load()
     S, H, D = q.shape
     dev = q.device
@@ -197,7 +200,8 @@ def _backward(dout, q, k, v, out, lse, sel, seg_off, tile_off, seg_dest, plan: M
     part_dq = torch.empty((S * H * (K + 1), D), dtype=torch.float32, device=dev)
     _lib.check(lib.moba_bwd(_ptr(dout), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(sel), _ptr(seg_off),
                             _ptr(tile_off), _ptr(seg_dest), _ptr(t.get("fchunk_tok")), _ptr(t["chunk_tok"]),
-                            _ptr(t["self_tile_prefix"]), _ptr(t.get("chunk_fid")),
+                            _ptr(t["self_tile_prefix"]), _ptr(tile_seg), _ptr(t["self_tile_chunk"]),
+                            _ptr(t.get("chunk_fid")),
                             _ptr(delta), _ptr(part_dq), _ptr(dq), _ptr(dk), _ptr(dv),
                             S, H, k.shape[1], D, K, plan.F, plan.N, plan.chunk_size, plan.hist_tile_bound(H),
                             plan.self_tiles,
@@ -210,9 +214,9 @@ class _MobaAttention(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q, k, v, plan, timer=None):
-        out, lse, sel, seg_off, tile_off, seg_dest = _forward(q, k, v, plan, timer)
+        out, lse, sel, seg_off, tile_off, seg_dest, tile_seg = _forward(q, k, v, plan, timer)
         ctx.plan = plan
-        ctx.aux = (sel, seg_off, tile_off, seg_dest)
+        ctx.aux = (sel, seg_off, tile_off, seg_dest, tile_seg)
         ctx.save_for_backward(q, k, v, out, lse)
         ctx.mark_non_differentiable(lse)
         return out, lse
@@ -220,8 +224,9 @@ class _MobaAttention(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dout, _dlse):
         q, k, v, out, lse = ctx.saved_tensors
-        sel, seg_off, tile_off, seg_dest = ctx.aux
-        dq, dk, dv = _backward(dout.contiguous(), q, k, v, out, lse, sel, seg_off, tile_off, seg_dest, ctx.plan)
+        sel, seg_off, tile_off, seg_dest, tile_seg = ctx.aux
+        dq, dk, dv = _backward(dout.contiguous(), q, k, v, out, lse, sel, seg_off, tile_off, seg_dest, tile_seg,
+                               ctx.plan)
         return dq, dk, dv, None, None
 
 

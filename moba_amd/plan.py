@@ -65,7 +65,8 @@ def _host_tables(cu: np.ndarray, B: int, topk: int):
     N = int(n_chunks.sum())
     tiles = (chunk_len + TILE_ROWS - 1) // TILE_ROWS
     self_tile_prefix = np.concatenate([[0], np.cumsum(tiles)])
-    out = dict(chunk_tok=chunk_tok, self_tile_prefix=self_tile_prefix)
+    out = dict(chunk_tok=chunk_tok, self_tile_prefix=self_tile_prefix,
+               self_tile_chunk=np.repeat(np.arange(N), tiles))
     info = dict(nseq=nseq, N=N, F=0 if fallback else F, k_eff=k_eff, fallback=fallback, K=0, P=0, cmax=0,
                 pairs_per_head=0, self_tiles=int(tiles.sum()))
     pairs_self = int((chunk_len.astype(np.int64) * (chunk_len + 1) // 2).sum())

@@ -97,7 +97,7 @@ def test_sampled_rows_and_invariants(lens, H, Hkv, B, topk):
     q, k, v, out = q.detach(), k.detach(), v.detach(), out.detach()
     kbar = E.chunk_mean(k, plan)
     sel = E.gate_topk(q, kbar, plan)
-    seg_off, tile_off, seg_dest = E.build_lists(sel, plan)
+    seg_off, tile_off, seg_dest, tile_seg = E.build_lists(sel, plan)
     torch.cuda.synchronize()
 
     # ---- selection invariants over every row (on the GPU) ----

@@ -98,7 +98,7 @@ def test_gather_lists(batch, seqlen, heads, B, topk):
     plan = _plan(cu, B, topk)
     kbar = O.chunk_mean(k, cu, B)
     sel = E.gate_topk(q.cuda(), kbar.cuda(), plan)
-    seg_off, tile_off, seg_dest = (x.cpu().numpy() for x in E.build_lists(sel, plan))
+    seg_off, tile_off, seg_dest, tile_seg = (x.cpu().numpy() for x in E.build_lists(sel, plan))
     sel = sel.cpu()
     counts, offs, rows, slots = O.gather_lists(sel, plan.F)
     H, K1 = heads, plan.K + 1
@@ -109,6 +109,10 @@ def test_gather_lists(batch, seqlen, heads, B, topk):
     assert np.array_equal(seg_dest[:offs[-1]], want_dest)
     tiles = (counts + 127) // 128
     assert np.array_equal(tile_off, np.concatenate([[0], np.cumsum(tiles)]))
+    # every history tile id names its segment; ids past the last tile are marked
+    want_seg = np.repeat(np.arange(plan.F * H), tiles)
+    assert tile_seg.size == plan.hist_tile_bound(H) >= want_seg.size
+    assert np.array_equal(tile_seg[:want_seg.size], want_seg) and (tile_seg[want_seg.size:] == -1).all()
 
 
 # ------------------------------------------------------------------ forward
