@@ -364,42 +364,54 @@ __global__ __launch_bounds__(256) void moba_merge_kernel(const typename E::elem*
                                                          const int* __restrict__ sel, typename E::elem* __restrict__ out,
                                                          float* __restrict__ lse, int64_t rows, int K1) {
   MOBA_ELEM_TYPES(E)
-  const int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
-  if (row >= rows) return;
+  const int64_t row_raw = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+  const bool row_ok = row_raw < rows;
+  const int64_t row = row_ok ? row_raw : rows - 1;  // whole 16-lane groups stay active for the shuffles
   const int c8 = threadIdx.x & 15;
   const int K = K1 - 1;
   const float* pl = part_lse + row * K1;
   const int* ps = sel + row * K;
-  // absent slots are redirected to slot 0 with weight 0, so every load below is
-  // unconditional and the loads of a group of four slots are in flight together
-  float mx = pl[0];
-  for (int j = 0; j < K; ++j) {
-    const float l = pl[1 + j];
-    mx = ps[j] >= 0 ? fmaxf(mx, l) : mx;
+  const elem* po = part_o + row * K1 * kHeadDim + c8 * 8;
+  // Lane c8 of the row's group fetches the LSE and the presence of slot j0 + c8, so the slot
+  // statistics cost one round trip per 16 slots; weights travel by lane shuffles.  Absent slots
+  // are redirected to slot 0 with weight 0, so the partial-output loads are unconditional and
+  // eight of them are in flight together.  Slots are accumulated in ascending order.
+  float mx = -INFINITY;
+  for (int j0 = 0; j0 < K1; j0 += 16) {
+    const int j = j0 + c8;
+    const bool ok = j < K1 && (j == 0 || ps[j - 1] >= 0);
+    const float l = ok ? pl[j] : -INFINITY;
+    mx = fmaxf(mx, l);
   }
+#pragma unroll
+  for (int o = 8; o >= 1; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 16));
   float acc[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.f;
   float wsum = 0.f;
-  const elem* po = part_o + row * K1 * kHeadDim + c8 * 8;
-  for (int j0 = 0; j0 < K1; j0 += 4) {
-    elem8 x[4];
-    float w[4];
+  for (int j0 = 0; j0 < K1; j0 += 16) {
+    const int j = j0 + c8;
+    const bool ok = j < K1 && (j == 0 || ps[j - 1] >= 0);
+    const float wl = ok ? fast_exp2(pl[j] - mx) : 0.f;
+    const int nslot = min(16, K1 - j0);
+    for (int u0 = 0; u0 < nslot; u0 += 8) {
+      elem8 x[8];
+      float w[8];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int j = j0 + u;
-      const bool ok = j < K1 && (j == 0 || ps[j < K1 ? j - 1 : 0] >= 0);
-      const int jj = ok ? j : 0;
-      x[u] = __builtin_nontemporal_load(reinterpret_cast<const elem8*>(po + (int64_t)jj * kHeadDim));
-      w[u] = ok ? fast_exp2(pl[jj] - mx) : 0.f;
-    }
+      for (int u = 0; u < 8; ++u) {
+        w[u] = __shfl(wl, u0 + u, 16);           // 0 for slots past K1 too (their lanes computed ok = false)
+        const int jj = w[u] > 0.f ? j0 + u0 + u : 0;
+        x[u] = __builtin_nontemporal_load(reinterpret_cast<const elem8*>(po + (int64_t)jj * kHeadDim));
+      }
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      wsum += w[u];
+      for (int u = 0; u < 8; ++u) {
+        wsum += w[u];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc[e] += w[u] * (float)x[u][e];
+        for (int e = 0; e < 8; ++e) acc[e] += w[u] * (float)x[u][e];
+      }
     }
   }
+  if (!row_ok) return;
   const float inv = 1.f / wsum;
   elem8 o;
 #pragma unroll
