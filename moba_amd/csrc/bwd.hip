@@ -257,8 +257,9 @@ __global__ __launch_bounds__(256) void bwd_dq_reduce_kernel(const float* __restr
                                                             typename E::elem* __restrict__ dq, int64_t rows, int K1,
                                                             float scale) {
   MOBA_ELEM_TYPES(E)
-  const int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
-  if (row >= rows) return;
+  const int64_t row_raw = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+  const bool row_ok = row_raw < rows;
+  const int64_t row = row_ok ? row_raw : rows - 1;  // whole 16-lane groups stay active for the shuffles
   const int c8 = threadIdx.x & 15;
   const int K = K1 - 1;
   const int* ps = sel + row * K;
@@ -266,13 +267,36 @@ __global__ __launch_bounds__(256) void bwd_dq_reduce_kernel(const float* __restr
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.f;
   const float* src = part_dq + row * K1 * kHeadDim + c8 * 8;
-  for (int j = 0; j < K1; ++j) {
-    if (j > 0 && ps[j - 1] < 0) continue;
-    const f32x4 a = *reinterpret_cast<const f32x4*>(src + (int64_t)j * kHeadDim);
-    const f32x4 b = *reinterpret_cast<const f32x4*>(src + (int64_t)j * kHeadDim + 4);
+  // lane c8 fetches the presence of slot j0 + c8; absent slots are redirected to slot 0 and
+  // multiplied by 0, so the loads of four slots are unconditional and in flight together
+  for (int j0 = 0; j0 < K1; j0 += 16) {
+    const int j = j0 + c8;
+    const float present = (j < K1 && (j == 0 || ps[j - 1] >= 0)) ? 1.f : 0.f;
+    const int nslot = min(16, K1 - j0);
+    for (int u0 = 0; u0 < nslot; u0 += 4) {
+      f32x4 a[4], b[4];
+      float w[4];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) { acc[e] += a[e]; acc[4 + e] += b[e]; }
+      for (int u = 0; u < 4; ++u) {
+        w[u] = __shfl(present, u0 + u, 16);
+        const int jj = w[u] > 0.f ? j0 + u0 + u : 0;
+        if (u0 + u < nslot) {  // uniform: no loads for slots that do not exist
+          a[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(src + (int64_t)jj * kHeadDim));
+          b[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(src + (int64_t)jj * kHeadDim + 4));
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        if (u0 + u >= nslot) break;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          acc[e] += w[u] * a[u][e];
+          acc[4 + e] += w[u] * b[u][e];
+        }
+      }
+    }
   }
+  if (!row_ok) return;
   elem8 o;
 #pragma unroll
   for (int e = 0; e < 8; ++e) o[e] = (elem)(acc[e] * scale);

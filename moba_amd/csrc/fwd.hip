@@ -401,10 +401,12 @@ __global__ __launch_bounds__(256) void moba_merge_kernel(const typename E::elem*
       for (int u = 0; u < 8; ++u) {
         w[u] = __shfl(wl, u0 + u, 16);           // 0 for slots past K1 too (their lanes computed ok = false)
         const int jj = w[u] > 0.f ? j0 + u0 + u : 0;
-        x[u] = __builtin_nontemporal_load(reinterpret_cast<const elem8*>(po + (int64_t)jj * kHeadDim));
+        if (u0 + u < nslot)                      // uniform: no loads for slots that do not exist
+          x[u] = __builtin_nontemporal_load(reinterpret_cast<const elem8*>(po + (int64_t)jj * kHeadDim));
       }
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
+        if (u0 + u >= nslot) break;
         wsum += w[u];
 #pragma unroll
         for (int e = 0; e < 8; ++e) acc[e] += w[u] * (float)x[u][e];
