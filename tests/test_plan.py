@@ -36,6 +36,10 @@ def test_plan_tables_match_oracle(seed):
     assert plan.flops_per_head * 128 == pytest.approx(O.attention_flops(cu, B, topk, 1, 128))
     lens = np.diff(m["cu_chunk"])
     assert plan.self_tiles == int(((lens + TILE_ROWS - 1) // TILE_ROWS).sum())
+    # every per-head self tile names its chunk: prefix[c] <= t < prefix[c+1]
+    stc, pre = plan.host["self_tile_chunk"], plan.host["self_tile_prefix"]
+    assert stc.size == plan.self_tiles
+    assert all(pre[c] <= t < pre[c + 1] for t, c in enumerate(stc.tolist()))
 
 
 def test_plan_headline_config_sizes():

@@ -82,6 +82,34 @@ def test_moba_layer_prefill_calls_impl_with_reference_arguments():
     assert out.reshape(b, s, -1).shape == (b, s, hq * d)
 
 
+def test_moba_layer_hands_grouped_heads_to_an_impl_that_takes_them():
+    """An implementation that advertises a grouped-query variant receives k, v with their own
+    head count (no repeat_interleave copies); the result layout is unchanged."""
+    from moba_amd import MoBAConfig, moba_attn_varlen, moba_attn_varlen_gqa
+    from moba_amd.wrapper import moba_layer
+
+    assert moba_attn_varlen.grouped_query_impl is moba_attn_varlen_gqa
+    seen = {}
+
+    def impl(q, k, v, cu_seqlens, max_seqlen, moba_chunk_size, moba_topk):
+        raise AssertionError("the grouped variant must be called")
+
+    def grouped(q, k, v, cu_seqlens, max_seqlen, moba_chunk_size, moba_topk):
+        seen.update(k=k, v=v)
+        return q
+
+    impl.grouped_query_impl = grouped
+
+    class Mod(torch.nn.Module):
+        is_causal = True
+
+    b, hq, hkv, s, d = 2, 4, 2, 6, 8
+    query, key, value = torch.randn(b, hq, s, d), torch.randn(b, hkv, s, d), torch.randn(b, hkv, s, d)
+    out, _ = moba_layer(impl, MoBAConfig(4, 3), Mod(), query, key, value, None)
+    assert out.shape == (b * s, hq, d)
+    assert seen["k"].shape == (b * s, hkv, d) and torch.equal(seen["k"][1 * s + 2, 1], key[1, 1, 2])
+
+
 def test_moba_layer_decode_is_full_attention():
     from moba_amd import MoBAConfig
     from moba_amd.wrapper import moba_layer
