@@ -215,7 +215,7 @@ extern "C" int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, co
   if (hist_bound <= 0 || hist_bound >= 0x7fffffffLL) return MOBA_ERR_ARG;
   if (S <= 0 || H <= 0 || K <= 0 || N <= 0 || F <= 0 || P <= 0 || cmax <= 0 || tile_rows <= 0) return MOBA_ERR_ARG;
   if ((int64_t)S * H * (K + 1) >= 0x7fffffffLL || (int64_t)P * H >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
-  if (H > 65535 || (size_t)cmax * 48 > 160 * 1024) return MOBA_ERR_LIMIT;
+  if (H > 65535 || (size_t)cmax * 48 > 64 * 1024) return MOBA_ERR_LIMIT;
   hipStream_t st = (hipStream_t)stream;
   dim3 grid(N, H);
   hipLaunchKernelGGL(lists_count_kernel, grid, dim3(256), (size_t)cmax * 4, st, sel, chunk_tok, chunk_fb,
