@@ -19,7 +19,7 @@ MAX_ABS, MEAN_ABS = 2e-2, 2e-3
 REF_MAX_ABS, REF_MEAN_ABS = 4e-2, 4e-4
 
 
-def run_case(batch, seqlen, heads, B, topk, seed=0, check_grad=True, dtype=torch.bfloat16):
+def run_case(batch, seqlen, heads, B, topk, seed=0, check_grad=True, dtype=torch.bfloat16, ref_bounds=True):
     from moba_amd import moba_efficient as E
     from moba_amd.plan import make_plan
 
@@ -55,13 +55,18 @@ def run_case(batch, seqlen, heads, B, topk, seed=0, check_grad=True, dtype=torch
     assert err.max() < MAX_ABS and err.mean() < MEAN_ABS, ("out", err.max().item(), err.mean().item())
     # the reference test compares two bf16 outputs (moba_naive returns o.type_as(q)): round the oracle likewise
     err16 = (out.detach().cpu().float() - ref.detach().to(dtype).float()).abs()
-    assert err16.max() < REF_MAX_ABS and err16.mean() < REF_MEAN_ABS, ("out16", err16.max().item(), err16.mean().item())
+    # (those bounds belong to the reference's grid, where every row averages hundreds of keys)
+    if ref_bounds:
+        assert err16.max() < REF_MAX_ABS and err16.mean() < REF_MEAN_ABS, ("out16", err16.max().item(), err16.mean().item())
     if check_grad:
         ref.backward(do.float())
         got_g = torch.stack([qg.grad.cpu().float(), kg.grad.cpu().float(), vg.grad.cpu().float()], dim=1)
         ref_g = torch.stack([qc.grad, kc.grad, vc.grad], dim=1)
         gerr = (got_g - ref_g).abs()
-        assert gerr.max() < REF_MAX_ABS and gerr.mean() < REF_MEAN_ABS, ("grad", gerr.max().item(), gerr.mean().item())
+        if ref_bounds:
+            assert gerr.max() < REF_MAX_ABS and gerr.mean() < REF_MEAN_ABS, ("grad", gerr.max().item(), gerr.mean().item())
+        else:
+            assert gerr.mean() < MEAN_ABS, ("grad", gerr.mean().item())
         # per-tensor, relative to the tensor's scale
         for i, name in enumerate(("dq", "dk", "dv")):
             e = gerr[:, i]
@@ -139,6 +144,22 @@ def test_grouped_query(batch, seqlen, heads, kv_heads, B, topk, dtype):
         assert err.mean() <= 4e-3 * want.abs().mean() + 1e-6, (err.mean().item(), want.abs().mean().item())
     with pytest.raises(ValueError):
         moba_attn_varlen(qa, ka, va, cu_t, mx, B, topk)       # the 7-argument operator keeps the reference's contract
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_shapes(seed):
+    """Seeded random shapes: odd sequence lengths, chunk sizes that divide nothing, one to many
+    sequences, both dtypes; forward and backward against the oracle."""
+    rng = np.random.default_rng(100 + seed)
+    for _ in range(8):
+        seqlen = int(rng.integers(40, 3000))
+        batch = int(rng.integers(1, min(9, seqlen // 4)))
+        heads = int(rng.integers(1, 6))
+        B = int(rng.integers(8, 300))
+        topk = int(rng.integers(1, 9))
+        dtype = torch.float16 if rng.integers(0, 2) else torch.bfloat16
+        print("random case", batch, seqlen, heads, B, topk, dtype, flush=True)
+        run_case(batch, seqlen, heads, B, topk, seed=int(rng.integers(0, 1000)), dtype=dtype, ref_bounds=False)
 
 
 def test_one_token_sequences():
