@@ -263,6 +263,9 @@ def moba_attn_varlen_gqa(q, k, v, cu_seqlens, max_seqlen, moba_chunk_size, moba_
 
 # lets moba_layer skip the key/value head expansion when it drives this operator
 moba_attn_varlen.grouped_query_impl = moba_attn_varlen_gqa
+# ... and tells it that make_plan(host_lengths=...) spares the device-to-host read of cu_seqlens
+moba_attn_varlen.takes_host_lengths = True
+moba_attn_varlen_gqa.takes_host_lengths = True
 
 
 def moba_attn_varlen_with_lse(q, k, v, cu_seqlens, max_seqlen, moba_chunk_size, moba_topk, timer=None, gqa=False):

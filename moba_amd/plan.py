@@ -4,12 +4,13 @@ Counterpart of ``calc_chunks`` (moba/moba_efficient.py:14-64) plus everything el
 that depends only on the sequence lengths: buffer sizes, tile counts and the small
 int32 tables the kernels index.  All sizes are data independent (a token in the c-th
 chunk of its sequence selects exactly min(k, c) history chunks), so one device-to-host
-read of ``cu_seqlens`` is the only synchronisation of a forward call; plans are cached
-per (tensor identity, tensor version, chunk size, top-k).
+read of ``cu_seqlens`` is the only synchronisation of a forward call, and a caller that
+knows the lengths on the host (the transformers adapter does) avoids even that.
 """
 
 from __future__ import annotations
 
+from collections import OrderedDict
 from dataclasses import dataclass, field
 from typing import Dict, List, Tuple
 
@@ -92,34 +93,44 @@ def _host_tables(cu: np.ndarray, B: int, topk: int):
     return out, info
 
 
-_CACHE: Dict[Tuple, MobaPlan] = {}
+# Plans are cached two ways.  By value: (lengths, chunk size, top-k, device) -> plan, so equal
+# batches share tables whatever tensor describes them.  By tensor: (id, version) of a device
+# cu_seqlens tensor -> plan, which saves the device-to-host read on later calls; the entry keeps the
+# tensor alive, so its id cannot be reused by another tensor while the entry exists (the reference
+# memoises on tensor identity too, moba/moba_efficient.py:14, and is stale after an in-place update;
+# the version number closes that hole here).
+_BY_VALUE: "OrderedDict[Tuple, MobaPlan]" = OrderedDict()
+_BY_TENSOR: "OrderedDict[Tuple, Tuple[MobaPlan, torch.Tensor]]" = OrderedDict()
+_CACHE_SIZE = 16
 
 
-def make_plan(cu_seqlens, chunk_size: int, moba_topk: int, device=None) -> MobaPlan:
-    """Build (or fetch) the plan for a batch.  ``cu_seqlens`` may be a device tensor (read
-    once, then cached on identity + version) or a Python sequence."""
-    key = None
-    if torch.is_tensor(cu_seqlens):
-        device = cu_seqlens.device if device is None else device
-        key = (cu_seqlens.data_ptr(), cu_seqlens._version, cu_seqlens.numel(), str(device), chunk_size, moba_topk)
-        hit = _CACHE.get(key)
-        if hit is not None:
-            return hit
-        cu = cu_seqlens.detach().to("cpu", torch.int64).numpy()
-    else:
-        cu = np.asarray(list(cu_seqlens), dtype=np.int64)
+def _remember(cache, key, value):
+    cache[key] = value
+    cache.move_to_end(key)
+    while len(cache) > _CACHE_SIZE:
+        cache.popitem(last=False)
+
+
+def _build(cu: np.ndarray, chunk_size: int, moba_topk: int, device) -> MobaPlan:
     if cu.ndim != 1 or cu.size < 2:
         raise ValueError("cu_seqlens must be a 1-D tensor with at least two entries")
     if cu[0] != 0 or (np.diff(cu) <= 0).any():
         raise ValueError("cu_seqlens must start at 0 and be strictly increasing (zero-length sequences are unsupported)")
     if chunk_size <= 0 or moba_topk <= 0:
         raise ValueError("moba_chunk_size and moba_topk must be positive")
+    on_device = device is not None and torch.device(device).type != "cpu"
+    vkey = (cu.tobytes(), int(chunk_size), int(moba_topk), str(device) if on_device else None)
+    hit = _BY_VALUE.get(vkey)
+    if hit is not None:
+        _BY_VALUE.move_to_end(vkey)
+        return hit
     host, info = _host_tables(cu, int(chunk_size), int(moba_topk))
+    host["cu_seqlens"] = cu  # the kernels read the plan's own copy, never the caller's tensor
     plan = MobaPlan(cu=cu.tolist(), chunk_size=int(chunk_size), moba_topk=int(moba_topk), S=int(cu[-1]),
                     nseq=info["nseq"], N=info["N"], F=info["F"], k_eff=info["k_eff"], K=info["K"],
                     fallback=info["fallback"], P=info["P"], cmax=info["cmax"], pairs_per_head=info["pairs_per_head"],
                     self_tiles=info["self_tiles"], flops_per_head=info["flops_per_head_per_d"], host=host)
-    if device is not None and torch.device(device).type != "cpu":
+    if on_device:
         names = list(host)
         flat = np.concatenate([host[n_].astype(np.int32) for n_ in names])
         dev = torch.from_numpy(flat).to(device)
@@ -127,12 +138,26 @@ def make_plan(cu_seqlens, chunk_size: int, moba_topk: int, device=None) -> MobaP
         for n_ in names:
             plan.tables[n_] = dev[off:off + host[n_].size]
             off += host[n_].size
-        if torch.is_tensor(cu_seqlens) and cu_seqlens.dtype == torch.int32 and cu_seqlens.is_contiguous():
-            plan.tables["cu_seqlens"] = cu_seqlens
-        else:
-            plan.tables["cu_seqlens"] = torch.from_numpy(cu.astype(np.int32)).to(device)
-    if key is not None:
-        if len(_CACHE) >= 16:
-            _CACHE.pop(next(iter(_CACHE)))
-        _CACHE[key] = plan
+    _remember(_BY_VALUE, vkey, plan)
+    return plan
+
+
+def make_plan(cu_seqlens, chunk_size: int, moba_topk: int, device=None, host_lengths=None) -> MobaPlan:
+    """Build (or fetch) the plan for a batch.  ``cu_seqlens`` may be a device tensor (read once, then
+    remembered for that tensor and version) or a Python sequence.  ``host_lengths`` is an optional host
+    copy of a device ``cu_seqlens`` supplied by a caller that built it: no device-to-host read happens."""
+    if not torch.is_tensor(cu_seqlens):
+        return _build(np.asarray(list(cu_seqlens), dtype=np.int64), chunk_size, moba_topk, device)
+    device = cu_seqlens.device if device is None else device
+    tkey = (id(cu_seqlens), cu_seqlens._version, str(device), int(chunk_size), int(moba_topk))
+    hit = _BY_TENSOR.get(tkey)
+    if hit is not None and hit[1] is cu_seqlens:
+        _BY_TENSOR.move_to_end(tkey)
+        return hit[0]
+    if host_lengths is not None:
+        cu = np.asarray(list(host_lengths), dtype=np.int64)
+    else:
+        cu = cu_seqlens.detach().to("cpu", torch.int64).numpy()
+    plan = _build(cu, chunk_size, moba_topk, device)
+    _remember(_BY_TENSOR, tkey, (plan, cu_seqlens))
     return plan

@@ -15,6 +15,22 @@ import torch.nn.functional as F
 from .config import MoBAConfig
 
 
+_CU_SEQLENS = {}  # (batch, seq_len, device) -> int32 tensor of multiples of seq_len
+
+
+def _cu_seqlens_for(batch: int, seq_len: int, device) -> torch.Tensor:
+    """cu_seqlens of `batch` sequences of `seq_len` tokens; one tensor per shape, so that an operator
+    which remembers the batch layout per tensor recognises it on every layer and step."""
+    key = (batch, seq_len, str(device))
+    t = _CU_SEQLENS.get(key)
+    if t is None:
+        if len(_CU_SEQLENS) >= 16:
+            _CU_SEQLENS.pop(next(iter(_CU_SEQLENS)))
+        t = torch.arange(0, (batch + 1) * seq_len, seq_len, dtype=torch.int32, device=device)
+        _CU_SEQLENS[key] = t
+    return t
+
+
 def hf_to_fa(x: torch.Tensor) -> torch.Tensor:
     """[batch, heads, seqlen, head_dim] -> [batch * seqlen, heads, head_dim] (moba/wrapper.py:7-15)."""
     b, h, s, d = x.shape
@@ -64,7 +80,12 @@ def moba_layer(
             else:
                 k = torch.repeat_interleave(k, rep, dim=1)
                 v = torch.repeat_interleave(v, rep, dim=1)
-        cu_seqlens = torch.arange(0, (batch + 1) * kv_len, kv_len, dtype=torch.int32, device=query.device)
+        cu_seqlens = _cu_seqlens_for(batch, kv_len, query.device)
+        if getattr(moba_impl, "takes_host_lengths", False):
+            # the lengths are known here on the host: spare the operator its device-to-host read
+            from .plan import make_plan
+            make_plan(cu_seqlens, moba_config.moba_chunk_size, moba_config.moba_topk,
+                      host_lengths=range(0, (batch + 1) * kv_len, kv_len))
         out = moba_impl(
             q=q,
             k=k,

@@ -54,3 +54,21 @@ def test_plan_rejects_bad_input():
         make_plan([0, 5, 5, 9], 4, 3)
     with pytest.raises(ValueError):
         make_plan([1, 5], 4, 3)
+
+
+def test_plan_cache_follows_the_tensor_contents():
+    import torch
+    cu = torch.tensor([0, 100, 260], dtype=torch.int32)
+    a = make_plan(cu, 32, 3)
+    assert make_plan(cu, 32, 3) is a                      # same tensor, same version
+    assert make_plan(cu.clone(), 32, 3) is a              # equal lengths share one plan
+    assert make_plan([0, 100, 260], 32, 3) is a
+    cu[1] = 120                                           # in-place update: the version changes
+    b = make_plan(cu, 32, 3)
+    assert b is not a and b.cu == [0, 120, 260] and a.cu == [0, 100, 260]
+    assert b.host["cu_seqlens"].tolist() == [0, 120, 260]
+    # a host copy supplied by the caller is used instead of reading the tensor
+    c = make_plan(torch.tensor([0, 7, 9], dtype=torch.int32), 4, 2, host_lengths=[0, 7, 9])
+    assert c.cu == [0, 7, 9]
+    # different chunk size or top-k: different plan
+    assert make_plan(cu, 16, 3) is not b and make_plan(cu, 32, 2) is not b
