@@ -225,7 +225,7 @@ class _MobaAttention(torch.autograd.Function):
     def backward(ctx, dout, _dlse):
         q, k, v, out, lse = ctx.saved_tensors
         sel, seg_off, tile_off, seg_dest, tile_seg = ctx.aux
-        dq, dk, dv = _backward(dout.contiguous(), q, k, v, out, lse, sel, seg_off, tile_off, seg_dest, tile_seg,
+        dq, dk, dv = _backward(dout.to(q.dtype).contiguous(), q, k, v, out, lse, sel, seg_off, tile_off, seg_dest, tile_seg,
                                ctx.plan)
         return dq, dk, dv, None, None
 
