@@ -107,21 +107,38 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams<E> p) {
   const uint32_t lds_base = lds_addr(smem);
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   const int ld_kin = lane >> 4, ld_pc = lane & 15;
-  auto issue_tile = [&](int kt, int buf) {
+  uint32_t ld_off[4];  // per-lane byte offset of its 16 bytes inside a full tile (slab 4*i + wave)
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int key = 4 * (4 * i + wave_u) + ld_kin;
+    ld_off[i] = (uint32_t)(key * row_bytes + sw_col16(key, ld_pc) * 16);
+  }
+  const char* k_head = (const char*)p.k + (int64_t)kv_tok0 * row_bytes + hkv * (kHeadDim * 2);
+  const char* v_head = (const char*)p.v + (int64_t)kv_tok0 * row_bytes + hkv * (kHeadDim * 2);
+  auto issue_tile = [&](int kt, int buf) __attribute__((always_inline)) {
     const uint32_t kdst = lds_base + buf * kTileBytes;
     const uint32_t vdst = lds_base + (2 + buf) * kTileBytes;
     const int key0 = kt * TN;
     const bool full = (key0 + TN <= nkeys) && (kv_tok0 + key0 + TN <= p.t.S);
+    if (full) {  // uniform tile base in SGPRs + constant per-lane offsets: no address arithmetic
+      const char* kb_ = k_head + (int64_t)key0 * row_bytes;
+      const char* vb_ = v_head + (int64_t)key0 * row_bytes;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int slab = 4 * i + wave_u;
-      const int key = 4 * slab + ld_kin;
-      const int c16 = sw_col16(key, ld_pc);
-      int64_t tk = kv_tok0 + key0 + key;
-      if (!full) tk = min(tk, (int64_t)p.t.S - 1);
-      const int64_t off = tk * row_bytes + hkv * (kHeadDim * 2) + c16 * 16;
-      async_copy16((const char*)p.k + off, kdst + slab * 1024);
-      async_copy16((const char*)p.v + off, vdst + slab * 1024);
+      for (int i = 0; i < 4; ++i) {
+        async_copy16_sv(kb_, ld_off[i], kdst + (4 * i + wave_u) * 1024);
+        async_copy16_sv(vb_, ld_off[i], vdst + (4 * i + wave_u) * 1024);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int slab = 4 * i + wave_u;
+        const int key = 4 * slab + ld_kin;
+        const int c16 = sw_col16(key, ld_pc);
+        const int64_t tk = min((int64_t)kv_tok0 + key0 + key, (int64_t)p.t.S - 1);
+        const int64_t off = tk * row_bytes + hkv * (kHeadDim * 2) + c16 * 16;
+        async_copy16((const char*)p.k + off, kdst + slab * 1024);
+        async_copy16((const char*)p.v + off, vdst + slab * 1024);
+      }
     }
   };
   // rows past the key range are multiplied by dS = 0: clear them so that no NaN can form
@@ -142,9 +159,13 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams<E> p) {
   };
 
   const int nkt = (nkeys + TN - 1) / TN;
-  issue_tile(0, 0);
+  // history tiles may visit their key tiles in any order: co-resident tiles of one chunk start
+  // at different key tiles so that they do not all ask for the same lines at the same time
+  const int rot = t.rot % nkt;
+  auto key_tile = [&](int it) __attribute__((always_inline)) { const int x = it + rot; return x >= nkt ? x - nkt : x; };
+  issue_tile(key_tile(0), 0);
   wait_vmem();
-  scrub_tile(0, 0);
+  scrub_tile(key_tile(0), 0);
   __syncthreads();
 
   f32x16 dqacc[4];
@@ -160,10 +181,11 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams<E> p) {
   const int tr_c16 = 2 * (g16 & 1) + (i1 >> 1);
   const int tr_sub = (i1 & 1) * 8;
 
-  for (int kt = 0; kt < nkt; ++kt) {
-    const int buf = kt & 1;
-    const bool has_next = kt + 1 < nkt;
-    if (has_next) issue_tile(kt + 1, buf ^ 1);
+  for (int it = 0; it < nkt; ++it) {
+    const int kt = key_tile(it);
+    const int buf = it & 1;
+    const bool has_next = it + 1 < nkt;
+    if (has_next) issue_tile(key_tile(it + 1), buf ^ 1);
 
     if (kt * TN <= t.wave_max_limit) {
       const char* ks = smem + buf * kTileBytes;
@@ -231,7 +253,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams<E> p) {
     }
     if (has_next) {
       wait_vmem();
-      scrub_tile(kt + 1, buf ^ 1);
+      scrub_tile(key_tile(it + 1), buf ^ 1);
     }
     __syncthreads();
   }
