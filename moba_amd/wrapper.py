@@ -81,10 +81,16 @@ def moba_layer(
                 k = torch.repeat_interleave(k, rep, dim=1)
                 v = torch.repeat_interleave(v, rep, dim=1)
         cu_seqlens = _cu_seqlens_for(batch, kv_len, query.device)
+        chunk_size = moba_config.moba_chunk_size
+        num_layers = getattr(getattr(module, "config", None), "num_hidden_layers", None)
+        if moba_config.is_full_attention_layer(getattr(module, "layer_idx", None), num_layers):
+            # one chunk per sequence: no history chunks, and every implementation of the operator then
+            # computes plain causal attention (moba/moba_efficient.py:313-321, moba/moba_naive.py:58-81)
+            chunk_size = max(chunk_size, kv_len)
         if getattr(moba_impl, "takes_host_lengths", False):
             # the lengths are known here on the host: spare the operator its device-to-host read
             from .plan import make_plan
-            make_plan(cu_seqlens, moba_config.moba_chunk_size, moba_config.moba_topk,
+            make_plan(cu_seqlens, chunk_size, moba_config.moba_topk,
                       host_lengths=range(0, (batch + 1) * kv_len, kv_len))
         out = moba_impl(
             q=q,
@@ -92,7 +98,7 @@ def moba_layer(
             v=v,
             cu_seqlens=cu_seqlens,
             max_seqlen=kv_len,
-            moba_chunk_size=moba_config.moba_chunk_size,
+            moba_chunk_size=chunk_size,
             moba_topk=moba_config.moba_topk,
         )
     else:

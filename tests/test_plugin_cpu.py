@@ -110,6 +110,42 @@ def test_moba_layer_hands_grouped_heads_to_an_impl_that_takes_them():
     assert seen["k"].shape == (b * s, hkv, d) and torch.equal(seen["k"][1 * s + 2, 1], key[1, 1, 2])
 
 
+def test_full_attention_layers_switch():
+    """Layers named in full_attention_layers get one chunk per sequence (= causal attention in every
+    implementation); the others keep the configured chunk size.  Negative indices count from the end."""
+    from types import SimpleNamespace
+    from moba_amd import MoBAConfig
+    from moba_amd.moba_naive import moba_attn_varlen_naive
+    from moba_amd.wrapper import moba_layer
+
+    cfg = MoBAConfig(4, 2, full_attention_layers=[0, -1])
+    assert cfg.is_full_attention_layer(0, 6) and cfg.is_full_attention_layer(5, 6)
+    assert not cfg.is_full_attention_layer(3, 6) and not MoBAConfig(4, 2).is_full_attention_layer(0, 6)
+    seen = []
+
+    def impl(q, k, v, cu_seqlens, max_seqlen, moba_chunk_size, moba_topk):
+        seen.append(moba_chunk_size)
+        return moba_attn_varlen_naive(q, k, v, cu_seqlens, max_seqlen, moba_chunk_size, moba_topk)
+
+    class Mod(torch.nn.Module):
+        is_causal = True
+
+        def __init__(self, idx):
+            super().__init__()
+            self.layer_idx = idx
+            self.config = SimpleNamespace(num_hidden_layers=6)
+
+    b, h, s, d = 1, 2, 24, 8
+    query, key, value = torch.randn(b, h, s, d), torch.randn(b, h, s, d), torch.randn(b, h, s, d)
+    full, _ = moba_layer(impl, cfg, Mod(5), query, key, value, None)
+    sparse, _ = moba_layer(impl, cfg, Mod(2), query, key, value, None)
+    assert seen == [24, 4]
+    mask = torch.tril(torch.ones(s, s, dtype=torch.bool))
+    ref = torch.softmax((query @ key.transpose(-1, -2) / d ** 0.5).masked_fill(~mask, float("-inf")), -1) @ value
+    torch.testing.assert_close(full.view(b, s, h, d).transpose(1, 2), ref, atol=1e-5, rtol=1e-5)
+    assert not torch.allclose(sparse.view(b, s, h, d).transpose(1, 2), ref, atol=1e-3)
+
+
 def test_moba_layer_decode_is_full_attention():
     from moba_amd import MoBAConfig
     from moba_amd.wrapper import moba_layer
