@@ -162,6 +162,51 @@ def test_random_shapes(seed):
         run_case(batch, seqlen, heads, B, topk, seed=int(rng.integers(0, 1000)), dtype=dtype, ref_bounds=False)
 
 
+def test_peaked_softmax_and_exact_gate_ties():
+    """(a) Scores with a large spread (q, k scaled by 6: near one-hot softmax, running max far from
+    the first tile's) stay within the tolerances.  (b) Keys that repeat with the chunk period give
+    every chunk the same representative, hence exactly tied gate scores: the tie rule (lower chunk
+    id) must then pick the same chunks as the oracle, bit for bit."""
+    from moba_amd import moba_efficient as E
+    from moba_amd.plan import make_plan
+    q, k, v, do, cu, mx = make_case(2, 2048, 2, seed=21)
+    q, k = (q.float() * 6).to(torch.bfloat16), (k.float() * 6).to(torch.bfloat16)
+    cu_t = torch.tensor(cu, dtype=torch.int32, device="cuda")
+    B, topk = 128, 4
+    qg, kg, vg = (x.cuda().requires_grad_(True) for x in (q, k, v))
+    out = E.moba_attn_varlen(qg, kg, vg, cu_t, mx, B, topk)
+    out.backward(do.cuda())
+    plan = make_plan(cu_t, B, topk)
+    sel = E.gate_topk(qg.detach(), E.chunk_mean(kg.detach(), plan), plan).cpu()
+    qc, kc, vc = (x.clone().requires_grad_(True) for x in (q, k, v))
+    ref = O.moba_attn_varlen_oracle(qc, kc, vc, cu, mx, B, topk, sel=sel)
+    ref.backward(do.float())
+    assert torch.isfinite(out.float()).all() and torch.isfinite(qg.grad.float()).all()
+    err = (out.detach().cpu().float() - ref.detach().float()).abs()
+    assert err.max() < 3e-2 and err.mean() < MEAN_ABS, (err.max().item(), err.mean().item())
+    for a, b in ((qg.grad, qc.grad), (kg.grad, kc.grad), (vg.grad, vc.grad)):
+        e = (a.cpu().float() - b.float()).abs()
+        assert e.max() < 3e-2 * b.float().abs().max().clamp_min(1.0) and e.mean() < 2e-2 * b.float().abs().mean() + 1e-4
+
+    # (b) exact ties
+    S, H, B = 1024, 2, 64
+    g = torch.Generator().manual_seed(5)
+    blk = torch.randn((B, H, 128), generator=g).to(torch.bfloat16)
+    k = blk.repeat(S // B, 1, 1)
+    q = torch.randn((S, H, 128), generator=g).to(torch.bfloat16)
+    cu = [0, S]
+    plan = make_plan(cu, B, 4, device="cuda")
+    sel = E.gate_topk(q.cuda(), E.chunk_mean(k.cuda(), plan), plan).cpu()
+    got = torch.sort(torch.where(sel < 0, torch.full_like(sel, 1 << 30), sel), dim=-1).values
+    got = torch.where(got == 1 << 30, torch.full_like(got, -1), got)
+    want = O.select_topk(O.gate_scores(q, O.chunk_mean(k, cu, B), cu, B), plan.K)
+    assert torch.equal(got, want.to(got.dtype))
+    tok = torch.arange(S)
+    c = tok // B
+    for j in range(plan.K):                       # lowest ids win: slot j holds chunk j wherever it exists
+        assert torch.equal(got[:, :, j], torch.where(c > j, torch.tensor(j), torch.tensor(-1))[:, None].expand(S, H).to(got.dtype))
+
+
 def test_one_token_sequences():
     from moba_amd import moba_efficient as E
     g = torch.Generator().manual_seed(3)
