@@ -177,8 +177,7 @@ def _forward(q, k, v, plan: MobaPlan, timer: Optional[StageTimer] = None):
         _lib.check(lib.moba_fwd_partials(_ptr(q), _ptr(k), _ptr(v), _ptr(part_o), _ptr(part_lse), _ptr(seg_off),
                                          _ptr(tile_off), _ptr(seg_dest), _ptr(t.get("fchunk_tok")),
                                          _ptr(t["chunk_tok"]), _ptr(t["self_tile_prefix"]), _ptr(tile_seg),
-                                         _ptr(t["self_tile_chunk"]), S, H, k.shape[1], D, K, plan.F,
-                                         plan.N,
+                                         _ptr(t["self_tile_chunk"]), S, H, k.shape[1], D, K, plan.F, plan.N,
                                          plan.chunk_size, plan.hist_tile_bound(H), plan.self_tiles, _dtype_code(q),
                                          _stream(dev)), "moba_fwd_partials")
     with span("fwd_merge"):
@@ -201,11 +200,9 @@ def _backward(dout, q, k, v, out, lse, sel, seg_off, tile_off, seg_dest, tile_se
     _lib.check(lib.moba_bwd(_ptr(dout), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(sel), _ptr(seg_off),
                             _ptr(tile_off), _ptr(seg_dest), _ptr(t.get("fchunk_tok")), _ptr(t["chunk_tok"]),
                             _ptr(t["self_tile_prefix"]), _ptr(tile_seg), _ptr(t["self_tile_chunk"]),
-                            _ptr(t.get("chunk_fid")),
-                            _ptr(delta), _ptr(part_dq), _ptr(dq), _ptr(dk), _ptr(dv),
+                            _ptr(t.get("chunk_fid")), _ptr(delta), _ptr(part_dq), _ptr(dq), _ptr(dk), _ptr(dv),
                             S, H, k.shape[1], D, K, plan.F, plan.N, plan.chunk_size, plan.hist_tile_bound(H),
-                            plan.self_tiles,
-                            _dtype_code(q), _stream(dev)), "moba_bwd")
+                            plan.self_tiles, _dtype_code(q), _stream(dev)), "moba_bwd")
     return dq, dk, dv
 
 
