@@ -48,6 +48,7 @@ __global__ __launch_bounds__(256) void lists_count_kernel(
   for (int i = threadIdx.x; i < c; i += 256) cnt[cnt_index(pair_off, fb + i, h, H, c - i - 1)] = lds[i];
 }
 
+template <int KC>  // compile-time bound on K: a lane keeps its token's picks in registers
 __global__ __launch_bounds__(256) void lists_fill_kernel(
     const int* __restrict__ sel, const int* __restrict__ chunk_tok, const int* __restrict__ chunk_fb,
     const int* __restrict__ chunk_local, const int* __restrict__ pair_off, const int* __restrict__ base,
@@ -73,7 +74,9 @@ __global__ __launch_bounds__(256) void lists_fill_kernel(
   // per-wave counts
   for (int s = w0 + lane; s < w1; s += 64) {
     const int* src = sel + ((int64_t)s * H + h) * K;
-    for (int j = 0; j < K; ++j) {
+#pragma unroll
+    for (int j = 0; j < KC; ++j) {
+      if (j >= K) break;
       const int i = src[j] - fb;
       if ((unsigned)i < (unsigned)c) atomicAdd(&pos[wave * c + i], 1);
     }
@@ -98,23 +101,33 @@ __global__ __launch_bounds__(256) void lists_fill_kernel(
     const int s = w0 + bi * 64 + lane;
     const bool active = s < w1;
     const int* src = sel + ((int64_t)(active ? s : t0) * H + h) * K;
-    for (int j = 0; j < K; ++j) {
-      const int i = src[j] - fb;
-      if (active && (unsigned)i < (unsigned)c) atomicOr(&wbits[2 * i + (lane >> 5)], 1u << (lane & 31));
+    int pick[KC];  // candidate index of each pick, -1 when it is not a list entry
+#pragma unroll
+    for (int j = 0; j < KC; ++j) {
+      pick[j] = -1;
+      if (j < K) {
+        const int i = src[j] - fb;
+        if (active && (unsigned)i < (unsigned)c) pick[j] = i;
+      }
     }
+#pragma unroll
+    for (int j = 0; j < KC; ++j)
+      if (pick[j] >= 0) atomicOr(&wbits[2 * pick[j] + (lane >> 5)], 1u << (lane & 31));
     __syncthreads();
-    for (int j = 0; j < K; ++j) {
-      const int i = src[j] - fb;
-      if (active && (unsigned)i < (unsigned)c) {
+#pragma unroll
+    for (int j = 0; j < KC; ++j) {
+      if (pick[j] >= 0) {
+        const int i = pick[j];
         const uint64_t m = (uint64_t)wbits[2 * i] | ((uint64_t)wbits[2 * i + 1] << 32);
         const int rank = __popcll(m & below);
         seg_dest[wpos[i] + rank] = (s * H + h) * K1 + 1 + j;
       }
     }
     __syncthreads();
-    for (int j = 0; j < K; ++j) {
-      const int i = src[j] - fb;
-      if (active && (unsigned)i < (unsigned)c) {
+#pragma unroll
+    for (int j = 0; j < KC; ++j) {
+      if (pick[j] >= 0) {
+        const int i = pick[j];
         const uint64_t m = (uint64_t)wbits[2 * i] | ((uint64_t)wbits[2 * i + 1] << 32);
         if ((m & below) == 0) {  // the first lane of this pick closes the batch for it
           wpos[i] += __popcll(m);
@@ -221,8 +234,14 @@ extern "C" int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, co
   hipLaunchKernelGGL(lists_count_kernel, grid, dim3(256), (size_t)cmax * 4, st, sel, chunk_tok, chunk_fb,
                      chunk_local, pair_off, cnt, H, K);
   hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(1024), 0, st, cnt, P * H);
-  hipLaunchKernelGGL(lists_fill_kernel, grid, dim3(256), (size_t)cmax * 48, st, sel, chunk_tok, chunk_fb,
-                     chunk_local, pair_off, (const int*)cnt, seg_dest, H, K);
+#define MOBA_FILL(KC)                                                                                   \
+  hipLaunchKernelGGL(lists_fill_kernel<KC>, grid, dim3(256), (size_t)cmax * 48, st, sel, chunk_tok, chunk_fb, \
+                     chunk_local, pair_off, (const int*)cnt, seg_dest, H, K)
+  if (K <= 4) MOBA_FILL(4);
+  else if (K <= 16) MOBA_FILL(16);
+  else if (K <= 64) MOBA_FILL(64);
+  else return MOBA_ERR_LIMIT;
+#undef MOBA_FILL
   hipLaunchKernelGGL(lists_segments_kernel, dim3((F * H + 1 + 255) / 256), dim3(256), 0, st, (const int*)cnt,
                      pair_off, seg_off, tile_off, F, H, tile_rows);
   hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(1024), 0, st, tile_off, F * H);
