@@ -7,7 +7,7 @@
 // does not depend on how the chunk is split over workgroups, and the rounded
 // mean is reproducible bit for bit (fp64 -> fp32 -> element type, round to nearest even).
 //
-// Stage 1: grid (column blocks, token splits, F); each thread owns 8 adjacent
+// Stage 1: grid (F, token splits, column blocks); each thread owns 8 adjacent
 //          columns of the [H*D] token row and sums its token split.
 // Stage 2: sums the splits in order, divides by B, rounds.
 #include "common.h"
@@ -19,10 +19,10 @@ __global__ __launch_bounds__(256) void chunk_mean_partial_kernel(
     const typename E::elem* __restrict__ k, const int* __restrict__ fchunk_tok, double* __restrict__ partial,
     int HD8 /* H*D/8 */, int B, int nsplit, int tok_per_split) {
   MOBA_ELEM_TYPES(E)
-  const int col = blockIdx.x * 256 + threadIdx.x;
+  const int col = blockIdx.z * 256 + threadIdx.x;
   if (col >= HD8) return;
   const int split = blockIdx.y;
-  const int f = blockIdx.z;
+  const int f = blockIdx.x;  // the only grid dimension without a 65535 limit
   const int t0 = split * tok_per_split;
   const int t1 = min(B, t0 + tok_per_split);
   const int64_t row_stride = (int64_t)HD8 * 8;
@@ -107,7 +107,7 @@ extern "C" int moba_chunk_mean(const void* k, const int32_t* fchunk_tok, void* k
   const int nsplit = pick_nsplit(HD8, F, B);
   const int tps = (B + nsplit - 1) / nsplit;
   hipStream_t st = (hipStream_t)stream;
-  dim3 grid((HD8 + 255) / 256, nsplit, F);
+  dim3 grid(F, nsplit, (HD8 + 255) / 256);
   const int64_t n = (int64_t)F * HD8;
   const dim3 fgrid((unsigned)((n + 255) / 256));
   if (dtype == MOBA_DTYPE_F16) {

@@ -156,3 +156,18 @@ def test_sampled_rows_and_invariants(lens, H, Hkv, B, topk):
                 e = (dv[s, h].double().cpu() - want_dv).abs().max().item()
                 assert e <= 2e-2 and e <= 3e-2 * want_dv.abs().max().item() + 1e-4, ("dv", s, h, e)
     print("  worst sampled max-abs", worst, flush=True)
+
+
+def test_chunk_mean_many_chunks():
+    """More filtered chunks than a 16-bit grid dimension holds; exact against an fp64 mean."""
+    from moba_amd import moba_efficient as E
+    from moba_amd.plan import make_plan
+    B, F, H = 8, 70000, 2
+    S = B * (F + 1)
+    g = torch.Generator(device="cuda").manual_seed(3)
+    k = torch.randn((S, H, 128), generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    plan = make_plan([0, S], B, 3, device="cuda")
+    assert plan.F == F
+    kbar = E.chunk_mean(k, plan)
+    want = (k[:F * B].double().view(F, B, H, 128).sum(1) / B).float().to(torch.bfloat16)
+    assert torch.equal(kbar, want)
