@@ -228,18 +228,25 @@ extern "C" int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, co
   if (hist_bound <= 0 || hist_bound >= 0x7fffffffLL) return MOBA_ERR_ARG;
   if (S <= 0 || H <= 0 || K <= 0 || N <= 0 || F <= 0 || P <= 0 || cmax <= 0 || tile_rows <= 0) return MOBA_ERR_ARG;
   if ((int64_t)S * H * (K + 1) >= 0x7fffffffLL || (int64_t)P * H >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
-  if (H > 65535 || (size_t)cmax * 48 > 64 * 1024) return MOBA_ERR_LIMIT;
+  if (H > 65535 || (size_t)cmax * 48 > 160 * 1024) return MOBA_ERR_LIMIT;
   hipStream_t st = (hipStream_t)stream;
   dim3 grid(N, H);
   hipLaunchKernelGGL(lists_count_kernel, grid, dim3(256), (size_t)cmax * 4, st, sel, chunk_tok, chunk_fb,
                      chunk_local, pair_off, cnt, H, K);
   hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(1024), 0, st, cnt, P * H);
-#define MOBA_FILL(KC)                                                                                   \
-  hipLaunchKernelGGL(lists_fill_kernel<KC>, grid, dim3(256), (size_t)cmax * 48, st, sel, chunk_tok, chunk_fb, \
-                     chunk_local, pair_off, (const int*)cnt, seg_dest, H, K)
-  if (K <= 4) MOBA_FILL(4);
-  else if (K <= 16) MOBA_FILL(16);
-  else if (K <= 64) MOBA_FILL(64);
+  // more than 64 KiB of dynamic LDS has to be asked for explicitly
+#define MOBA_FILL(KC)                                                                                          \
+  {                                                                                                            \
+    if ((size_t)cmax * 48 > 64 * 1024 &&                                                                       \
+        hipFuncSetAttribute((const void*)lists_fill_kernel<KC>, hipFuncAttributeMaxDynamicSharedMemorySize,    \
+                            (int)((size_t)cmax * 48)) != hipSuccess)                                           \
+      return MOBA_ERR_LAUNCH;                                                                                  \
+    hipLaunchKernelGGL(lists_fill_kernel<KC>, grid, dim3(256), (size_t)cmax * 48, st, sel, chunk_tok, chunk_fb, \
+                       chunk_local, pair_off, (const int*)cnt, seg_dest, H, K);                                \
+  }
+  if (K <= 4) MOBA_FILL(4)
+  else if (K <= 16) MOBA_FILL(16)
+  else if (K <= 64) MOBA_FILL(64)
   else return MOBA_ERR_LIMIT;
 #undef MOBA_FILL
   hipLaunchKernelGGL(lists_segments_kernel, dim3((F * H + 1 + 255) / 256), dim3(256), 0, st, (const int*)cnt,

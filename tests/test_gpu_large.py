@@ -76,6 +76,7 @@ def _key_dkdv(q, k, v, out, lse, dout, sel, j, h, s0, s1, B, fb):
     ([131072], 32, 8, 4096, 12),                     # headline configuration
     ([59436, 29343, 53769, 62439, 31658, 6749, 21064, 37602], 32, 32, 2048, 3),   # varlen batch
     ([1048576], 32, 8, 4096, 12),                    # 1M tokens: largest index ranges
+    ([32005, 777], 2, 2, 16, 3),                     # 2001 chunks in one sequence: the list builder's big-LDS path
 ])
 def test_sampled_rows_and_invariants(lens, H, Hkv, B, topk):
     from moba_amd import moba_efficient as E
@@ -137,7 +138,7 @@ def test_sampled_rows_and_invariants(lens, H, Hkv, B, topk):
     rows = sorted(set(rng.integers(0, S, size=14).tolist() + [0, S - 1, int(cu[1]) - 1, min(S - 1, B), min(S - 1, B - 1)]))
     worst = 0.0
     for s in rows:
-        for h in (0, H // 2 + 1, H - 1):
+        for h in sorted({0, min(H // 2 + 1, H - 1), H - 1}):
             b = int(np.searchsorted(cu, s, side="right") - 1)
             ref, ref_lse = _row_oracle(q, k, v, sel[s, h].cpu(), s, h, int(cu[b]), B, int(plan.host["seq_fbase"][b]))
             err = (out[s, h].float().cpu() - ref).abs().max().item()
