@@ -91,6 +91,37 @@ def cpu_baseline(q, k, v, B, topk, budget_tokens=32768, heads=4):
                       f"algorithm of moba_naive, {dt:.1f} s"}
 
 
+def bench_decode(dev, skv, heads, kv_heads=8, iters=50):
+    """One query token per sequence against a cache of skv keys: the HIP decode kernel and PyTorch's
+    scaled_dot_product_attention on the same tensors.  HBM-bound: K and V are read once."""
+    import torch.nn.functional as F
+
+    from moba_amd.decode import decode_attention
+    kv_heads = min(kv_heads, heads)
+    g = torch.Generator(device=dev).manual_seed(2)
+    q = torch.randn((1, heads, 1, 128), generator=g, device=dev).to(torch.bfloat16)
+    k = torch.randn((1, kv_heads, skv, 128), generator=g, device=dev).to(torch.bfloat16)
+    v = torch.randn((1, kv_heads, skv, 128), generator=g, device=dev).to(torch.bfloat16)
+
+    def timed(fn):
+        for _ in range(5):
+            fn()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(iters):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / iters
+
+    ms = timed(lambda: decode_attention(q, k, v))
+    ms_sdpa = timed(lambda: F.scaled_dot_product_attention(q, k, v, enable_gqa=heads != kv_heads))
+    gbs = 2 * k.numel() * 2 / (ms * 1e-3) / 1e9
+    return {"tokens_in_cache": skv, "heads": heads, "kv_heads": kv_heads, "ms": ms, "sdpa_ms": ms_sdpa,
+            "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": gbs / HBM_PEAK_GBS}}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -99,6 +130,9 @@ def main():
     ap.add_argument("--workload", default=DEFAULT, help="one of %s, or its cfgN prefix" % ", ".join(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--backward", action="store_true", help="also time forward + backward")
+    ap.add_argument("--decode", action="store_true",
+                    help="also time the decode kernel (one token against a cache of the workload's length, "
+                         "8 KV heads) next to PyTorch SDPA")
     ap.add_argument("--gqa", action="store_true",
                     help="keep the key/value heads unexpanded (grouped-query operator) instead of the reference "
                          "wrapper's repeat_kv; not the headline configuration")
@@ -184,6 +218,8 @@ def main():
         gbs = k.numel() * 2 / (stage_ms["chunk_mean"] * 1e-3) / 1e9
         result["chunk_mean_hbm"] = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                     "frac": gbs / HBM_PEAK_GBS}
+    if args.decode:
+        result["decode"] = bench_decode(dev, S if len(cu) == 2 else max_seqlen, H)
     if not args.no_cpu_baseline:
         rep = H // k.shape[1]
         result["cpu_baseline"] = cpu_baseline(q, k[:, ::1] if rep == 1 else torch.repeat_interleave(k[:, :1], 4, dim=1),

@@ -110,6 +110,19 @@ int moba_bwd(const void* dout, const void* q, const void* k, const void* v, cons
              int Hkv, int D, int K, int F, int N, int B, int64_t hist_bound, int64_t self_tiles, int dtype,
              void* stream);
 
+/* Decode: one query token per sequence against the key/value cache.  Replaces the
+ * flash_attn_func call of the adapter's decode branch, moba/wrapper.py:76-82 (full attention
+ * over the cache, grouped-query heads).
+ *   q [B,H,D]: element strides q_stride_b, q_stride_h, D contiguous
+ *   k, v [B,Hkv,Skv,D]: element strides kv_stride_b, kv_stride_h; key rows contiguous and D apart
+ *   out [B,H,D] elem, contiguous
+ *   part_o [B*H*splits, D] fp32 and part_lse [B*H*splits] fp32 scratch, splits = moba_decode_splits()
+ * H/Hkv in {1,2,4,8}; strides multiples of 8 elements; scale = softmax scale. */
+int moba_decode_splits(int B, int Hkv, int Skv);
+int moba_decode(const void* q, const void* k, const void* v, void* out, float* part_o, float* part_lse, int B, int H,
+                int Hkv, int Skv, int D, int64_t q_stride_b, int64_t q_stride_h, int64_t kv_stride_b,
+                int64_t kv_stride_h, float scale, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

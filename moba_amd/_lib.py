@@ -8,7 +8,7 @@ from __future__ import annotations
 
 import ctypes
 import os
-from ctypes import c_char_p, c_int, c_int64, c_size_t, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # MOBA_HIP_LIBRARY overrides the location (e.g. to try a differently built library)
@@ -34,6 +34,8 @@ _SIGNATURES = {
                                           c_int, c_void_p]),
     "moba_bwd": (c_int, [c_void_p] * 21 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_int64,
                                           c_int, c_void_p]),
+    "moba_decode_splits": (c_int, [c_int, c_int, c_int]),
+    "moba_decode": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_int64] * 4 + [c_float, c_int, c_void_p]),
 }
 OPTIONAL = set()
 DTYPE_BF16, DTYPE_F16 = 0, 1

@@ -4,7 +4,8 @@ Prefill (q_len == kv_len) converts the HF layout [batch, heads, seq, dim] to the
 varlen layout and calls the MoBA operator (KV heads are expanded to the query heads first
 unless the operator handles grouped-query attention itself).
 Decode (q_len != kv_len) is full causal attention over the KV cache, as in the
-reference (moba/wrapper.py:76-82), done with PyTorch's scaled_dot_product_attention.
+reference (moba/wrapper.py:76-82): the HIP decode kernel for one new token with the "moba"
+implementation, PyTorch's scaled_dot_product_attention otherwise.
 """
 
 from typing import Callable, Optional, Tuple
@@ -29,6 +30,15 @@ def _cu_seqlens_for(batch: int, seq_len: int, device) -> torch.Tensor:
         t = torch.arange(0, (batch + 1) * seq_len, seq_len, dtype=torch.int32, device=device)
         _CU_SEQLENS[key] = t
     return t
+
+
+def _hip_decode(moba_impl, query, key, value) -> bool:
+    """The HIP decode kernel serves the HIP operator's registrations ("moba"), for the shapes it supports;
+    anything else decodes with PyTorch's scaled_dot_product_attention."""
+    if not getattr(moba_impl, "takes_host_lengths", False):
+        return False
+    from .decode import supported
+    return supported(query, key, value)
 
 
 def hf_to_fa(x: torch.Tensor) -> torch.Tensor:
@@ -101,6 +111,10 @@ def moba_layer(
             moba_chunk_size=chunk_size,
             moba_topk=moba_config.moba_topk,
         )
+    elif q_len == 1 and dropout == 0.0 and _hip_decode(moba_impl, query, key, value):
+        # one new token against the cache: the HIP decode kernel reads K and V once, in place
+        from .decode import decode_attention
+        out = decode_attention(query, key, value, scaling)
     else:
         # decode: every cached key is visible to the new queries (bottom-right aligned causal mask)
         mask = None
