@@ -79,6 +79,19 @@ def test_generate_runs_prefill_then_decode():
     model = _model(torch.bfloat16)
     model.config._attn_implementation = "moba"
     ids = torch.randint(0, 128, (1, 300), device="cuda")
-    with torch.no_grad():
-        out = model.generate(ids, max_new_tokens=4, do_sample=False)
+    import moba_amd.decode as D
+    calls, real = [], D.decode_attention
+
+    def counting(query, key, value, scaling=None):
+        calls.append(key.shape[2])
+        return real(query, key, value, scaling)
+
+    D.decode_attention = counting
+    try:
+        with torch.no_grad():
+            out = model.generate(ids, max_new_tokens=4, do_sample=False)
+    finally:
+        D.decode_attention = real
     assert out.shape == (1, 304)
+    # every decode step of every layer went through the HIP decode kernel, over a growing cache
+    assert len(calls) == 3 * model.config.num_hidden_layers and calls[0] == 301 and calls[-1] == 303
