@@ -137,3 +137,39 @@ def test_forward_vs_oracle(batch, seqlen, heads, B, topk):
     assert err.max() < 2e-2 and err.mean() < 2e-3           # the stated bf16 tolerance
     assert err.mean() < 4e-4                                 # the reference test's own mean bound
     assert (lse - want_lse).abs().max() < 2e-3
+
+
+# ------------------------------------------------------------------ LSE merge alone
+@pytest.mark.parametrize("K,dtype", [(2, torch.bfloat16), (11, torch.bfloat16), (20, torch.float16)])
+def test_merge_of_random_partials(K, dtype):
+    """moba_fwd_merge on random per-slot partials (some slots absent, log-sum-exps far apart)
+    against the merge algebra of the oracle (moba/moba_efficient.py:130-168)."""
+    import ctypes
+    import math
+    from moba_amd import _lib
+    lib = _lib.load()
+    S, H, K1 = 300, 3, K + 1
+    g = torch.Generator().manual_seed(K)
+    part_o = torch.randn((S * H * K1, 128), generator=g).to(dtype)
+    lse_nat = torch.randn((S * H, K1), generator=g) * 6                    # natural-log LSE of each slot
+    sel = torch.randint(0, 50, (S, H, K), generator=g, dtype=torch.int32)
+    sel[torch.rand((S, H, K), generator=g) < 0.3] = -1                     # absent slots
+    part_o_dev = part_o.cuda()
+    # absent slots hold garbage in the real buffers: poison them
+    absent = torch.cat([torch.zeros((S * H, 1), dtype=torch.bool), (sel < 0).view(S * H, K)], dim=1)
+    part_o_dev.view(S * H, K1, 128)[absent.cuda()] = float("nan")
+    part_lse = (lse_nat / math.log(2.0)).float()                           # the kernels keep it in the log2 domain
+    part_lse_dev = part_lse.clone()
+    part_lse_dev[absent] = float("nan")
+    part_lse_dev = part_lse_dev.view(-1).cuda()
+    out = torch.empty((S, H, 128), dtype=dtype, device="cuda")
+    lse = torch.empty((S, H), dtype=torch.float32, device="cuda")
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+    code = _lib.DTYPE_F16 if dtype == torch.float16 else _lib.DTYPE_BF16
+    _lib.check(lib.moba_fwd_merge(p(part_o_dev), p(part_lse_dev), p(sel.cuda()), p(out), p(lse), S, H, 128, K, code,
+                                  ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)), "moba_fwd_merge")
+    lses = lse_nat.clone()
+    lses[absent] = float("-inf")
+    want, want_lse = O.merge_partials(part_o.float().view(S * H, K1, 128).permute(1, 0, 2), lses.t())
+    assert (out.float().cpu().view(S * H, 128) - want).abs().max() < 2e-2
+    assert (lse.cpu().view(-1) - want_lse).abs().max() < 1e-3
