@@ -40,6 +40,11 @@ def _dtype_code(t: torch.Tensor) -> int:
     raise TypeError("moba_attn_varlen supports bfloat16 and float16 q, k, v")
 
 
+def _aligned(t: torch.Tensor) -> torch.Tensor:
+    t = t.contiguous()
+    return t if t.data_ptr() % 16 == 0 else t.clone()
+
+
 def _check_qkv(q, k, v, gqa=False):
     if not (q.is_cuda and k.is_cuda and v.is_cuda):
         raise RuntimeError("moba_attn_varlen needs tensors on an AMD GPU (there is no CPU path)")
@@ -222,7 +227,7 @@ class _MobaAttention(torch.autograd.Function):
     def backward(ctx, dout, _dlse):
         q, k, v, out, lse = ctx.saved_tensors
         sel, seg_off, tile_off, seg_dest, tile_seg = ctx.aux
-        dq, dk, dv = _backward(dout.to(q.dtype).contiguous(), q, k, v, out, lse, sel, seg_off, tile_off, seg_dest, tile_seg,
+        dq, dk, dv = _backward(_aligned(dout.to(q.dtype)), q, k, v, out, lse, sel, seg_off, tile_off, seg_dest, tile_seg,
                                ctx.plan)
         return dq, dk, dv, None, None
 
@@ -272,5 +277,6 @@ def moba_attn_varlen_with_lse(q, k, v, cu_seqlens, max_seqlen, moba_chunk_size, 
     plan = make_plan(cu_seqlens, moba_chunk_size, moba_topk, device=q.device)
     if plan.S != q.shape[0]:
         raise ValueError(f"cu_seqlens ends at {plan.S} but q has {q.shape[0]} tokens")
-    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    # the kernels read 16 bytes per lane: contiguous rows at 16-byte aligned addresses
+    q, k, v = (_aligned(x) for x in (q, k, v))
     return _MobaAttention.apply(q, k, v, plan, timer)
