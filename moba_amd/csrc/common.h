@@ -32,15 +32,14 @@ struct F16 {
   typedef f16x4 elem4;
   typedef f16x8 elem8;
 };
-#define MOBA_ELEM_TYPES(E)            \
-  using elem = typename E::elem;      \
-  using elem2 = typename E::elem2;    \
-  using elem4 = typename E::elem4;    \
-  using elem8 = typename E::elem8;
+#define MOBA_ELEM_TYPES(E)                              \
+  using elem [[maybe_unused]] = typename E::elem;       \
+  using elem2 [[maybe_unused]] = typename E::elem2;     \
+  using elem4 [[maybe_unused]] = typename E::elem4;     \
+  using elem8 [[maybe_unused]] = typename E::elem8;
 enum : int { MOBA_DTYPE_BF16 = 0, MOBA_DTYPE_F16 = 1 };
 
 constexpr int kHeadDim = 128;  // the MFMA kernels are specialised for D = 128
-constexpr int kWave = 64;
 
 // error codes returned by every extern "C" entry point
 enum : int {
@@ -64,9 +63,6 @@ __device__ __forceinline__ f32x16 mfma32(f16x8 a, f16x8 b, f32x16 c) {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
-// value held by the lane 32 positions away (the other half of the wave)
-__device__ __forceinline__ float xhalf(float x) { return __shfl_xor(x, 32, 64); }
-
 // two floats rounded (to nearest even) to the element type, packed into 32 bits
 template <class E>
 __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
@@ -84,15 +80,6 @@ __device__ __forceinline__ int upper_row(const int* __restrict__ a, int n, int x
     if (a[mid] <= x) lo = mid; else hi = mid;
   }
   return lo;
-}
-
-// Workgroup ids are dealt round-robin to the 8 XCDs (each with its own L2).
-// Remap so that a contiguous range of logical ids lands on one XCD.
-__device__ __forceinline__ int xcd_remap(int bid, int nblocks) {
-  constexpr int X = 8;
-  int per = (nblocks + X - 1) / X;
-  int logical = (bid % X) * per + bid / X;
-  return logical;  // may be >= nblocks for the padded tail: callers bound-check
 }
 
 }  // namespace moba
