@@ -392,10 +392,8 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
     for (int i = 0; i < 4; ++i) raw[i] = src[min(base + 4 * (4 * i + wave_u) + ld_rin, list_rows - 1)];
     raw[4] = src[min(base + lane, list_rows - 1)];
   };
-  auto issue_stage = [&](int qi, int buf) __attribute__((always_inline)) {
-    const uint32_t qdst = lds_base + buf * kQStage;
-    const uint32_t odst = qdst + TQ * kHeadDim * 2;
-    int toks[5];
+  int toks[5];  // tokens of the rows of the stage whose copies are being issued
+  auto prepare_stage = [&](int qi) __attribute__((always_inline)) {
     if (qi < nself) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) toks[i] = c0 + key0 + min(qi * TQ + 4 * (4 * i + wave_u) + ld_rin, self_rows - 1);
@@ -404,20 +402,30 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
 #pragma unroll
       for (int i = 0; i < 5; ++i) toks[i] = (int)(((uint64_t)(uint32_t)raw[i] * p.hk_magic) >> p.hk_shift);
     }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int slab = 4 * i + wave_u;
-      const int row = 4 * slab + ld_rin;
-      const int c16 = sw_col16(row, ld_pc);
-      const int64_t off = (((int64_t)toks[i] * H + h) * kHeadDim + c16 * 8) * 2;
-      async_copy16((const char*)p.q + off, qdst + slab * 1024);
-      async_copy16((const char*)p.dout + off, odst + slab * 1024);
-    }
-    if (wave_u < 2) {
+  };
+  // part g of the 8 row copies of a stage (slab g/2 of Q for even g, of dO for odd g); the last part also
+  // brings the softmax statistics.  A copy instruction occupies the wave for tens of cycles while the
+  // address unit takes its 64 lanes, so the parts are issued one at a time between MFMAs, not in a burst.
+  auto issue_part = [&](int g, int buf) __attribute__((always_inline)) {
+    const uint32_t qdst = lds_base + buf * kQStage;
+    const int i = g >> 1;
+    const int slab = 4 * i + wave_u;
+    const int row = 4 * slab + ld_rin;
+    const int c16 = sw_col16(row, ld_pc);
+    const int64_t off = (((int64_t)toks[i] * H + h) * kHeadDim + c16 * 8) * 2;
+    if ((g & 1) == 0) async_copy16((const char*)p.q + off, qdst + slab * 1024);
+    else              async_copy16((const char*)p.dout + off, qdst + TQ * kHeadDim * 2 + slab * 1024);
+    if (g == 7 && wave_u < 2) {
       const float* src = (wave_u == 0 ? p.lse2 : p.delta) + ((int64_t)toks[4] * H + h);
       async_copy4(src, qdst + 2 * TQ * kHeadDim * 2 + wave_u * (TQ * 4));
     }
   };
+  auto issue_stage = [&](int qi, int buf) __attribute__((always_inline)) {
+    prepare_stage(qi);
+#pragma unroll
+    for (int g = 0; g < 8; ++g) issue_part(g, buf);
+  };
+  auto no_dma = [](int) __attribute__((always_inline)) {};
 
   f32x16 dkacc[4], dvacc[4];
 #pragma unroll
@@ -466,7 +474,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
   // S and dO V^T from qa/oa into (s_next, dp_next); P and dS of (s_cur, dp_cur) with l4/d4.
   // Block rows are 32*qb + 8g + 4hh + r; `rows_ok` rows of the stage are real, self stages are causal.
   auto phase_a = [&](f32x16& s_next, f32x16& dp_next, const f32x16& s_cur, const f32x16& dp_cur, auto masked_c,
-                     int qb, int rows_ok, bool is_self, int qpos0, elem8 (&pb)[2], elem8 (&dsb)[2])
+                     int qb, int rows_ok, bool is_self, int qpos0, elem8 (&pb)[2], elem8 (&dsb)[2], auto dma)
                      __attribute__((always_inline)) {
     f32x16 zero;
 #pragma unroll
@@ -496,6 +504,8 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
       pb[k >> 3][(k & 7) + 1] = (elem)pe[1];
       dsb[k >> 3][k & 7] = (elem)ds[0];
       dsb[k >> 3][(k & 7) + 1] = (elem)ds[1];
+      dma(k >> 1);  // one global -> LDS copy (or nothing) per pair of MFMAs
+      __builtin_amdgcn_sched_barrier(0);
     }
     __builtin_amdgcn_sched_barrier(0);
   };
@@ -566,7 +576,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
 #pragma unroll
     for (int g = 0; g < 4; ++g) { l4[g] = f32x4{0.f, 0.f, 0.f, 0.f}; d4[g] = l4[g]; }
     load_frags(smem, 0);
-    phase_a(sA, dA, sB, dB, std::false_type{}, 0, 0, false, 0, pb, dsb);
+    phase_a(sA, dA, sB, dB, std::false_type{}, 0, 0, false, 0, pb, dsb, no_dma);
     load_stats(smem, 0);
     load_frags(smem, 1);
   }
@@ -586,17 +596,20 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
     const char* qs_next = has_next ? smem + buf1 * kQStage : qs;
     elem8 pb[2], dsb[2];
 
-    if (masked) phase_a(sB, dB, sA, dA, std::true_type{}, 0, rows_here, is_self, qpos0, pb, dsb);
-    else        phase_a(sB, dB, sA, dA, std::false_type{}, 0, rows_here, is_self, qpos0, pb, dsb);
+    if (masked) phase_a(sB, dB, sA, dA, std::true_type{}, 0, rows_here, is_self, qpos0, pb, dsb, no_dma);
+    else        phase_a(sB, dB, sA, dA, std::false_type{}, 0, rows_here, is_self, qpos0, pb, dsb, no_dma);
 
     if (has_next) wait_vmem();
     __syncthreads();
-    if (qi + 2 < ntile) issue_stage(qi + 2, buf2);
+    // the copies of stage qi+2 go out one at a time inside the next phase A
+    const bool issue_next = qi + 2 < ntile;
+    if (issue_next) prepare_stage(qi + 2);
     fetch_rows(qi + 3);
 
     phase_b(qs, 0, pb, dsb, qs_next, 0, qs, 1);
-    if (masked) phase_a(sA, dA, sB, dB, std::true_type{}, 1, rows_here, is_self, qpos0, pb, dsb);
-    else        phase_a(sA, dA, sB, dB, std::false_type{}, 1, rows_here, is_self, qpos0, pb, dsb);
+    auto dma = [&](int g) __attribute__((always_inline)) { if (issue_next) issue_part(g, buf2); };
+    if (masked) phase_a(sA, dA, sB, dB, std::true_type{}, 1, rows_here, is_self, qpos0, pb, dsb, dma);
+    else        phase_a(sA, dA, sB, dB, std::false_type{}, 1, rows_here, is_self, qpos0, pb, dsb, dma);
     phase_b(qs, 1, pb, dsb, qs_next, 1, qs_next, 0);
     buf = buf1;
   }
