@@ -3,7 +3,8 @@
  * The reference (MoonshotAI/MoBA) has no native code: its hot path is torch ops plus
  * the private varlen entry points of the flash-attn wheel.  Each entry point below
  * names the reference lines whose arithmetic it replaces.  All pointers are device
- * pointers unless stated otherwise; tensors are contiguous; `stream` is a hipStream_t.
+ * pointers unless stated otherwise; tensors are contiguous except q, k, v (see `strides`);
+ * `stream` is a hipStream_t.
  * The library allocates nothing, frees nothing, and never synchronises the device:
  * every launch is enqueued on `stream`.  Return value: 0, or a negative code that
  * moba_strerror() explains.  head_dim 128; q, k, v and everything derived from them are
@@ -16,6 +17,14 @@
  * F filtered chunks (chunks that are not the last of their sequence), K selected
  * history chunks per (token, head), M = number of selected (token, head, chunk)
  * triples, P = number of (filtered chunk, later chunk of the same sequence) pairs.
+ *
+ * `strides` (a host pointer, read during the call) describes q, k and v where an entry point
+ * takes it: {q token stride, q head stride, k/v token stride, k/v head stride} in elements; the
+ * D elements of one (token, head) are contiguous, k and v share their strides, every stride is a
+ * positive multiple of 8 and the k/v token stride is at most 2^23.  NULL means packed
+ * [S,H,D] / [S,Hkv,D].  This is what lets a slice of a fused qkv projection or a
+ * [heads, tokens, D] cache be read in place, as flash-attn reads them for the reference
+ * (moba/moba_efficient.py:89-128 passes such views on unchanged).  Outputs are always packed.
  */
 #ifndef MOBA_HIP_H
 #define MOBA_HIP_H
@@ -34,13 +43,13 @@ const char* moba_strerror(int code);
 
 /* Key chunk-mean.  Replaces moba/moba_efficient.py:326-340 (index_select of the
  * filtered chunks, .mean(dim=1) on bf16, .float()).
- *   k          [S,H,D] elem (H here is the number of key/value heads)
+ *   k          [S,H,D] elem (H here is the number of key/value heads); strides[2], strides[3] apply
  *   fchunk_tok [F] int32, first token of each filtered chunk
  *   kbar       [F,H,D] elem out (the mean rounded once to the element type)
  *   workspace  moba_chunk_mean_workspace_bytes() bytes, 8-byte aligned */
 size_t moba_chunk_mean_workspace_bytes(int H, int D, int F, int B);
 int moba_chunk_mean(const void* k, const int32_t* fchunk_tok, void* kbar, void* workspace, int64_t S, int H, int D,
-                    int F, int B, int dtype, void* stream);
+                    int F, int B, const int64_t* strides, int dtype, void* stream);
 
 /* Gate scores + causal top-k.  Replaces moba/moba_efficient.py:341-371 (fp32 einsum,
  * -inf mask, torch.topk, dropping -inf picks).
@@ -48,10 +57,10 @@ int moba_chunk_mean(const void* k, const int32_t* fchunk_tok, void* kbar, void* 
  *   sel        [S,H,K] int32 out: filtered-chunk ids, descending score, -1 padded
  *   scores_out optional [S,H,F] fp32, pre-filled with -inf by the caller; receives the
  *              score of every valid candidate (debug / test output), may be NULL
- * K <= 64. */
+ * K <= 64.  strides[0], strides[1] apply to q; kbar is packed [F,Hkv,D]. */
 int moba_gate_topk(const void* q, const void* kbar, const int32_t* cu_seqlens, const int32_t* seq_fbase, int32_t* sel,
-                   float* scores_out, int64_t S, int H, int Hkv, int D, int nseq, int F, int B, int K, int dtype,
-                   void* stream);
+                   float* scores_out, int64_t S, int H, int Hkv, int D, int nseq, int F, int B, int K,
+                   const int64_t* strides, int dtype, void* stream);
 
 /* The selection step of moba/moba_efficient.py:365-371 alone, on caller-supplied
  * scores [S,H,F] fp32 (-inf = not a candidate).  Same routine as moba_gate_topk. */
@@ -88,27 +97,30 @@ int moba_fwd_tile_rows(void);
 int moba_fwd_partials(const void* q, const void* k, const void* v, void* part_o, float* part_lse,
                       const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest,
                       const int32_t* fchunk_tok, const int32_t* chunk_tok, const int32_t* self_tile_prefix,
-                      const int32_t* tile_seg, const int32_t* self_tile_chunk, int64_t S, int H, int Hkv, int D, int K, int F, int N, int B, int64_t hist_bound, int64_t self_tiles,
-                      int dtype, void* stream);
+                      const int32_t* tile_seg, const int32_t* self_tile_chunk, int64_t S, int H, int Hkv, int D, int K,
+                      int F, int N, int B, int64_t hist_bound, int64_t self_tiles, const int64_t* strides, int dtype,
+                      void* stream);
 int moba_fwd_merge(const void* part_o, const float* part_lse, const int32_t* sel, void* out, float* lse, int64_t S,
                    int H, int D, int K, int dtype, void* stream);
 int moba_fwd(const void* q, const void* k, const void* v, void* part_o, float* part_lse, const int32_t* sel,
              const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest, const int32_t* fchunk_tok,
              const int32_t* chunk_tok, const int32_t* self_tile_prefix, const int32_t* tile_seg,
-             const int32_t* self_tile_chunk, void* out, float* lse, int64_t S, int H, int Hkv, int D, int K, int F, int N, int B, int64_t hist_bound, int64_t self_tiles, int dtype, void* stream);
+             const int32_t* self_tile_chunk, void* out, float* lse, int64_t S, int H, int Hkv, int D, int K, int F,
+             int N, int B, int64_t hist_bound, int64_t self_tiles, const int64_t* strides, int dtype, void* stream);
 
 /* Backward.  Replaces MixedAttention.backward, moba/moba_efficient.py:185-267, and the
  * autograd scatter of its gathered gradients.  Deterministic (no floating-point atomics).
  *   dout, q, out, dq [S,H,D] elem; k, v, dk, dv [S,Hkv,D] elem; lse [S,H] fp32 from the forward
+ *   (`strides` applies to q, k, v; dout, out, dq, dk, dv are packed)
  *   chunk_fid [N] int32: filtered id of each chunk, -1 for the last chunk of a sequence
  *   delta [2,S,H] fp32 scratch (rowsum(dO*O), then the LSE in the log2 domain); part_dq [S*H*(K+1), D] fp32 scratch
  *   dq, dk, dv: out; dk and dv of a key/value head sum over its query heads */
 int moba_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out, const float* lse,
              const int32_t* sel, const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest,
              const int32_t* fchunk_tok, const int32_t* chunk_tok, const int32_t* self_tile_prefix,
-             const int32_t* tile_seg, const int32_t* self_tile_chunk, const int32_t* chunk_fid, float* delta, float* part_dq, void* dq, void* dk, void* dv, int64_t S, int H,
-             int Hkv, int D, int K, int F, int N, int B, int64_t hist_bound, int64_t self_tiles, int dtype,
-             void* stream);
+             const int32_t* tile_seg, const int32_t* self_tile_chunk, const int32_t* chunk_fid, float* delta,
+             float* part_dq, void* dq, void* dk, void* dv, int64_t S, int H, int Hkv, int D, int K, int F, int N, int B,
+             int64_t hist_bound, int64_t self_tiles, const int64_t* strides, int dtype, void* stream);
 
 /* Decode: one query token per sequence against the key/value cache.  Replaces the
  * flash_attn_func call of the adapter's decode branch, moba/wrapper.py:76-82 (full attention

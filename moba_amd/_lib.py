@@ -8,7 +8,9 @@ from __future__ import annotations
 
 import ctypes
 import os
-from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
+from ctypes import POINTER, c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
+
+c_strides = POINTER(c_int64)  # {q token, q head, k/v token, k/v head} in elements, or None for packed tensors
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # MOBA_HIP_LIBRARY overrides the location (e.g. to try a differently built library)
@@ -20,20 +22,20 @@ _SIGNATURES = {
     "moba_version": (c_int, []),
     "moba_strerror": (c_char_p, [c_int]),
     "moba_chunk_mean_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
-    "moba_chunk_mean": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_int,
-                                c_void_p]),
+    "moba_chunk_mean": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_strides,
+                                c_int, c_void_p]),
     "moba_gate_topk": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                               c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+                               c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_strides, c_int, c_void_p]),
     "moba_topk_from_scores": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_void_p]),
     "moba_build_lists": (c_int, [c_void_p] * 10 + [c_int64] + [c_int] * 7 + [c_int64, c_void_p]),
     "moba_fwd_tile_rows": (c_int, []),
     "moba_fwd_partials": (c_int, [c_void_p] * 13 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int64,
-                                                   c_int64, c_int, c_void_p]),
+                                                   c_int64, c_strides, c_int, c_void_p]),
     "moba_fwd_merge": (c_int, [c_void_p] * 5 + [c_int64, c_int, c_int, c_int, c_int, c_void_p]),
     "moba_fwd": (c_int, [c_void_p] * 16 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_int64,
-                                          c_int, c_void_p]),
+                                          c_strides, c_int, c_void_p]),
     "moba_bwd": (c_int, [c_void_p] * 21 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_int64,
-                                          c_int, c_void_p]),
+                                          c_strides, c_int, c_void_p]),
     "moba_decode_splits": (c_int, [c_int, c_int, c_int]),
     "moba_decode": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_int64] * 4 + [c_float, c_int, c_void_p]),
 }

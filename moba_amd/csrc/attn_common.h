@@ -25,7 +25,28 @@ struct TileTables {
   int Hkv, rep;                 // key/value heads and query heads per key/value head (H = Hkv * rep)
   int hist_bound;               // logical tile ids below it are history tiles
   int self_total;               // self_tile_prefix[N] * H
+  // byte strides of q[token][head][:] and of k, v[token][kv head][:] (k and v share theirs); the
+  // 128 elements of a (token, head) are contiguous
+  int64_t q_tok_b, q_head_b, kv_tok_b, kv_head_b;
 };
+
+// strides: {q token, q head, k/v token, k/v head} in elements, or null for packed [S, H, 128] /
+// [S, Hkv, 128] tensors.  Returns false for strides the kernels cannot address: not multiples of
+// 8 elements (16-byte accesses), not positive, or a key/value token stride whose 64-row tile
+// offsets leave 31 bits.
+inline bool set_layout(TileTables& t, const int64_t* strides) {
+  if (!strides) {
+    t.q_tok_b = (int64_t)t.H * kHeadDim * 2; t.q_head_b = kHeadDim * 2;
+    t.kv_tok_b = (int64_t)t.Hkv * kHeadDim * 2; t.kv_head_b = kHeadDim * 2;
+    return true;
+  }
+  for (int i = 0; i < 4; ++i)
+    if (strides[i] <= 0 || (strides[i] & 7)) return false;
+  if (strides[2] > (1 << 23)) return false;
+  t.q_tok_b = strides[0] * 2; t.q_head_b = strides[1] * 2;
+  t.kv_tok_b = strides[2] * 2; t.kv_head_b = strides[3] * 2;
+  return true;
+}
 
 // One tile of up to TM query rows of one head, as seen by a lane.
 struct Tile {

@@ -93,9 +93,10 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams<E> p) {
   elem8 bq[8], bdo[8];
   {
     const int64_t off = ((int64_t)t.tok * H + h) * kHeadDim + 8 * hh;
+    const elem* qsrc = reinterpret_cast<const elem*>((const char*)p.q + t.tok * p.t.q_tok_b + h * p.t.q_head_b) + 8 * hh;
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
-      bq[ks] = *reinterpret_cast<const elem8*>(p.q + off + 16 * ks);
+      bq[ks] = *reinterpret_cast<const elem8*>(qsrc + 16 * ks);
       bdo[ks] = *reinterpret_cast<const elem8*>(p.dout + off + 16 * ks);
     }
   }
@@ -103,7 +104,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams<E> p) {
   const float dl = p.delta[(int64_t)t.tok * H + h];
 
   const int hkv = h / p.t.rep;                                // key/value head of this query head
-  const int64_t row_bytes = (int64_t)p.t.Hkv * kHeadDim * 2;   // of a K or V token row
+  const int64_t row_bytes = p.t.kv_tok_b;                     // from one K or V token to the next
   const uint32_t lds_base = lds_addr(smem);
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   const int ld_kin = lane >> 4, ld_pc = lane & 15;
@@ -113,8 +114,8 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams<E> p) {
     const int key = 4 * (4 * i + wave_u) + ld_kin;
     ld_off[i] = (uint32_t)(key * row_bytes + sw_col16(key, ld_pc) * 16);
   }
-  const char* k_head = (const char*)p.k + (int64_t)kv_tok0 * row_bytes + hkv * (kHeadDim * 2);
-  const char* v_head = (const char*)p.v + (int64_t)kv_tok0 * row_bytes + hkv * (kHeadDim * 2);
+  const char* k_head = (const char*)p.k + (int64_t)kv_tok0 * row_bytes + hkv * p.t.kv_head_b;
+  const char* v_head = (const char*)p.v + (int64_t)kv_tok0 * row_bytes + hkv * p.t.kv_head_b;
   auto issue_tile = [&](int kt, int buf) __attribute__((always_inline)) {
     const uint32_t kdst = lds_base + buf * kTileBytes;
     const uint32_t vdst = lds_base + (2 + buf) * kTileBytes;
@@ -135,7 +136,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams<E> p) {
         const int key = 4 * slab + ld_kin;
         const int c16 = sw_col16(key, ld_pc);
         const int64_t tk = min((int64_t)kv_tok0 + key0 + key, (int64_t)p.t.S - 1);
-        const int64_t off = tk * row_bytes + hkv * (kHeadDim * 2) + c16 * 16;
+        const int64_t off = tk * row_bytes + hkv * p.t.kv_head_b + c16 * 16;
         async_copy16((const char*)p.k + off, kdst + slab * 1024);
         async_copy16((const char*)p.v + off, vdst + slab * 1024);
       }
@@ -368,11 +369,11 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
   // ---- K^T and V^T operands of this lane's key: [16*ks + 8*hh .. +7] ----
   elem8 bk[8], bv[8];
   {
-    const int64_t off = ((int64_t)(c0 + min(mykey, len - 1)) * Hkv + hkv) * kHeadDim + 8 * hh;
+    const int64_t off = (c0 + min(mykey, len - 1)) * p.t.kv_tok_b + hkv * p.t.kv_head_b + 16 * hh;  // bytes
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
-      bk[ks] = *reinterpret_cast<const elem8*>(p.k + off + 16 * ks);
-      bv[ks] = *reinterpret_cast<const elem8*>(p.v + off + 16 * ks);
+      bk[ks] = *reinterpret_cast<const elem8*>((const char*)p.k + off + 32 * ks);
+      bv[ks] = *reinterpret_cast<const elem8*>((const char*)p.v + off + 32 * ks);
     }
   }
 
@@ -412,9 +413,11 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
     const int slab = 4 * i + wave_u;
     const int row = 4 * slab + ld_rin;
     const int c16 = sw_col16(row, ld_pc);
-    const int64_t off = (((int64_t)toks[i] * H + h) * kHeadDim + c16 * 8) * 2;
-    if ((g & 1) == 0) async_copy16((const char*)p.q + off, qdst + slab * 1024);
-    else              async_copy16((const char*)p.dout + off, qdst + TQ * kHeadDim * 2 + slab * 1024);
+    if ((g & 1) == 0)
+      async_copy16((const char*)p.q + (toks[i] * p.t.q_tok_b + h * p.t.q_head_b + c16 * 16), qdst + slab * 1024);
+    else
+      async_copy16((const char*)p.dout + (((int64_t)toks[i] * H + h) * kHeadDim + c16 * 8) * 2,
+                   qdst + TQ * kHeadDim * 2 + slab * 1024);
     if (g == 7 && wave_u < 2) {
       const float* src = (wave_u == 0 ? p.lse2 : p.delta) + ((int64_t)toks[4] * H + h);
       async_copy4(src, qdst + 2 * TQ * kHeadDim * 2 + wave_u * (TQ * 4));
@@ -683,7 +686,7 @@ extern "C" int moba_bwd(const void* dout, const void* q, const void* k, const vo
                         const int32_t* self_tile_prefix, const int32_t* tile_seg, const int32_t* self_tile_chunk,
                         const int32_t* chunk_fid, float* delta, float* part_dq,
                         void* dq, void* dk, void* dv, int64_t S, int H, int Hkv, int D, int K, int F, int N, int B,
-                        int64_t hist_bound, int64_t self_tiles, int dtype, void* stream) {
+                        int64_t hist_bound, int64_t self_tiles, const int64_t* strides, int dtype, void* stream) {
   if (!dout || !q || !k || !v || !out || !lse || !chunk_tok || !self_tile_prefix || !self_tile_chunk || !delta ||
       !part_dq || !dq || !dk || !dv)
     return MOBA_ERR_ARG;
@@ -709,6 +712,7 @@ extern "C" int moba_bwd(const void* dout, const void* q, const void* k, const vo
   t.Hkv = Hkv; t.rep = H / Hkv;
   t.hist_bound = (K > 0) ? (int)hist_bound : 0;
   t.self_total = (int)(self_tiles * H);
+  if (!set_layout(t, strides)) return MOBA_ERR_ARG;
   hipStream_t st = (hipStream_t)stream;
   return dtype == MOBA_DTYPE_F16
              ? launch_bwd<F16>(dout, q, k, v, out, lse, sel, chunk_fid, delta, part_dq, dq, dk, dv, t, S, H, D, K,

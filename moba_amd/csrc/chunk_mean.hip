@@ -17,7 +17,8 @@ namespace moba {
 template <class E>
 __global__ __launch_bounds__(256) void chunk_mean_partial_kernel(
     const typename E::elem* __restrict__ k, const int* __restrict__ fchunk_tok, double* __restrict__ partial,
-    int HD8 /* H*D/8 */, int B, int nsplit, int tok_per_split) {
+    int HD8 /* H*D/8 */, int D8 /* D/8 */, int B, int nsplit, int tok_per_split, int64_t row_stride,
+    int64_t head_stride) {
   MOBA_ELEM_TYPES(E)
   const int col = blockIdx.z * 256 + threadIdx.x;
   if (col >= HD8) return;
@@ -25,8 +26,8 @@ __global__ __launch_bounds__(256) void chunk_mean_partial_kernel(
   const int f = blockIdx.x;  // the only grid dimension without a 65535 limit
   const int t0 = split * tok_per_split;
   const int t1 = min(B, t0 + tok_per_split);
-  const int64_t row_stride = (int64_t)HD8 * 8;
-  const elem* src = k + ((int64_t)fchunk_tok[f] + t0) * row_stride + (int64_t)col * 8;
+  const int head = col / D8;
+  const elem* src = k + ((int64_t)fchunk_tok[f] + t0) * row_stride + head * head_stride + (col - head * D8) * 8;
   double acc[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.0;
@@ -98,11 +99,16 @@ extern "C" size_t moba_chunk_mean_workspace_bytes(int H, int D, int F, int B) {
 }
 
 extern "C" int moba_chunk_mean(const void* k, const int32_t* fchunk_tok, void* kbar, void* workspace,
-                               int64_t S, int H, int D, int F, int B, int dtype, void* stream) {
+                               int64_t S, int H, int D, int F, int B, const int64_t* strides, int dtype,
+                               void* stream) {
   if (F == 0) return MOBA_OK;
   if (dtype != MOBA_DTYPE_BF16 && dtype != MOBA_DTYPE_F16) return MOBA_ERR_UNSUPPORTED;
   if (!k || !fchunk_tok || !kbar || !workspace || S <= 0 || H <= 0 || D <= 0 || F < 0 || B <= 0) return MOBA_ERR_ARG;
   if ((H * D) % 8 != 0 || ((uintptr_t)k & 15) || ((uintptr_t)kbar & 15) || ((uintptr_t)workspace & 7)) return MOBA_ERR_ARG;
+  if (D % 8 != 0) return MOBA_ERR_ARG;
+  // strides (elements): {., ., k token, k head}; null = packed [S, H, D]
+  const int64_t kts = strides ? strides[2] : (int64_t)H * D, khs = strides ? strides[3] : D;
+  if (kts <= 0 || khs <= 0 || (kts & 7) || (khs & 7)) return MOBA_ERR_ARG;
   const int HD8 = H * D / 8;
   const int nsplit = pick_nsplit(HD8, F, B);
   const int tps = (B + nsplit - 1) / nsplit;
@@ -112,12 +118,12 @@ extern "C" int moba_chunk_mean(const void* k, const int32_t* fchunk_tok, void* k
   const dim3 fgrid((unsigned)((n + 255) / 256));
   if (dtype == MOBA_DTYPE_F16) {
     hipLaunchKernelGGL(chunk_mean_partial_kernel<F16>, grid, dim3(256), 0, st, (const f16*)k, fchunk_tok,
-                       (double*)workspace, HD8, B, nsplit, tps);
+                       (double*)workspace, HD8, D / 8, B, nsplit, tps, kts, khs);
     hipLaunchKernelGGL(chunk_mean_finish_kernel<F16>, fgrid, dim3(256), 0, st, (const double*)workspace, (f16*)kbar,
                        HD8, B, nsplit, F);
   } else {
     hipLaunchKernelGGL(chunk_mean_partial_kernel<Bf16>, grid, dim3(256), 0, st, (const bf16*)k, fchunk_tok,
-                       (double*)workspace, HD8, B, nsplit, tps);
+                       (double*)workspace, HD8, D / 8, B, nsplit, tps, kts, khs);
     hipLaunchKernelGGL(chunk_mean_finish_kernel<Bf16>, fgrid, dim3(256), 0, st, (const double*)workspace,
                        (bf16*)kbar, HD8, B, nsplit, F);
   }

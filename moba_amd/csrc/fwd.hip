@@ -58,7 +58,7 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
   // ---- Q^T operand: lane (n, hh) holds q[tok][16*ks + 8*hh .. +7] ----
   elem8 bq[8];
   {
-    const elem* src = p.q + ((int64_t)t.tok * H + h) * kHeadDim + 8 * hh;
+    const elem* src = reinterpret_cast<const elem*>((const char*)p.q + t.tok * p.t.q_tok_b + h * p.t.q_head_b) + 8 * hh;
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) bq[ks] = *reinterpret_cast<const elem8*>(src + 16 * ks);
   }
@@ -68,7 +68,7 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
   // w, w+4, w+8, w+12.  Lane i lands at slab + 16*i, so the lane picks the global column
   // whose swizzled LDS position is i.  LDS: K stages at 0 and 16 KiB, V stages at 32 and 48 KiB.
   const int hkv = h / p.t.rep;                                   // key/value head of this query head
-  const int64_t row_bytes = (int64_t)p.t.Hkv * kHeadDim * 2;      // of a K or V token row
+  const int64_t row_bytes = p.t.kv_tok_b;                        // from one K or V token to the next
   const uint32_t lds_base = lds_addr(smem);
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   const int ld_kin = lane >> 4;  // key within the slab
@@ -79,8 +79,8 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
     const int key = 4 * (4 * i + wave_u) + ld_kin;
     ld_off[i] = (uint32_t)(key * row_bytes + sw_col16(key, ld_pc) * 16);  // the swizzle is an involution
   }
-  const char* k_head = (const char*)p.k + (int64_t)kv_tok0 * row_bytes + hkv * (kHeadDim * 2);
-  const char* v_head = (const char*)p.v + (int64_t)kv_tok0 * row_bytes + hkv * (kHeadDim * 2);
+  const char* k_head = (const char*)p.k + (int64_t)kv_tok0 * row_bytes + hkv * p.t.kv_head_b;
+  const char* v_head = (const char*)p.v + (int64_t)kv_tok0 * row_bytes + hkv * p.t.kv_head_b;
   auto issue = [&](const char* head, const char* tensor, int kt, uint32_t dst) __attribute__((always_inline)) {
     const int key0 = kt * TN;
     const bool full = (key0 + TN <= nkeys) && (kv_tok0 + key0 + TN <= p.t.S);
@@ -94,7 +94,7 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
         const int slab = 4 * i + wave_u;
         const int key = 4 * slab + ld_kin;
         const int64_t tk = min((int64_t)kv_tok0 + key0 + key, (int64_t)p.t.S - 1);
-        async_copy16(tensor + tk * row_bytes + hkv * (kHeadDim * 2) + sw_col16(key, ld_pc) * 16, dst + slab * 1024);
+        async_copy16(tensor + tk * row_bytes + hkv * p.t.kv_head_b + sw_col16(key, ld_pc) * 16, dst + slab * 1024);
       }
     }
   };
@@ -453,7 +453,8 @@ extern "C" int moba_fwd_partials(const void* q, const void* k, const void* v, vo
                                  const int32_t* fchunk_tok, const int32_t* chunk_tok,
                                  const int32_t* self_tile_prefix, const int32_t* tile_seg,
                                  const int32_t* self_tile_chunk, int64_t S, int H, int Hkv, int D, int K, int F,
-                                 int N, int B, int64_t hist_bound, int64_t self_tiles, int dtype, void* stream) {
+                                 int N, int B, int64_t hist_bound, int64_t self_tiles, const int64_t* strides,
+                                 int dtype, void* stream) {
   if (!q || !k || !v || !part_o || !part_lse || !chunk_tok || !self_tile_prefix || !self_tile_chunk) return MOBA_ERR_ARG;
   if (Hkv <= 0 || H % Hkv != 0) return MOBA_ERR_ARG;
   if (K > 0 && (!seg_off || !tile_off || !seg_dest || !fchunk_tok || !tile_seg)) return MOBA_ERR_ARG;
@@ -472,6 +473,7 @@ extern "C" int moba_fwd_partials(const void* q, const void* k, const void* v, vo
   t.Hkv = Hkv; t.rep = H / Hkv;
   t.hist_bound = (K > 0) ? (int)hist_bound : 0;
   t.self_total = (int)(self_tiles * H);
+  if (!set_layout(t, strides)) return MOBA_ERR_ARG;
   hipStream_t st = (hipStream_t)stream;
   return dtype == MOBA_DTYPE_F16 ? launch_partials<F16>(q, k, v, part_o, part_lse, t, D, grid, st)
                                  : launch_partials<Bf16>(q, k, v, part_o, part_lse, t, D, grid, st);
@@ -499,10 +501,10 @@ extern "C" int moba_fwd(const void* q, const void* k, const void* v, void* part_
                         const int32_t* seg_dest, const int32_t* fchunk_tok, const int32_t* chunk_tok,
                         const int32_t* self_tile_prefix, const int32_t* tile_seg, const int32_t* self_tile_chunk,
                         void* out, float* lse, int64_t S, int H, int Hkv, int D, int K, int F, int N, int B,
-                        int64_t hist_bound, int64_t self_tiles, int dtype, void* stream) {
+                        int64_t hist_bound, int64_t self_tiles, const int64_t* strides, int dtype, void* stream) {
   int rc = moba_fwd_partials(q, k, v, part_o, part_lse, seg_off, tile_off, seg_dest, fchunk_tok, chunk_tok,
                              self_tile_prefix, tile_seg, self_tile_chunk, S, H, Hkv, D, K, F, N, B, hist_bound,
-                             self_tiles, dtype, stream);
+                             self_tiles, strides, dtype, stream);
   if (rc != MOBA_OK) return rc;
   return moba_fwd_merge(part_o, part_lse, sel, out, lse, S, H, D, K, dtype, stream);
 }

@@ -45,6 +45,40 @@ def _aligned(t: torch.Tensor) -> torch.Tensor:
     return t if t.data_ptr() % 16 == 0 else t.clone()
 
 
+def _row_strides(t: torch.Tensor):
+    """(token stride, head stride) in elements of a [tokens, heads, head_dim] tensor; the stride of a
+    dimension of size 1 means nothing and is replaced by the packed one."""
+    S, H, D = t.shape
+    return (t.stride(0) if S > 1 else H * D), (t.stride(1) if H > 1 else D)
+
+
+def _addressable(t: torch.Tensor) -> bool:
+    """The kernels read 16 bytes per lane from rows of head_dim contiguous elements: any token and head
+    strides that keep those reads aligned are read in place (a slice of a packed qkv projection, a
+    [heads, tokens, head_dim] cache seen as [tokens, heads, head_dim], ...), as flash-attn does for
+    the reference (moba/moba_efficient.py:89-128 hands such views straight to it)."""
+    ts, hs = _row_strides(t)
+    return (t.stride(2) == 1 and ts > 0 and hs > 0 and ts % 8 == 0 and hs % 8 == 0 and ts <= 1 << 23
+            and t.data_ptr() % 16 == 0)
+
+
+def _in_place(q, k, v):
+    """q, k, v as the kernels will read them: untouched where addressable (k and v must share their
+    strides), packed copies otherwise."""
+    if not _addressable(q):
+        q = _aligned(q)
+    if not (_addressable(k) and _addressable(v) and _row_strides(k) == _row_strides(v)):
+        k, v = _aligned(k), _aligned(v)
+    return q, k, v
+
+
+def _strides(q: Optional[torch.Tensor], k: Optional[torch.Tensor]):
+    """The strides argument of the C ABI: {q token, q head, k/v token, k/v head} in elements."""
+    qs = _row_strides(q) if q is not None else (HEAD_DIM, HEAD_DIM)
+    ks = _row_strides(k) if k is not None else (HEAD_DIM, HEAD_DIM)
+    return (ctypes.c_int64 * 4)(qs[0], qs[1], ks[0], ks[1])
+
+
 def _check_qkv(q, k, v, gqa=False):
     if not (q.is_cuda and k.is_cuda and v.is_cuda):
         raise RuntimeError("moba_attn_varlen needs tensors on an AMD GPU (there is no CPU path)")
@@ -66,11 +100,14 @@ def chunk_mean(k: torch.Tensor, plan: MobaPlan) -> torch.Tensor:
     """kbar [F, H, D] in k's dtype: mean of K over every filtered chunk (exact sum, rounded once)."""
     lib = _lib.load()
     S, H, D = k.shape
+    if not _addressable(k):
+        k = _aligned(k)
     kbar = torch.empty((plan.F, H, D), dtype=k.dtype, device=k.device)
     nbytes = lib.moba_chunk_mean_workspace_bytes(H, D, plan.F, plan.chunk_size)
     ws = torch.empty(nbytes // 8, dtype=torch.float64, device=k.device)
     _lib.check(lib.moba_chunk_mean(_ptr(k), _ptr(plan.tables["fchunk_tok"]), _ptr(kbar), _ptr(ws), S, H, D, plan.F,
-                                   plan.chunk_size, _dtype_code(k), _stream(k.device)), "moba_chunk_mean")
+                                   plan.chunk_size, _strides(None, k), _dtype_code(k), _stream(k.device)),
+               "moba_chunk_mean")
     return kbar
 
 
@@ -80,13 +117,15 @@ def gate_topk(q: torch.Tensor, kbar: torch.Tensor, plan: MobaPlan, return_scores
     lib = _lib.load()
     S, H, D = q.shape
     Hkv = kbar.shape[1]
+    if not _addressable(q):
+        q = _aligned(q)
     sel = torch.empty((S, H, plan.K), dtype=torch.int32, device=q.device)
     scores = None
     if return_scores:
         scores = torch.full((S, H, plan.F), float("-inf"), dtype=torch.float32, device=q.device)
     _lib.check(lib.moba_gate_topk(_ptr(q), _ptr(kbar), _ptr(plan.tables["cu_seqlens"]), _ptr(plan.tables["seq_fbase"]),
                                   _ptr(sel), _ptr(scores), S, H, Hkv, D, plan.nseq, plan.F, plan.chunk_size, plan.K,
-                                  _dtype_code(q), _stream(q.device)), "moba_gate_topk")
+                                  _strides(q, None), _dtype_code(q), _stream(q.device)), "moba_gate_topk")
     return (sel, scores) if return_scores else sel
 
 
@@ -176,15 +215,15 @@ def _forward(q, k, v, plan: MobaPlan, timer: Optional[StageTimer] = None):
             seg_off, tile_off, seg_dest, tile_seg = build_lists(sel, plan)
     part_o = torch.empty((S * H * (K + 1), D), dtype=q.dtype, device=dev)
     part_lse = torch.empty((S * H * (K + 1),), dtype=torch.float32, device=dev)
-    out = torch.empty_like(q)
+    out = torch.empty((S, H, D), dtype=q.dtype, device=dev)
     lse = torch.empty((S, H), dtype=torch.float32, device=dev)
     with span("fwd_partials"):
         _lib.check(lib.moba_fwd_partials(_ptr(q), _ptr(k), _ptr(v), _ptr(part_o), _ptr(part_lse), _ptr(seg_off),
                                          _ptr(tile_off), _ptr(seg_dest), _ptr(t.get("fchunk_tok")),
                                          _ptr(t["chunk_tok"]), _ptr(t["self_tile_prefix"]), _ptr(tile_seg),
                                          _ptr(t["self_tile_chunk"]), S, H, k.shape[1], D, K, plan.F, plan.N,
-                                         plan.chunk_size, plan.hist_tile_bound(H), plan.self_tiles, _dtype_code(q),
-                                         _stream(dev)), "moba_fwd_partials")
+                                         plan.chunk_size, plan.hist_tile_bound(H), plan.self_tiles, _strides(q, k),
+                                         _dtype_code(q), _stream(dev)), "moba_fwd_partials")
     with span("fwd_merge"):
         _lib.check(lib.moba_fwd_merge(_ptr(part_o), _ptr(part_lse), _ptr(sel), _ptr(out), _ptr(lse), S, H, D, K,
                                       _dtype_code(q), _stream(dev)), "moba_fwd_merge")
@@ -197,9 +236,9 @@ def _backward(dout, q, k, v, out, lse, sel, seg_off, tile_off, seg_dest, tile_se
     dev = q.device
     K = plan.K
     t = plan.tables
-    dq = torch.empty_like(q)
-    dk = torch.empty_like(k)
-    dv = torch.empty_like(v)
+    dq = torch.empty(q.shape, dtype=q.dtype, device=dev)  # packed, whatever the strides of q, k, v
+    dk = torch.empty(k.shape, dtype=k.dtype, device=dev)
+    dv = torch.empty(v.shape, dtype=v.dtype, device=dev)
     delta = torch.empty((2, S, H), dtype=torch.float32, device=dev)
     part_dq = torch.empty((S * H * (K + 1), D), dtype=torch.float32, device=dev)
     _lib.check(lib.moba_bwd(_ptr(dout), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(sel), _ptr(seg_off),
@@ -207,7 +246,7 @@ def _backward(dout, q, k, v, out, lse, sel, seg_off, tile_off, seg_dest, tile_se
                             _ptr(t["self_tile_prefix"]), _ptr(tile_seg), _ptr(t["self_tile_chunk"]),
                             _ptr(t.get("chunk_fid")), _ptr(delta), _ptr(part_dq), _ptr(dq), _ptr(dk), _ptr(dv),
                             S, H, k.shape[1], D, K, plan.F, plan.N, plan.chunk_size, plan.hist_tile_bound(H),
-                            plan.self_tiles, _dtype_code(q), _stream(dev)), "moba_bwd")
+                            plan.self_tiles, _strides(q, k), _dtype_code(q), _stream(dev)), "moba_bwd")
     return dq, dk, dv
 
 
@@ -277,6 +316,5 @@ def moba_attn_varlen_with_lse(q, k, v, cu_seqlens, max_seqlen, moba_chunk_size, 
     plan = make_plan(cu_seqlens, moba_chunk_size, moba_topk, device=q.device)
     if plan.S != q.shape[0]:
         raise ValueError(f"cu_seqlens ends at {plan.S} but q has {q.shape[0]} tokens")
-    # the kernels read 16 bytes per lane: contiguous rows at 16-byte aligned addresses
-    q, k, v = (_aligned(x) for x in (q, k, v))
+    q, k, v = _in_place(q, k, v)
     return _MobaAttention.apply(q, k, v, plan, timer)

@@ -256,3 +256,69 @@ def test_argument_validation():
         moba_attn_varlen(q, q, q, torch.tensor([0, 32], dtype=torch.int32, device="cuda"), 64, 16, 2)
     with pytest.raises(RuntimeError):
         moba_attn_varlen(q.cpu(), q.cpu(), q.cpu(), cu, 64, 16, 2)
+
+
+@pytest.mark.parametrize("layout", ["qkv_slices", "head_major", "gqa_head_major", "mixed", "unaligned"])
+def test_strided_inputs(layout):
+    """q, k, v that are views with token and head strides (slices of a fused qkv projection, a
+    [heads, tokens, dim] cache seen token-first) are read where they lie -- flash-attn does the same
+    for the reference (moba/moba_efficient.py:89-128) -- and give bit for bit the result and the
+    gradients of packed copies.  Layouts the kernels cannot address are copied, with the same result."""
+    from moba_amd import moba_attn_varlen, moba_attn_varlen_gqa
+    from moba_amd import moba_efficient as E
+
+    seqlen, heads, B, topk = 3000, 4, 256, 3
+    kv_heads = 2 if layout == "gqa_head_major" else heads
+    q, _, _, do, cu, mx = make_case(3, seqlen, heads, seed=21)
+    _, k, v, _, _, _ = make_case(3, seqlen, kv_heads, seed=22)
+    cu_t = torch.tensor(cu, dtype=torch.int32, device="cuda")
+    op = moba_attn_varlen_gqa if kv_heads != heads else moba_attn_varlen
+    in_place = True
+    if layout == "qkv_slices":
+        base = torch.stack([q, k, v], dim=1).cuda().requires_grad_(True)       # [S, 3, H, D]
+        views = [base[:, 0], base[:, 1], base[:, 2]]
+    elif layout in ("head_major", "gqa_head_major"):
+        leaves = [x.cuda().transpose(0, 1).contiguous().requires_grad_(True) for x in (q, k, v)]   # [H, S, D]
+        views = [x.transpose(0, 1) for x in leaves]
+    elif layout == "mixed":   # k token-major, v head-major: their strides differ, so both are copied
+        leaves = [q.cuda().requires_grad_(True), k.cuda().requires_grad_(True),
+                  v.cuda().transpose(0, 1).contiguous().requires_grad_(True)]
+        views = [leaves[0], leaves[1], leaves[2].transpose(0, 1)]
+    else:                     # rows that start 8 bytes into a 16-byte line
+        leaves = [torch.zeros(x.numel() + 4, dtype=x.dtype, device="cuda") for x in (q, k, v)]
+        views = []
+        for buf, x in zip(leaves, (q, k, v)):
+            buf[4:].copy_(x.cuda().reshape(-1))
+            views.append(buf[4:].view(x.shape).requires_grad_(True))
+        in_place = False
+    got = E._in_place(*views)
+    if layout in ("qkv_slices", "head_major", "gqa_head_major"):
+        assert all(a is b for a, b in zip(got, views))
+    elif layout == "mixed":
+        assert got[0] is views[0] and got[1].is_contiguous() and got[2].is_contiguous()
+    else:
+        assert not in_place and all(a.data_ptr() % 16 == 0 for a in got)
+
+    out = op(views[0], views[1], views[2], cu_t, mx, B, topk)
+    out.backward(do.cuda())
+    qc, kc, vc = (x.cuda().requires_grad_(True) for x in (q, k, v))
+    want = op(qc, kc, vc, cu_t, mx, B, topk)
+    want.backward(do.cuda())
+    assert out.is_contiguous() and torch.equal(out, want)
+    if layout == "qkv_slices":
+        grads = [base.grad[:, 0], base.grad[:, 1], base.grad[:, 2]]
+    elif layout in ("head_major", "gqa_head_major"):
+        grads = [x.grad.transpose(0, 1) for x in leaves]
+    elif layout == "mixed":
+        grads = [leaves[0].grad, leaves[1].grad, leaves[2].grad.transpose(0, 1)]
+    else:
+        grads = [x.grad for x in views]
+    for g, w in zip(grads, (qc.grad, kc.grad, vc.grad)):
+        assert torch.equal(g, w)
+
+    # the stages on their own
+    from moba_amd.plan import make_plan
+    plan = make_plan(cu_t, B, topk)
+    kbar = E.chunk_mean(views[1].detach(), plan)
+    assert torch.equal(kbar, E.chunk_mean(kc.detach(), plan))
+    assert torch.equal(E.gate_topk(views[0].detach(), kbar, plan), E.gate_topk(qc.detach(), kbar, plan))
