@@ -168,7 +168,10 @@ def main():
         E.moba_attn_varlen_with_lse(q, k, v, cu_t, max_seqlen, B, topk, timer=timer, gqa=args.gqa)
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / args.steps
-    stage_ms = {name: sum(x) / len(x) for name, x in timer.ms().items()}
+    per_stage = timer.ms()
+    stage_ms = {name: sum(x) / len(x) for name, x in per_stage.items()}
+    # device time of each step (sum of its stage spans): median and minimum over the timed steps
+    step_ms = sorted(sum(x[i] for x in per_stage.values()) for i in range(args.steps))
 
     # forward + backward (reported beside the forward figure for the workloads that name it)
     fwd_bwd_ms = None
@@ -207,6 +210,7 @@ def main():
                    "sequences": len(cu) - 1, "fwd_flops": flops},
         "pct_mfma_peak_whole_op": 100.0 * flops / dt / 1e12 / MFMA_BF16_PEAK_TFLOPS,
         "stage_ms": stage_ms,
+        "device_ms_per_step": {"median": step_ms[len(step_ms) // 2], "min": step_ms[0]},
         "roofline": {"kernel": "moba_fwd_kernel", "bound": "mfma", "achieved": achieved,
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
                      "traffic": FWD_KERNEL_TRAFFIC_BYTES.get(args.workload)},
