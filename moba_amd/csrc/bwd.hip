@@ -661,15 +661,10 @@ static int launch_bwd(const void* dout, const void* q, const void* k, const void
   p.hk_shift = 31 + lg;
   p.hk_magic = (uint32_t)((1ull << p.hk_shift) / hk + 1);
 
-  static bool attr_set = false;  // one flag per element type
-  if (!attr_set) {
-    if (hipFuncSetAttribute((const void*)bwd_dq_kernel<E>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdDqLds) !=
-            hipSuccess ||
-        hipFuncSetAttribute((const void*)bwd_dkv_kernel<E>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdDkvLds) !=
-            hipSuccess)
-      return MOBA_ERR_LAUNCH;
-    attr_set = true;
-  }
+  static bool allowed_dq[kMaxDevices], allowed_dkv[kMaxDevices];  // one pair per element type
+  if (!allow_dynamic_lds((const void*)bwd_dq_kernel<E>, kBwdDqLds, allowed_dq) ||
+      !allow_dynamic_lds((const void*)bwd_dkv_kernel<E>, kBwdDkvLds, allowed_dkv))
+    return MOBA_ERR_LAUNCH;
   const int64_t rows = S * H;
   hipLaunchKernelGGL(bwd_delta_kernel<E>, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st, (const elem*)dout,
                      (const elem*)out, lse, delta, delta + S * H, rows);

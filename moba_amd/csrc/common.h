@@ -72,6 +72,18 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, p);
 }
 
+// Dynamic LDS above 64 KiB must be allowed per kernel, and the allowance belongs to the current
+// device: `done` (one array per kernel) remembers the devices it was given on.
+constexpr int kMaxDevices = 64;
+inline bool allow_dynamic_lds(const void* kernel, int bytes, bool (&done)[kMaxDevices]) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0) return false;
+  if (dev < kMaxDevices && done[dev]) return true;
+  if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) return false;
+  if (dev < kMaxDevices) done[dev] = true;
+  return true;
+}
+
 // largest i in [0, n) with a[i] <= x, for ascending a with a[0] <= x
 __device__ __forceinline__ int upper_row(const int* __restrict__ a, int n, int x) {
   int lo = 0, hi = n;  // invariant: a[lo] <= x, a[hi] > x (hi == n means +inf)

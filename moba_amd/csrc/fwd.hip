@@ -436,13 +436,8 @@ static int launch_partials(const void* q, const void* k, const void* v, void* pa
   p.part_o = (typename E::elem*)part_o; p.part_lse = part_lse;
   p.t = t;
   p.scale_log2 = (float)(1.4426950408889634 / sqrt((double)D));
-  static bool attr_set = false;  // one flag per element type
-  if (!attr_set) {
-    if (hipFuncSetAttribute((const void*)moba_fwd_kernel<E>, hipFuncAttributeMaxDynamicSharedMemorySize, kFwdLds) !=
-        hipSuccess)
-      return MOBA_ERR_LAUNCH;
-    attr_set = true;
-  }
+  static bool allowed[kMaxDevices];  // one array per element type
+  if (!allow_dynamic_lds((const void*)moba_fwd_kernel<E>, kFwdLds, allowed)) return MOBA_ERR_LAUNCH;
   hipLaunchKernelGGL(moba_fwd_kernel<E>, dim3((unsigned)grid), dim3(256), kFwdLds, st, p);
   return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
 }
