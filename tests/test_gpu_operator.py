@@ -94,6 +94,8 @@ def test_reference_grid(chunk):
     (5, 2000, 2, 128, 64),     # topk beyond the chunk count: everything selected
     (6, 777, 5, 96, 2),        # odd sizes, 1-token tails
     (1, 8192, 1, 512, 3),
+    (1, 4096, 1, 64, 24),      # k = 23: the 32-entry selection lists
+    (2, 4096, 2, 32, 40),      # k = 39: the 64-entry selection lists, 64 chunks per sequence
 ])
 def test_edge_shapes(batch, seqlen, heads, B, topk):
     run_case(batch, seqlen, heads, B, topk, seed=7)
@@ -322,3 +324,14 @@ def test_strided_inputs(layout):
     kbar = E.chunk_mean(views[1].detach(), plan)
     assert torch.equal(kbar, E.chunk_mean(kc.detach(), plan))
     assert torch.equal(E.gate_topk(views[0].detach(), kbar, plan), E.gate_topk(qc.detach(), kbar, plan))
+
+
+def test_more_than_64_history_chunks_is_refused():
+    """The selection kernel keeps at most 64 candidates per row: a larger k is an error, not a wrong answer."""
+    from moba_amd import moba_attn_varlen
+    q, k, v, _, cu, mx = make_case(1, 4096, 1, seed=3)
+    cu_t = torch.tensor(cu, dtype=torch.int32, device="cuda")
+    with pytest.raises(RuntimeError, match="moba_gate_topk"):
+        moba_attn_varlen(q.cuda(), k.cuda(), v.cuda(), cu_t, mx, 32, 80)
+    out = moba_attn_varlen(q.cuda(), k.cuda(), v.cuda(), cu_t, mx, 32, 65)   # k = 64 is the last one served
+    assert torch.isfinite(out.float()).all()
