@@ -59,6 +59,7 @@ struct Tile {
   int limit;      // this lane's row attends keys <= limit
   int wave_min_limit, wave_max_limit;  // over the wave's 32 rows
   int rot;        // history tiles may visit their key tiles in any order: start offset
+  int base;       // history tile: index of row 0 in seg_dest; self tile: -(row 0 inside the chunk) - 1
 };
 
 // Workgroup ids are dealt round-robin to the 8 XCDs; give each XCD runs of kXcdBlock
@@ -68,8 +69,10 @@ __device__ __forceinline__ int logical_tile_id() {
   return ((y / kXcdBlock) * 8 + x) * kXcdBlock + (y % kXcdBlock);
 }
 
-// r = row of this lane inside the tile (wave*32 + lane%32).  Returns false for ids past the end.
-__device__ __forceinline__ bool decode_tile(const TileTables& p, int logical, int wave, int r, Tile& t) {
+// Tile decoding in two steps, so that a kernel can start the key/value copies (which need only the
+// wave-uniform part) before the per-row lookup has returned.
+// Step 1, wave-uniform: head, key range, number of rows.  Returns false for ids past the end.
+__device__ __forceinline__ bool decode_tile_head(const TileTables& p, int logical, Tile& t) {
   const int H = p.H;
   if (logical < p.hist_bound) {
     const int seg = p.tile_seg[logical];   // one lookup instead of a search in tile_off
@@ -77,15 +80,10 @@ __device__ __forceinline__ bool decode_tile(const TileTables& p, int logical, in
     const int tile = logical - p.tile_off[seg];
     const int f = seg / H;
     t.h = seg - f * H;
-    const int base = p.seg_off[seg] + tile * TM;
-    t.row_count = min(TM, p.seg_off[seg + 1] - base);
+    t.base = p.seg_off[seg] + tile * TM;
+    t.row_count = min(TM, p.seg_off[seg + 1] - t.base);
     t.kv_tok0 = p.fchunk_tok[f];
     t.nkeys = p.B;
-    t.dest = p.seg_dest[base + min(r, t.row_count - 1)];
-    t.tok = t.dest / (H * p.K1);
-    t.limit = t.nkeys - 1;
-    t.wave_min_limit = t.limit;
-    t.wave_max_limit = t.limit;
     t.rot = tile;
     return true;
   }
@@ -98,16 +96,34 @@ __device__ __forceinline__ bool decode_tile(const TileTables& p, int logical, in
   const int tin = nt - 1 - (rem - t.h * nt);  // longest tiles first
   const int c0 = p.chunk_tok[c];
   const int len = p.chunk_tok[c + 1] - c0;
-  const int r0 = tin * TM;
-  t.row_count = min(TM, len - r0);
+  t.base = -1 - tin * TM;                   // self tile: -(first row of the tile inside its chunk) - 1
+  t.row_count = min(TM, len - tin * TM);
   t.kv_tok0 = c0;
-  t.nkeys = min(len, r0 + TM);
-  t.tok = c0 + r0 + min(r, t.row_count - 1);
-  t.dest = (t.tok * H + t.h) * p.K1;
-  t.limit = r0 + min(r, t.row_count - 1);
-  t.wave_min_limit = r0 + min(wave * 32, t.row_count - 1);
-  t.wave_max_limit = r0 + min(wave * 32 + 31, t.row_count - 1);
+  t.nkeys = min(len, tin * TM + TM);
   t.rot = 0;
+  return true;
+}
+// Step 2, per row: r = row of this lane inside the tile (wave*32 + lane%32).
+__device__ __forceinline__ void decode_tile_rows(const TileTables& p, int wave, int r, Tile& t) {
+  const int H = p.H;
+  if (t.base >= 0) {
+    t.dest = p.seg_dest[t.base + min(r, t.row_count - 1)];
+    t.tok = t.dest / (H * p.K1);
+    t.limit = t.nkeys - 1;
+    t.wave_min_limit = t.limit;
+    t.wave_max_limit = t.limit;
+  } else {
+    const int r0 = -1 - t.base;
+    t.tok = t.kv_tok0 + r0 + min(r, t.row_count - 1);
+    t.dest = (t.tok * H + t.h) * p.K1;
+    t.limit = r0 + min(r, t.row_count - 1);
+    t.wave_min_limit = r0 + min(wave * 32, t.row_count - 1);
+    t.wave_max_limit = r0 + min(wave * 32 + 31, t.row_count - 1);
+  }
+}
+__device__ __forceinline__ bool decode_tile(const TileTables& p, int logical, int wave, int r, Tile& t) {
+  if (!decode_tile_head(p, logical, t)) return false;
+  decode_tile_rows(p, wave, r, t);
   return true;
 }
 

@@ -49,19 +49,15 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
   const int n = lane & 31, hh = lane >> 5;
   const int H = p.t.H;
 
+  // The wave-uniform half of the tile description is enough to start the key/value copies; the per-row
+  // lookup and the Q rows follow while those are in flight.
   Tile t;
   const int r = wave * 32 + n;
-  if (!decode_tile(p.t, logical_tile_id(), wave, r, t)) return;
-  const int h = t.h, nkeys = t.nkeys, kv_tok0 = t.kv_tok0, limit = t.limit;
+  if (!decode_tile_head(p.t, logical_tile_id(), t)) return;
+  const int h = t.h, nkeys = t.nkeys, kv_tok0 = t.kv_tok0;
   const bool row_valid = r < t.row_count;
-
-  // ---- Q^T operand: lane (n, hh) holds q[tok][16*ks + 8*hh .. +7] ----
+  int limit = 0;  // this lane's row attends keys <= limit (set with the per-row half below)
   elem8 bq[8];
-  {
-    const elem* src = reinterpret_cast<const elem*>((const char*)p.q + t.tok * p.t.q_tok_b + h * p.t.q_head_b) + 8 * hh;
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks) bq[ks] = *reinterpret_cast<const elem8*>(src + 16 * ks);
-  }
 
   // ---- K/V tile loader: global -> LDS without passing through registers.
   // A wave copy fills 1 KiB = 4 keys x 16 columns of 16 bytes; wave w issues slabs
@@ -183,6 +179,17 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
   issue_k(key_tile(0), 0);
   issue_v(key_tile(0), 0);
   if (nkt > 1) issue_k(key_tile(1), 1);
+
+  // ---- Q^T operand: lane (n, hh) holds q[tok][16*ks + 8*hh .. +7] ----
+  decode_tile_rows(p.t, wave, r, t);
+  limit = t.limit;
+  {
+    const elem* src = reinterpret_cast<const elem*>((const char*)p.q + t.tok * p.t.q_tok_b + h * p.t.q_head_b) + 8 * hh;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) bq[ks] = *reinterpret_cast<const elem8*>(src + 16 * ks);
+  }
+  // whether or not the row loads above are still among the newest operations, all copies but the last
+  // group (the second K tile) have landed after this
   wait_newer4(nkt > 1);
   scrub_v(key_tile(0), 0);
   __syncthreads();
@@ -339,10 +346,14 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
 #undef MOBA_PIN
 
   // ---- epilogue: normalise, write the partial ----
+  // The accumulators hold O^T (a lane owns 4-element pieces of one row); the rows go through this
+  // wave's 8 KiB of LDS (free since the barrier that ended the last tile) so that they leave as
+  // whole 256-byte rows, four per store instruction, instead of 8-byte pieces of 32 rows.
   const float l_tot = sum_xhalf(l_run);
   const float inv = 1.f / l_tot;
-  if (row_valid) {
-    elem* dst = p.part_o + (int64_t)t.dest * kHeadDim;
+  {
+    char* stage = smem + wave * 8192;
+    char* wrow = stage + n * 256 + 8 * hh;
 #pragma unroll
     for (int db = 0; db < 4; ++db)
 #pragma unroll
@@ -350,9 +361,19 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
         u32x2 w;
         w[0] = pack2<E>(oacc[db][4 * g + 0] * inv, oacc[db][4 * g + 1] * inv);
         w[1] = pack2<E>(oacc[db][4 * g + 2] * inv, oacc[db][4 * g + 3] * inv);
-        *reinterpret_cast<u32x2*>(dst + 32 * db + 8 * g + 4 * hh) = w;
+        // elements 32*db + 8*g + 4*hh .. +3 of row n: 16-byte column 4*db + g, swizzled by the row
+        *reinterpret_cast<u32x2*>(wrow + (((4 * db + g) ^ (n & 15)) << 4)) = w;
       }
-    if (hh == 0) p.part_lse[t.dest] = m_run + fast_log2(l_tot);
+    if (row_valid && hh == 0) p.part_lse[t.dest] = m_run + fast_log2(l_tot);
+    const int c16 = lane & 15;
+    const int rows_here = t.row_count - wave * 32;  // rows of this wave that exist
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int row = 4 * i + (lane >> 4);
+      const int dest = __shfl(t.dest, row, 64);
+      const u32x4 x = *reinterpret_cast<const u32x4*>(stage + row * 256 + ((c16 ^ (row & 15)) << 4));
+      if (row < rows_here) *reinterpret_cast<u32x4*>(p.part_o + (int64_t)dest * kHeadDim + c16 * 8) = x;
+    }
   }
 }
 
