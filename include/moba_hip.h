@@ -92,21 +92,25 @@ int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, const int32_t
  *   tile_seg: from moba_build_lists (may be NULL when K = 0)
  *   out [S,H,D] elem, lse [S,H] fp32 (natural log)
  *   hist_bound: upper bound on the number of history tiles, e.g. M/tile_rows + F*H
- *   self_tiles: self_tile_prefix[N] */
+ *   self_tiles: self_tile_prefix[N]
+ *   queues [8] int32 scratch: the tile counters of the forward kernel, whose workgroups (two per CU) stay
+ *              resident and draw tiles from one queue per XCD; the call zeroes them with a kernel of its own.
+ *              Calls that overlap in time need their own eight counters each. */
 int moba_fwd_tile_rows(void);
 int moba_fwd_partials(const void* q, const void* k, const void* v, void* part_o, float* part_lse,
                       const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest,
                       const int32_t* fchunk_tok, const int32_t* chunk_tok, const int32_t* self_tile_prefix,
                       const int32_t* tile_seg, const int32_t* self_tile_chunk, int64_t S, int H, int Hkv, int D, int K,
-                      int F, int N, int B, int64_t hist_bound, int64_t self_tiles, const int64_t* strides, int dtype,
-                      void* stream);
+                      int F, int N, int B, int64_t hist_bound, int64_t self_tiles, const int64_t* strides,
+                      int32_t* queues, int dtype, void* stream);
 int moba_fwd_merge(const void* part_o, const float* part_lse, const int32_t* sel, void* out, float* lse, int64_t S,
                    int H, int D, int K, int dtype, void* stream);
 int moba_fwd(const void* q, const void* k, const void* v, void* part_o, float* part_lse, const int32_t* sel,
              const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest, const int32_t* fchunk_tok,
              const int32_t* chunk_tok, const int32_t* self_tile_prefix, const int32_t* tile_seg,
              const int32_t* self_tile_chunk, void* out, float* lse, int64_t S, int H, int Hkv, int D, int K, int F,
-             int N, int B, int64_t hist_bound, int64_t self_tiles, const int64_t* strides, int dtype, void* stream);
+             int N, int B, int64_t hist_bound, int64_t self_tiles, const int64_t* strides, int32_t* queues, int dtype,
+             void* stream);
 
 /* Backward.  Replaces MixedAttention.backward, moba/moba_efficient.py:185-267, and the
  * autograd scatter of its gathered gradients.  Deterministic (no floating-point atomics).

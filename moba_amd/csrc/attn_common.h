@@ -69,14 +69,28 @@ __device__ __forceinline__ int logical_tile_id() {
   return ((y / kXcdBlock) * 8 + x) * kXcdBlock + (y % kXcdBlock);
 }
 
-// Tile decoding in two steps, so that a kernel can start the key/value copies (which need only the
-// wave-uniform part) before the per-row lookup has returned.
-// Step 1, wave-uniform: head, key range, number of rows.  Returns false for ids past the end.
-__device__ __forceinline__ bool decode_tile_head(const TileTables& p, int logical, Tile& t) {
+// Tile decoding in steps, so that a kernel can start the key/value copies (which need only the
+// wave-uniform part) before the per-row lookup has returned, and so that a kernel that walks many
+// tiles can keep the lookups of later tiles in flight behind the work on the current one.
+// Step 0, wave-uniform: the one entry of the big tables.  History tile: its segment (-1 for an unused
+// id below hist_bound); self tile: its chunk; -2 past the last tile.
+constexpr int kTileUnused = -1, kTilePastEnd = -2;
+__device__ __forceinline__ int decode_tile_code(const TileTables& p, int logical) {
+  if (logical < 0) return kTileUnused;
+  if (logical < p.hist_bound) return p.tile_seg[logical];
+  const int st = logical - p.hist_bound;
+  if (st >= p.self_total) return kTilePastEnd;
+  return p.self_tile_chunk[st / p.H];  // self_tile_prefix[c]*H <= st < self_tile_prefix[c+1]*H
+}
+// Step 1, wave-uniform: head, key range, number of rows, from the small per-segment / per-chunk tables.
+// Returns false (and row_count = 0) for a code that is not a tile.
+__device__ __forceinline__ bool decode_tile_head(const TileTables& p, int logical, int code, Tile& t) {
   const int H = p.H;
+  t.row_count = 0;
+  t.base = -1;
+  if (code < 0) return false;
   if (logical < p.hist_bound) {
-    const int seg = p.tile_seg[logical];   // one lookup instead of a search in tile_off
-    if (seg < 0) return false;
+    const int seg = code;
     const int tile = logical - p.tile_off[seg];
     const int f = seg / H;
     t.h = seg - f * H;
@@ -88,8 +102,7 @@ __device__ __forceinline__ bool decode_tile_head(const TileTables& p, int logica
     return true;
   }
   const int st = logical - p.hist_bound;
-  if (st >= p.self_total) return false;
-  const int c = p.self_tile_chunk[st / H];  // self_tile_prefix[c]*H <= st < self_tile_prefix[c+1]*H
+  const int c = code;
   const int rem = st - p.self_tile_prefix[c] * H;
   const int nt = p.self_tile_prefix[c + 1] - p.self_tile_prefix[c];
   t.h = rem / nt;
@@ -103,11 +116,18 @@ __device__ __forceinline__ bool decode_tile_head(const TileTables& p, int logica
   t.rot = 0;
   return true;
 }
-// Step 2, per row: r = row of this lane inside the tile (wave*32 + lane%32).
-__device__ __forceinline__ void decode_tile_rows(const TileTables& p, int wave, int r, Tile& t) {
+__device__ __forceinline__ bool decode_tile_head(const TileTables& p, int logical, Tile& t) {
+  return decode_tile_head(p, logical, decode_tile_code(p, logical), t);
+}
+// Step 2a, per row: the gather-list entry of row r (history tiles; self tiles need no lookup).
+__device__ __forceinline__ int decode_tile_row_entry(const TileTables& p, int r, const Tile& t) {
+  return (t.row_count > 0 && t.base >= 0) ? p.seg_dest[t.base + min(r, t.row_count - 1)] : 0;
+}
+// Step 2b, per row: everything else from that entry.  r = row of this lane inside the tile (wave*32 + lane%32).
+__device__ __forceinline__ void decode_tile_rows(const TileTables& p, int wave, int r, int entry, Tile& t) {
   const int H = p.H;
   if (t.base >= 0) {
-    t.dest = p.seg_dest[t.base + min(r, t.row_count - 1)];
+    t.dest = entry;
     t.tok = t.dest / (H * p.K1);
     t.limit = t.nkeys - 1;
     t.wave_min_limit = t.limit;
@@ -120,6 +140,9 @@ __device__ __forceinline__ void decode_tile_rows(const TileTables& p, int wave, 
     t.wave_min_limit = r0 + min(wave * 32, t.row_count - 1);
     t.wave_max_limit = r0 + min(wave * 32 + 31, t.row_count - 1);
   }
+}
+__device__ __forceinline__ void decode_tile_rows(const TileTables& p, int wave, int r, Tile& t) {
+  decode_tile_rows(p, wave, r, decode_tile_row_entry(p, r, t), t);
 }
 __device__ __forceinline__ bool decode_tile(const TileTables& p, int logical, int wave, int r, Tile& t) {
   if (!decode_tile_head(p, logical, t)) return false;

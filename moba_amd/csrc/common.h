@@ -72,6 +72,20 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, p);
 }
 
+// A fresh copy of a piece of the running kernel's argument block, read where this is called.  A kernel
+// that needs some arguments only now and then (table pointers at a tile switch) reads them again there
+// instead of holding them in scalar registers all through its inner loop.  `offset` is the byte offset
+// of the piece inside the kernel's (single, by-value) parameter.
+template <class T>
+__device__ __forceinline__ T kernarg_now(int offset) {
+  typedef __attribute__((address_space(4))) const char* kernarg_ptr;
+  kernarg_ptr kp = (kernarg_ptr)__builtin_amdgcn_kernarg_segment_ptr();
+  asm volatile("" : "+s"(kp));  // not the pointer the compiler knows: the loads stay where they are written
+  T x;
+  __builtin_memcpy(&x, kp + offset, sizeof(T));
+  return x;
+}
+
 // Dynamic LDS above 64 KiB must be allowed per kernel, and the allowance belongs to the current
 // device: `done` (one array per kernel) remembers the devices it was given on.
 constexpr int kMaxDevices = 64;
@@ -82,6 +96,18 @@ inline bool allow_dynamic_lds(const void* kernel, int bytes, bool (&done)[kMaxDe
   if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) return false;
   if (dev < kMaxDevices) done[dev] = true;
   return true;
+}
+
+// compute units of the current device (0 on error), asked once per device
+inline int compute_units() {
+  static int count[kMaxDevices];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0) return 0;
+  if (dev < kMaxDevices && count[dev] > 0) return count[dev];
+  int n = 0;
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 0;
+  if (dev < kMaxDevices) count[dev] = n;
+  return n;
 }
 
 // largest i in [0, n) with a[i] <= x, for ascending a with a[0] <= x

@@ -15,12 +15,16 @@
 //
 // Algorithmic work: 4*D flops per attended (query, key) pair; the bound is the bf16
 // MFMA rate.  Compulsory HBM traffic is q, k, v once, the partials once each way.
+#include <cstddef>
 #include <type_traits>
 #include "attn_common.h"
 
 namespace moba {
 
-constexpr int kFwdLds = 4 * kTileBytes;  // K[2], V[2]
+// LDS: K[2], V[2] stages, then 256 bytes per wave for the gather-list entries of the next tile's rows,
+// then the slot through which wave 0 hands the tile id it drew to the other waves
+constexpr int kFwdEntries = 4 * kTileBytes, kFwdIdSlot = kFwdEntries + 4 * 256;
+constexpr int kFwdLds = kFwdIdSlot + 16;
 
 template <class E>
 struct FwdParams {
@@ -31,6 +35,7 @@ struct FwdParams {
   float* part_lse;  // [S*H*K1], log2 domain
   TileTables t;
   float scale_log2;  // D^-0.5 * log2(e)
+  int* queues;       // [8] tile counters, one per XCD, zero when the kernel starts
 };
 
 constexpr float kRescaleThreshold = 8.f;  // log2 units: the running max may lag the true max by this much
@@ -49,21 +54,29 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
   const int n = lane & 31, hh = lane >> 5;
   const int H = p.t.H;
 
-  // The wave-uniform half of the tile description is enough to start the key/value copies; the per-row
-  // lookup and the Q rows follow while those are in flight.
-  Tile t;
+  // The workgroups (two per CU, all resident) draw tiles from eight queues, one per XCD: queue x hands
+  // out the ids (8i + x) * kXcdBlock + j in order, so that the tiles in flight on an XCD are consecutive ids
+  // -- tiles that share a K/V chunk behind one L2 -- and an XCD that runs ahead (they differ by a few
+  // percent) goes on with the next queue when its own is empty.  A tile's description takes dependent
+  // lookups: the id (an atomic), the big table, the small tables, the gather-list entry of every row.
+  // They run three, two and one tile ahead of the tile being computed, each issued at one tile switch
+  // and used at the next; the entries travel global -> LDS, so nothing of this occupies vector registers.
   const int r = wave * 32 + n;
-  if (!decode_tile_head(p.t, logical_tile_id(), t)) return;
-  const int h = t.h, nkeys = t.nkeys, kv_tok0 = t.kv_tok0;
-  const bool row_valid = r < t.row_count;
-  int limit = 0;  // this lane's row attends keys <= limit (set with the per-row half below)
+  Tile t, t1;              // the tile being computed; the next one (its row entries on their way to LDS)
+  int id2 = -1, code2 = kTileUnused;   // id and first lookup of the tile after next
+  int id3 = -1;                        // id of the tile after that, as drawn
+  int queue = blockIdx.x & 7, empty_queues = 0;
+  t.row_count = 0; t.nkeys = 0; t.base = -1; t1 = t;   // row_count 0: not a tile; nkeys < 0: no tiles left
+  int h = 0, nkeys = 0, kv_tok0 = 0, hkv = 0;
+  int min_limit = 0;       // smallest row limit of the wave's 32 rows
+  bool row_valid = false;
+  int limit = 0;           // this lane's row attends keys <= limit
   elem8 bq[8];
 
   // ---- K/V tile loader: global -> LDS without passing through registers.
   // A wave copy fills 1 KiB = 4 keys x 16 columns of 16 bytes; wave w issues slabs
   // w, w+4, w+8, w+12.  Lane i lands at slab + 16*i, so the lane picks the global column
   // whose swizzled LDS position is i.  LDS: K stages at 0 and 16 KiB, V stages at 32 and 48 KiB.
-  const int hkv = h / p.t.rep;                                   // key/value head of this query head
   const int64_t row_bytes = p.t.kv_tok_b;                        // from one K or V token to the next
   const uint32_t lds_base = lds_addr(smem);
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
@@ -75,8 +88,8 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
     const int key = 4 * (4 * i + wave_u) + ld_kin;
     ld_off[i] = (uint32_t)(key * row_bytes + sw_col16(key, ld_pc) * 16);  // the swizzle is an involution
   }
-  const char* k_head = (const char*)p.k + (int64_t)kv_tok0 * row_bytes + hkv * p.t.kv_head_b;
-  const char* v_head = (const char*)p.v + (int64_t)kv_tok0 * row_bytes + hkv * p.t.kv_head_b;
+  const char* k_head = nullptr;  // key 0 of the current tile's key range, this tile's key/value head
+  const char* v_head = nullptr;
   auto issue = [&](const char* head, const char* tensor, int kt, uint32_t dst) __attribute__((always_inline)) {
     const int key0 = kt * TN;
     const bool full = (key0 + TN <= nkeys) && (kv_tok0 + key0 + TN <= p.t.S);
@@ -85,10 +98,14 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
 #pragma unroll
       for (int i = 0; i < 4; ++i) async_copy16_sv(base, ld_off[i], dst + (4 * i + wave_u) * 1024);
     } else {
+      // (rare path: its per-lane constants are derived here, from a value the compiler cannot trace, so
+      // that they are not computed ahead of the tile loop and carried through it in registers)
+      int kin = ld_kin;
+      asm volatile("" : "+v"(kin));
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int slab = 4 * i + wave_u;
-        const int key = 4 * slab + ld_kin;
+        const int key = 4 * slab + kin;
         const int64_t tk = min((int64_t)kv_tok0 + key0 + key, (int64_t)p.t.S - 1);
         async_copy16(tensor + tk * row_bytes + hkv * p.t.kv_head_b + sw_col16(key, ld_pc) * 16, dst + slab * 1024);
       }
@@ -101,11 +118,13 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
     const int key0 = kt * TN;
     if (key0 + TN <= nkeys) return;
     char* vdst = smem + (2 + stage) * kTileBytes;
+    int ln = lane;  // rare path: see the remark in the loader
+    asm volatile("" : "+v"(ln));
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int slab = 4 * i + wave;
-      const int key = 4 * slab + ld_kin;
-      if (key0 + key >= nkeys) *reinterpret_cast<u32x4*>(vdst + slab * 1024 + lane * 16) = u32x4{0, 0, 0, 0};
+      const int slab = 4 * i + wave_u;
+      const int key = 4 * slab + (ln >> 4);
+      if (key0 + key >= nkeys) *reinterpret_cast<u32x4*>(vdst + slab * 1024 + ln * 16) = u32x4{0, 0, 0, 0};
     }
   };
   auto wait_newer4 = [&](bool newer_issued) __attribute__((always_inline)) {  // all copies landed except the newest group of 4
@@ -114,8 +133,7 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
 
   // Tiles that run side by side on an XCD work on the same chunk; starting each at a
   // different key tile spreads their first touches of the chunk over all of it.
-  const int nkt = (nkeys + TN - 1) / TN;
-  const int rot = t.rot % nkt;
+  int nkt = 1, rot = 0;
   auto key_tile = [&](int it) __attribute__((always_inline)) { const int x = it + rot; return x >= nkt ? x - nkt : x; };
 
   // ---- fragment addressing: per-lane byte offsets inside a tile, everything else is an immediate ----
@@ -175,24 +193,120 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
 // keeps a value, and therefore the instructions that produce it, at this point of the program
 #define MOBA_PIN(x) asm volatile("" : "+v"(x))
 
-  // ---- prologue ----
-  issue_k(key_tile(0), 0);
-  issue_v(key_tile(0), 0);
-  if (nkt > 1) issue_k(key_tile(1), 1);
-
-  // ---- Q^T operand: lane (n, hh) holds q[tok][16*ks + 8*hh .. +7] ----
-  decode_tile_rows(p.t, wave, r, t);
-  limit = t.limit;
-  {
-    const elem* src = reinterpret_cast<const elem*>((const char*)p.q + t.tok * p.t.q_tok_b + h * p.t.q_head_b) + 8 * hh;
+  bool have_partial = false;  // the accumulators hold a finished tile whose partial is not written yet
+  int dest_done = 0, rows_done = 0;
+  bool valid_done = false;
+  while (true) {
+  // ================= tile switch =================
+  wait_vmem();  // nothing of this wave is in flight any more: the next tile's row entries are in LDS
+  if (have_partial) {
+    // ---- the finished tile's partial: normalise, write ----
+    // The accumulators hold O^T (a lane owns 4-element pieces of one row); the rows go through this
+    // wave's 8 KiB of LDS (free since the barrier that ended the tile) so that they leave as whole
+    // 256-byte rows, four per store instruction, instead of 8-byte pieces of 32 rows.
+    const FwdParams<E> pn = kernarg_now<FwdParams<E>>(0);
+    int ln = lane;  // taken afresh: none of the addresses below is computed ahead of the tile loop
+    asm volatile("" : "+v"(ln));
+    const int en = ln & 31, ehh = ln >> 5;
+    const float l_tot = sum_xhalf(l_run);
+    const float inv = 1.f / l_tot;
+    char* stage = smem + wave_u * 8192;
+    char* wrow = stage + en * 256 + 8 * ehh;
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) bq[ks] = *reinterpret_cast<const elem8*>(src + 16 * ks);
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        u32x2 w;
+        w[0] = pack2<E>(oacc[db][4 * g + 0] * inv, oacc[db][4 * g + 1] * inv);
+        w[1] = pack2<E>(oacc[db][4 * g + 2] * inv, oacc[db][4 * g + 3] * inv);
+        // elements 32*db + 8*g + 4*hh .. +3 of row n: 16-byte column 4*db + g, swizzled by the row
+        *reinterpret_cast<u32x2*>(wrow + (((4 * db + g) ^ (en & 15)) << 4)) = w;
+      }
+    if (valid_done && ehh == 0) pn.part_lse[dest_done] = m_run + fast_log2(l_tot);
+    const int c16 = ln & 15;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int row = 4 * i + (ln >> 4);
+      const int dest = __shfl(dest_done, row, 64);
+      const u32x4 x = *reinterpret_cast<const u32x4*>(stage + row * 256 + ((c16 ^ (row & 15)) << 4));
+      if (row < rows_done) *reinterpret_cast<u32x4*>(pn.part_o + (int64_t)dest * kHeadDim + c16 * 8) = x;
+    }
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) oacc[db][e] = 0.f;
+    m_run = -INFINITY;
+    l_run = 0.f;
+    __syncthreads();  // the K stages take the next tile's copies only after every wave has read its rows back
   }
-  // whether or not the row loads above are still among the newest operations, all copies but the last
-  // group (the second K tile) have landed after this
-  wait_newer4(nkt > 1);
-  scrub_v(key_tile(0), 0);
+  int drawn = 0;  // wave 0, lane 0: the value of the queue's counter
+  {
+    const FwdParams<E> pn = kernarg_now<FwdParams<E>>(0);
+    int tx = threadIdx.x;  // taken afresh, as above
+    asm volatile("" : "+v"(tx));
+    const int er = (tx >> 6) * 32 + (tx & 31);
+    // the next tile becomes the current one: its rows' gather-list entries are in LDS by now
+    t = t1;
+    if (t.row_count > 0) {
+      const int entry = *reinterpret_cast<const int*>(smem + kFwdEntries + 4 * tx);
+      decode_tile_rows(pn.t, tx >> 6, er, entry, t);
+      h = t.h; nkeys = t.nkeys; kv_tok0 = t.kv_tok0; limit = t.limit;
+      min_limit = __builtin_amdgcn_readfirstlane(t.wave_min_limit);
+      hkv = h / pn.t.rep;  // key/value head of this query head
+      row_valid = er < t.row_count;
+      k_head = (const char*)pn.k + (int64_t)kv_tok0 * row_bytes + hkv * pn.t.kv_head_b;
+      v_head = (const char*)pn.v + (int64_t)kv_tok0 * row_bytes + hkv * pn.t.kv_head_b;
+      nkt = (nkeys + TN - 1) / TN;
+      rot = t.rot % nkt;
+      // first loads of the tile: the first K and V tiles and the second K tile (global -> LDS), the Q rows.
+      // Q^T operand: lane (n, hh) holds q[tok][16*ks + 8*hh .. +7]
+      issue_k(key_tile(0), 0);
+      issue_v(key_tile(0), 0);
+      if (nkt > 1) issue_k(key_tile(1), 1);
+      const elem* src = reinterpret_cast<const elem*>((const char*)pn.q + t.tok * pn.t.q_tok_b + h * pn.t.q_head_b) + 8 * (tx >> 5 & 1);
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) bq[ks] = *reinterpret_cast<const elem8*>(src + 16 * ks);
+    }
+    // look-ahead: small-table lookups of the tile after, big-table lookup of the one after that, a new id
+    if (!decode_tile_head(pn.t, id2, code2, t1)) t1.nkeys = (code2 == kTilePastEnd) ? -1 : 0;
+    id2 = id3;
+    code2 = decode_tile_code(pn.t, id2);
+    if (tx == 0) drawn = __hip_atomic_fetch_add(pn.queues + queue, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  if (t.nkeys < 0) break;  // (uniform) no tiles left
+  // every copy of this wave has landed, and wave 0 has its draw
+  wait_vmem();
+  if (tid == 0) *reinterpret_cast<int*>(smem + kFwdIdSlot) = drawn;
+  if (t.row_count > 0) scrub_v(key_tile(0), 0);
   __syncthreads();
+  {
+    // the id drawn: queue `queue` counts the ids (8i + queue) * kXcdBlock + j; past the last tile the
+    // workgroup moves to the next queue, and after eight empty queues in a row there is nothing left
+    const TileTables tt = kernarg_now<TileTables>(offsetof(FwdParams<E>, t));
+    const int j = __builtin_amdgcn_readfirstlane(*reinterpret_cast<const int*>(smem + kFwdIdSlot));
+    const int64_t id = ((int64_t)(j / kXcdBlock) * 8 + queue) * kXcdBlock + (j % kXcdBlock);
+    if (id < (int64_t)tt.hist_bound + tt.self_total) {
+      id3 = (int)id;
+      empty_queues = 0;
+    } else {
+      queue = (queue + 1) & 7;
+      ++empty_queues;
+      id3 = empty_queues >= 8 ? 0x7fffffff : -1;   // past the end / no tile this time
+    }
+    // the entries of the next tile's rows start their way to LDS (its small-table lookups were issued
+    // at the switch, a few thousand cycles ago)
+    int tx = threadIdx.x;
+    asm volatile("" : "+v"(tx));
+    if (t1.row_count > 0 && t1.base >= 0) {
+      const int er = (tx >> 6) * 32 + (tx & 31);
+      async_copy4(tt.seg_dest + t1.base + min(er, t1.row_count - 1), lds_base + kFwdEntries + wave_u * 256);
+    }
+  }
+  have_partial = t.row_count > 0;
+  if (!have_partial) continue;
+  dest_done = t.dest;
+  valid_done = row_valid;
+  rows_done = t.row_count - wave_u * 32;  // rows of this wave that exist
 
   f32x16 s0, s1;   // S^T, then P^T, of the current and the next key block
   elem8 pb[2];    // P^T operand of the current block: elements 0..7 and 8..15
@@ -201,7 +315,7 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
     for (int e = 0; e < 16; ++e) s0[e] = 0.f;
 #pragma unroll
     for (int s8 = 0; s8 < 8; ++s8) s0 = mfma32(k_frag(0, 0, s8), bq[s8], s0);
-    if (key_tile(0) * TN + 31 > t.wave_min_limit) mask_block(s0, key_tile(0) * TN);
+    if (key_tile(0) * TN + 31 > min_limit) mask_block(s0, key_tile(0) * TN);
     float mx = s0[0];
 #pragma unroll
     for (int e = 1; e < 16; ++e) mx = fmaxf(mx, s0[e]);
@@ -311,8 +425,8 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
     const int key0 = key_tile(it) * TN;
     const int key0n = more ? key_tile(it + 1) * TN : 0;
     // the mask is needed once a key block reaches past the smallest row limit of the wave
-    const bool mask_a = key0 + 63 > t.wave_min_limit;
-    const bool mask_b = more && (key0n + 31 > t.wave_min_limit);
+    const bool mask_a = key0 + 63 > min_limit;
+    const bool mask_b = more && (key0n + 31 > min_limit);
     if constexpr (more) issue_v(key_tile(it + 1), st ^ 1);  // V(it-1) is dead since the barrier that ended tile it-1
 
     step(s0, s1, kcur, 1, key0 + 32, std::true_type{}, mask_a, vcur, 0);
@@ -343,38 +457,8 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
   } else {
     tile_body(it, St0{}, std::false_type{});
   }
+  }  // tiles
 #undef MOBA_PIN
-
-  // ---- epilogue: normalise, write the partial ----
-  // The accumulators hold O^T (a lane owns 4-element pieces of one row); the rows go through this
-  // wave's 8 KiB of LDS (free since the barrier that ended the last tile) so that they leave as
-  // whole 256-byte rows, four per store instruction, instead of 8-byte pieces of 32 rows.
-  const float l_tot = sum_xhalf(l_run);
-  const float inv = 1.f / l_tot;
-  {
-    char* stage = smem + wave * 8192;
-    char* wrow = stage + n * 256 + 8 * hh;
-#pragma unroll
-    for (int db = 0; db < 4; ++db)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        u32x2 w;
-        w[0] = pack2<E>(oacc[db][4 * g + 0] * inv, oacc[db][4 * g + 1] * inv);
-        w[1] = pack2<E>(oacc[db][4 * g + 2] * inv, oacc[db][4 * g + 3] * inv);
-        // elements 32*db + 8*g + 4*hh .. +3 of row n: 16-byte column 4*db + g, swizzled by the row
-        *reinterpret_cast<u32x2*>(wrow + (((4 * db + g) ^ (n & 15)) << 4)) = w;
-      }
-    if (row_valid && hh == 0) p.part_lse[t.dest] = m_run + fast_log2(l_tot);
-    const int c16 = lane & 15;
-    const int rows_here = t.row_count - wave * 32;  // rows of this wave that exist
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int row = 4 * i + (lane >> 4);
-      const int dest = __shfl(t.dest, row, 64);
-      const u32x4 x = *reinterpret_cast<const u32x4*>(stage + row * 256 + ((c16 ^ (row & 15)) << 4));
-      if (row < rows_here) *reinterpret_cast<u32x4*>(p.part_o + (int64_t)dest * kHeadDim + c16 * 8) = x;
-    }
-  }
 }
 
 // Combine the K1 slots of each (token, head): slot 0 is the self part, slot 1+j the
@@ -443,6 +527,8 @@ __global__ __launch_bounds__(256) void moba_merge_kernel(const typename E::elem*
   if (c8 == 0) lse[row] = (mx + fast_log2(wsum)) * 0.6931471805599453f;
 }
 
+__global__ void zero_queues_kernel(int* queues) { queues[threadIdx.x] = 0; }
+
 }  // namespace moba
 
 using namespace moba;
@@ -451,14 +537,16 @@ extern "C" int moba_fwd_tile_rows(void) { return TM; }
 
 template <class E>
 static int launch_partials(const void* q, const void* k, const void* v, void* part_o, float* part_lse,
-                           const TileTables& t, int D, int64_t grid, hipStream_t st) {
+                           const TileTables& t, int D, int64_t grid, int* queues, hipStream_t st) {
   FwdParams<E> p;
   p.q = (const typename E::elem*)q; p.k = (const typename E::elem*)k; p.v = (const typename E::elem*)v;
   p.part_o = (typename E::elem*)part_o; p.part_lse = part_lse;
   p.t = t;
   p.scale_log2 = (float)(1.4426950408889634 / sqrt((double)D));
+  p.queues = queues;
   static bool allowed[kMaxDevices];  // one array per element type
   if (!allow_dynamic_lds((const void*)moba_fwd_kernel<E>, kFwdLds, allowed)) return MOBA_ERR_LAUNCH;
+  hipLaunchKernelGGL(zero_queues_kernel, dim3(1), dim3(8), 0, st, queues);  // a kernel, not a memset: graph safe
   hipLaunchKernelGGL(moba_fwd_kernel<E>, dim3((unsigned)grid), dim3(256), kFwdLds, st, p);
   return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
 }
@@ -470,8 +558,9 @@ extern "C" int moba_fwd_partials(const void* q, const void* k, const void* v, vo
                                  const int32_t* self_tile_prefix, const int32_t* tile_seg,
                                  const int32_t* self_tile_chunk, int64_t S, int H, int Hkv, int D, int K, int F,
                                  int N, int B, int64_t hist_bound, int64_t self_tiles, const int64_t* strides,
-                                 int dtype, void* stream) {
-  if (!q || !k || !v || !part_o || !part_lse || !chunk_tok || !self_tile_prefix || !self_tile_chunk) return MOBA_ERR_ARG;
+                                 int32_t* queues, int dtype, void* stream) {
+  if (!q || !k || !v || !part_o || !part_lse || !chunk_tok || !self_tile_prefix || !self_tile_chunk || !queues)
+    return MOBA_ERR_ARG;
   if (Hkv <= 0 || H % Hkv != 0) return MOBA_ERR_ARG;
   if (K > 0 && (!seg_off || !tile_off || !seg_dest || !fchunk_tok || !tile_seg)) return MOBA_ERR_ARG;
   if (D != kHeadDim || (dtype != MOBA_DTYPE_BF16 && dtype != MOBA_DTYPE_F16)) return MOBA_ERR_UNSUPPORTED;
@@ -479,8 +568,12 @@ extern "C" int moba_fwd_partials(const void* q, const void* k, const void* v, vo
   if (((uintptr_t)q & 15) || ((uintptr_t)k & 15) || ((uintptr_t)v & 15) || ((uintptr_t)part_o & 15)) return MOBA_ERR_ARG;
   if ((int64_t)S * H * (K + 1) >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
   const int64_t total = (K > 0 ? hist_bound : 0) + self_tiles * H;
-  const int64_t grid = (total + 8 * kXcdBlock - 1) / (8 * kXcdBlock) * (8 * kXcdBlock);
-  if (grid >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
+  if (total >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
+  // two workgroups per CU (what the kernel's registers and LDS allow), all resident at once and drawing
+  // tiles from the queues; a multiple of 8 so that every XCD starts on its own queue with as many
+  const int cus = compute_units();
+  if (cus <= 0) return MOBA_ERR_LAUNCH;
+  const int64_t grid = (2 * (int64_t)cus + 7) / 8 * 8;
   TileTables t;
   t.seg_off = seg_off; t.tile_off = tile_off; t.seg_dest = seg_dest; t.fchunk_tok = fchunk_tok;
   t.chunk_tok = chunk_tok; t.self_tile_prefix = self_tile_prefix;
@@ -491,8 +584,8 @@ extern "C" int moba_fwd_partials(const void* q, const void* k, const void* v, vo
   t.self_total = (int)(self_tiles * H);
   if (!set_layout(t, strides)) return MOBA_ERR_ARG;
   hipStream_t st = (hipStream_t)stream;
-  return dtype == MOBA_DTYPE_F16 ? launch_partials<F16>(q, k, v, part_o, part_lse, t, D, grid, st)
-                                 : launch_partials<Bf16>(q, k, v, part_o, part_lse, t, D, grid, st);
+  return dtype == MOBA_DTYPE_F16 ? launch_partials<F16>(q, k, v, part_o, part_lse, t, D, grid, queues, st)
+                                 : launch_partials<Bf16>(q, k, v, part_o, part_lse, t, D, grid, queues, st);
 }
 
 extern "C" int moba_fwd_merge(const void* part_o, const float* part_lse, const int32_t* sel, void* out, float* lse,
@@ -517,10 +610,11 @@ extern "C" int moba_fwd(const void* q, const void* k, const void* v, void* part_
                         const int32_t* seg_dest, const int32_t* fchunk_tok, const int32_t* chunk_tok,
                         const int32_t* self_tile_prefix, const int32_t* tile_seg, const int32_t* self_tile_chunk,
                         void* out, float* lse, int64_t S, int H, int Hkv, int D, int K, int F, int N, int B,
-                        int64_t hist_bound, int64_t self_tiles, const int64_t* strides, int dtype, void* stream) {
+                        int64_t hist_bound, int64_t self_tiles, const int64_t* strides, int32_t* queues, int dtype,
+                        void* stream) {
   int rc = moba_fwd_partials(q, k, v, part_o, part_lse, seg_off, tile_off, seg_dest, fchunk_tok, chunk_tok,
                              self_tile_prefix, tile_seg, self_tile_chunk, S, H, Hkv, D, K, F, N, B, hist_bound,
-                             self_tiles, strides, dtype, stream);
+                             self_tiles, strides, queues, dtype, stream);
   if (rc != MOBA_OK) return rc;
   return moba_fwd_merge(part_o, part_lse, sel, out, lse, S, H, D, K, dtype, stream);
 }

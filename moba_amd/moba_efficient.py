@@ -217,13 +217,14 @@ def _forward(q, k, v, plan: MobaPlan, timer: Optional[StageTimer] = None):
     part_lse = torch.empty((S * H * (K + 1),), dtype=torch.float32, device=dev)
     out = torch.empty((S, H, D), dtype=q.dtype, device=dev)
     lse = torch.empty((S, H), dtype=torch.float32, device=dev)
+    queues = torch.empty(8, dtype=torch.int32, device=dev)  # the forward kernel's tile counters (it zeroes them)
     with span("fwd_partials"):
         _lib.check(lib.moba_fwd_partials(_ptr(q), _ptr(k), _ptr(v), _ptr(part_o), _ptr(part_lse), _ptr(seg_off),
                                          _ptr(tile_off), _ptr(seg_dest), _ptr(t.get("fchunk_tok")),
                                          _ptr(t["chunk_tok"]), _ptr(t["self_tile_prefix"]), _ptr(tile_seg),
                                          _ptr(t["self_tile_chunk"]), S, H, k.shape[1], D, K, plan.F, plan.N,
                                          plan.chunk_size, plan.hist_tile_bound(H), plan.self_tiles, _strides(q, k),
-                                         _dtype_code(q), _stream(dev)), "moba_fwd_partials")
+                                         _ptr(queues), _dtype_code(q), _stream(dev)), "moba_fwd_partials")
     with span("fwd_merge"):
         _lib.check(lib.moba_fwd_merge(_ptr(part_o), _ptr(part_lse), _ptr(sel), _ptr(out), _ptr(lse), S, H, D, K,
                                       _dtype_code(q), _stream(dev)), "moba_fwd_merge")
