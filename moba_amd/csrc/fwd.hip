@@ -46,7 +46,10 @@ constexpr float kRescaleThreshold = 8.f;  // log2 units: the running max may lag
 // so the vector work of one block executes under the MFMAs of its neighbours, and the
 // fragment reads from LDS run a few MFMAs ahead.  K and V tiles (64 keys) are double
 // buffered separately: K(t+1) must be resident half a tile before V(t+1).
-template <class E>
+// kQueued: resident workgroups that draw tiles from the queues (large problems).  Otherwise one tile per
+// workgroup, the id from the workgroup id: with few tiles the queue protocol's start-up and wind-down
+// (three passes to fill the look-ahead, eight empty draws to know that nothing is left) would dominate.
+template <class E, bool kQueued>
 __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) {
   MOBA_ELEM_TYPES(E)
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -235,6 +238,7 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
     for (int db = 0; db < 4; ++db)
 #pragma unroll
       for (int e = 0; e < 16; ++e) oacc[db][e] = 0.f;
+    if constexpr (!kQueued) return;
     m_run = -INFINITY;
     l_run = 0.f;
     __syncthreads();  // the K stages take the next tile's copies only after every wave has read its rows back
@@ -245,41 +249,51 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
     int tx = threadIdx.x;  // taken afresh, as above
     asm volatile("" : "+v"(tx));
     const int er = (tx >> 6) * 32 + (tx & 31);
-    // the next tile becomes the current one: its rows' gather-list entries are in LDS by now
-    t = t1;
+    if constexpr (kQueued) {
+      t = t1;  // the next tile becomes the current one: its rows' gather-list entries are in LDS by now
+    } else {
+      if (!decode_tile_head(pn.t, logical_tile_id(), t)) return;
+    }
     if (t.row_count > 0) {
-      const int entry = *reinterpret_cast<const int*>(smem + kFwdEntries + 4 * tx);
-      decode_tile_rows(pn.t, tx >> 6, er, entry, t);
-      h = t.h; nkeys = t.nkeys; kv_tok0 = t.kv_tok0; limit = t.limit;
-      min_limit = __builtin_amdgcn_readfirstlane(t.wave_min_limit);
+      // the wave-uniform half of the description is enough to start the first copies: the first K and V
+      // tiles and the second K tile (global -> LDS)
+      h = t.h; nkeys = t.nkeys; kv_tok0 = t.kv_tok0;
       hkv = h / pn.t.rep;  // key/value head of this query head
-      row_valid = er < t.row_count;
       k_head = (const char*)pn.k + (int64_t)kv_tok0 * row_bytes + hkv * pn.t.kv_head_b;
       v_head = (const char*)pn.v + (int64_t)kv_tok0 * row_bytes + hkv * pn.t.kv_head_b;
       nkt = (nkeys + TN - 1) / TN;
       rot = t.rot % nkt;
-      // first loads of the tile: the first K and V tiles and the second K tile (global -> LDS), the Q rows.
-      // Q^T operand: lane (n, hh) holds q[tok][16*ks + 8*hh .. +7]
       issue_k(key_tile(0), 0);
       issue_v(key_tile(0), 0);
       if (nkt > 1) issue_k(key_tile(1), 1);
+      // the per-row half, then the Q rows.  Q^T operand: lane (n, hh) holds q[tok][16*ks + 8*hh .. +7]
+      const int entry = kQueued ? *reinterpret_cast<const int*>(smem + kFwdEntries + 4 * tx)
+                                : decode_tile_row_entry(pn.t, er, t);
+      decode_tile_rows(pn.t, tx >> 6, er, entry, t);
+      limit = t.limit;
+      min_limit = __builtin_amdgcn_readfirstlane(t.wave_min_limit);
+      row_valid = er < t.row_count;
       const elem* src = reinterpret_cast<const elem*>((const char*)pn.q + t.tok * pn.t.q_tok_b + h * pn.t.q_head_b) + 8 * (tx >> 5 & 1);
 #pragma unroll
       for (int ks = 0; ks < 8; ++ks) bq[ks] = *reinterpret_cast<const elem8*>(src + 16 * ks);
     }
-    // look-ahead: small-table lookups of the tile after, big-table lookup of the one after that, a new id
-    if (!decode_tile_head(pn.t, id2, code2, t1)) t1.nkeys = (code2 == kTilePastEnd) ? -1 : 0;
-    id2 = id3;
-    code2 = decode_tile_code(pn.t, id2);
-    if (tx == 0) drawn = __hip_atomic_fetch_add(pn.queues + queue, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if constexpr (kQueued) {
+      // look-ahead: small-table lookups of the tile after, big-table lookup of the one after that, a new id
+      if (!decode_tile_head(pn.t, id2, code2, t1)) t1.nkeys = (code2 == kTilePastEnd) ? -1 : 0;
+      id2 = id3;
+      code2 = decode_tile_code(pn.t, id2);
+      if (tx == 0) drawn = __hip_atomic_fetch_add(pn.queues + queue, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
   }
   if (t.nkeys < 0) break;  // (uniform) no tiles left
   // every copy of this wave has landed, and wave 0 has its draw
   wait_vmem();
-  if (tid == 0) *reinterpret_cast<int*>(smem + kFwdIdSlot) = drawn;
+  if constexpr (kQueued) {
+    if (tid == 0) *reinterpret_cast<int*>(smem + kFwdIdSlot) = drawn;
+  }
   if (t.row_count > 0) scrub_v(key_tile(0), 0);
   __syncthreads();
-  {
+  if constexpr (kQueued) {
     // the id drawn: queue `queue` counts the ids (8i + queue) * kXcdBlock + j; past the last tile the
     // workgroup moves to the next queue, and after eight empty queues in a row there is nothing left
     const TileTables tt = kernarg_now<TileTables>(offsetof(FwdParams<E>, t));
@@ -544,10 +558,15 @@ static int launch_partials(const void* q, const void* k, const void* v, void* pa
   p.t = t;
   p.scale_log2 = (float)(1.4426950408889634 / sqrt((double)D));
   p.queues = queues;
-  static bool allowed[kMaxDevices];  // one array per element type
-  if (!allow_dynamic_lds((const void*)moba_fwd_kernel<E>, kFwdLds, allowed)) return MOBA_ERR_LAUNCH;
-  hipLaunchKernelGGL(zero_queues_kernel, dim3(1), dim3(8), 0, st, queues);  // a kernel, not a memset: graph safe
-  hipLaunchKernelGGL(moba_fwd_kernel<E>, dim3((unsigned)grid), dim3(256), kFwdLds, st, p);
+  static bool allowed[2][kMaxDevices];  // one pair of arrays per element type
+  if (grid > 0) {  // resident workgroups drawing from the queues
+    if (!allow_dynamic_lds((const void*)moba_fwd_kernel<E, true>, kFwdLds, allowed[1])) return MOBA_ERR_LAUNCH;
+    hipLaunchKernelGGL(zero_queues_kernel, dim3(1), dim3(8), 0, st, queues);  // a kernel, not a memset: graph safe
+    hipLaunchKernelGGL((moba_fwd_kernel<E, true>), dim3((unsigned)grid), dim3(256), kFwdLds, st, p);
+  } else {         // one workgroup per tile id
+    if (!allow_dynamic_lds((const void*)moba_fwd_kernel<E, false>, kFwdLds, allowed[0])) return MOBA_ERR_LAUNCH;
+    hipLaunchKernelGGL((moba_fwd_kernel<E, false>), dim3((unsigned)-grid), dim3(256), kFwdLds, st, p);
+  }
   return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
 }
 
@@ -573,7 +592,10 @@ extern "C" int moba_fwd_partials(const void* q, const void* k, const void* v, vo
   // tiles from the queues; a multiple of 8 so that every XCD starts on its own queue with as many
   const int cus = compute_units();
   if (cus <= 0) return MOBA_ERR_LAUNCH;
-  const int64_t grid = (2 * (int64_t)cus + 7) / 8 * 8;
+  int64_t grid = (2 * (int64_t)cus + 7) / 8 * 8;
+  // with fewer than a few tiles per resident workgroup the queues do not pay: one workgroup per id then
+  // (a negative grid tells the launcher)
+  if (total < 8 * grid) grid = -((total + 8 * kXcdBlock - 1) / (8 * kXcdBlock) * (8 * kXcdBlock));
   TileTables t;
   t.seg_off = seg_off; t.tile_off = tile_off; t.seg_dest = seg_dest; t.fchunk_tok = fchunk_tok;
   t.chunk_tok = chunk_tok; t.self_tile_prefix = self_tile_prefix;
