@@ -62,6 +62,10 @@ struct Tile {
   int base;       // history tile: index of row 0 in seg_dest; self tile: -(row 0 inside the chunk) - 1
 };
 
+// the tile counters of a kernel whose resident workgroups draw their tiles from per-XCD queues start at zero
+// (a kernel, not a memset: safe to record into a graph)
+static __global__ void zero_queues_kernel(int* queues) { queues[threadIdx.x] = 0; }
+
 // Workgroup ids are dealt round-robin to the 8 XCDs; give each XCD runs of kXcdBlock
 // consecutive logical tiles so that tiles sharing a K/V chunk share an L2.
 __device__ __forceinline__ int logical_tile_id() {

@@ -30,7 +30,8 @@ constexpr int TQ = 64;                                  // query rows per step o
 constexpr int kBwdDqLds = 4 * kTileBytes;               // K[2], V[2]
 constexpr int kQStage = 2 * TQ * kHeadDim * 2 + 2 * TQ * 4;  // Q tile, dO tile, lse, delta
 constexpr int kDkvStages = 3;
-constexpr int kBwdDkvLds = kDkvStages * kQStage;
+constexpr int kDkvIdSlot = kDkvStages * kQStage;  // where wave 0 hands the tile id it drew to the other waves
+constexpr int kBwdDkvLds = kDkvIdSlot + 16;
 
 template <class E>
 struct BwdParams {
@@ -50,6 +51,7 @@ struct BwdParams {
   float scale;
   uint32_t hk_magic;  // n / (H*K1) == (n * hk_magic) >> hk_shift for every n < 2^31
   uint32_t hk_shift;
+  int* queues;        // [8] tile counters of the dK/dV kernel, one per XCD, zero when it starts
 };
 
 template <class E>
@@ -335,9 +337,28 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
   const int n = lane & 31, hh = lane >> 5;
   const int H = p.t.H, K1 = p.t.K1, Hkv = p.t.Hkv, rep = p.t.rep;
 
+  // The workgroups (one per CU, all resident) draw their tiles from eight queues, one per XCD: queue x
+  // hands out the ids (8i + x) * kXcdBlock + j in order -- consecutive ids, i.e. key tiles of one
+  // (chunk, head) that gather the same Q and dO rows, run side by side behind one L2 -- and a workgroup whose
+  // queue is empty goes on with the next XCD's, so that the XCDs, which differ in speed by a few percent,
+  // finish together.  A tile runs for about a millisecond: the draw (one atomic, two barriers) is free.
+  int queue = blockIdx.x & 7, empty_queues = 0;
+  while (true) {
+  __syncthreads();  // every wave is done with the LDS of the previous tile and has read the previous draw
+  if (tid == 0)
+    *reinterpret_cast<int*>(smem + kDkvIdSlot) =
+        __hip_atomic_fetch_add(p.queues + queue, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __syncthreads();
+  const int drawn = __builtin_amdgcn_readfirstlane(*reinterpret_cast<const int*>(smem + kDkvIdSlot));
+  const int64_t id = ((int64_t)(drawn / kXcdBlock) * 8 + queue) * kXcdBlock + (drawn % kXcdBlock);
+  if (id >= p.t.self_total / rep) {
+    queue = (queue + 1) & 7;
+    if (++empty_queues == 8) break;
+    continue;
+  }
+  empty_queues = 0;
   // ---- which 128-key tile of which key/value head: the forward's self-tile enumeration over Hkv heads ----
-  const int st = logical_tile_id();
-  if (st >= p.t.self_total / rep) return;
+  const int st = (int)id;
   const int c = p.t.self_tile_chunk[st / Hkv];
   const int rem = st - p.t.self_tile_prefix[c] * Hkv;
   const int nt = p.t.self_tile_prefix[c + 1] - p.t.self_tile_prefix[c];
@@ -617,7 +638,6 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
     buf = buf1;
   }
   }  // query heads
-#undef MOBA_PIN
 
   if (key_valid) {
     const int64_t off = ((int64_t)(c0 + mykey) * Hkv + hkv) * kHeadDim;
@@ -634,6 +654,8 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
         *reinterpret_cast<u32x2*>(p.dv + off + 32 * db + 8 * g + 4 * hh) = wv;
       }
   }
+  }  // tiles
+#undef MOBA_PIN
 }
 
 }  // namespace moba
@@ -644,12 +666,13 @@ template <class E>
 static int launch_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out, const float* lse,
                       const int32_t* sel, const int32_t* chunk_fid, float* delta, float* part_dq, void* dq, void* dk,
                       void* dv, const TileTables& t, int64_t S, int H, int D, int K, int64_t grid_q, int64_t grid_kv,
-                      hipStream_t st) {
+                      int* queues, hipStream_t st) {
   typedef typename E::elem elem;
   BwdParams<E> p;
   p.q = (const elem*)q; p.k = (const elem*)k; p.v = (const elem*)v; p.dout = (const elem*)dout;
   p.lse = lse; p.delta = delta; p.lse2 = delta + S * H; p.part_dq = part_dq; p.dk = (elem*)dk; p.dv = (elem*)dv;
   p.chunk_fid = chunk_fid;
+  p.queues = queues;
   p.t = t;
   p.scale = (float)(1.0 / sqrt((double)D));
   p.scale_log2 = (float)(1.4426950408889634 / sqrt((double)D));
@@ -671,6 +694,7 @@ static int launch_bwd(const void* dout, const void* q, const void* k, const void
   hipLaunchKernelGGL(bwd_dq_kernel<E>, dim3((unsigned)grid_q), dim3(256), kBwdDqLds, st, p);
   hipLaunchKernelGGL(bwd_dq_reduce_kernel<E>, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st,
                      (const float*)part_dq, sel, (elem*)dq, rows, K + 1, p.scale);
+  hipLaunchKernelGGL(zero_queues_kernel, dim3(1), dim3(8), 0, st, queues);  // a kernel, not a memset: graph safe
   hipLaunchKernelGGL(bwd_dkv_kernel<E>, dim3((unsigned)grid_kv), dim3(256), kBwdDkvLds, st, p);
   return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
 }
@@ -681,9 +705,10 @@ extern "C" int moba_bwd(const void* dout, const void* q, const void* k, const vo
                         const int32_t* self_tile_prefix, const int32_t* tile_seg, const int32_t* self_tile_chunk,
                         const int32_t* chunk_fid, float* delta, float* part_dq,
                         void* dq, void* dk, void* dv, int64_t S, int H, int Hkv, int D, int K, int F, int N, int B,
-                        int64_t hist_bound, int64_t self_tiles, const int64_t* strides, int dtype, void* stream) {
+                        int64_t hist_bound, int64_t self_tiles, const int64_t* strides, int32_t* queues, int dtype,
+                        void* stream) {
   if (!dout || !q || !k || !v || !out || !lse || !chunk_tok || !self_tile_prefix || !self_tile_chunk || !delta ||
-      !part_dq || !dq || !dk || !dv)
+      !part_dq || !dq || !dk || !dv || !queues)
     return MOBA_ERR_ARG;
   if (K > 0 && (!sel || !seg_off || !tile_off || !seg_dest || !fchunk_tok || !chunk_fid || !tile_seg))
     return MOBA_ERR_ARG;
@@ -697,7 +722,10 @@ extern "C" int moba_bwd(const void* dout, const void* q, const void* k, const vo
   const int64_t per = 8 * kXcdBlock;
   const int64_t total_q = (K > 0 ? hist_bound : 0) + self_tiles * H;
   const int64_t grid_q = (total_q + per - 1) / per * per;
-  const int64_t grid_kv = (self_tiles * Hkv + per - 1) / per * per;
+  // the dK/dV kernel: one workgroup per CU, resident, drawing its tiles from the queues
+  const int cus = compute_units();
+  if (cus <= 0) return MOBA_ERR_LAUNCH;
+  const int64_t grid_kv = ((int64_t)cus + 7) / 8 * 8;
   if (grid_q >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
   TileTables t;
   t.seg_off = seg_off; t.tile_off = tile_off; t.seg_dest = seg_dest; t.fchunk_tok = fchunk_tok;
@@ -711,7 +739,7 @@ extern "C" int moba_bwd(const void* dout, const void* q, const void* k, const vo
   hipStream_t st = (hipStream_t)stream;
   return dtype == MOBA_DTYPE_F16
              ? launch_bwd<F16>(dout, q, k, v, out, lse, sel, chunk_fid, delta, part_dq, dq, dk, dv, t, S, H, D, K,
-                               grid_q, grid_kv, st)
+                               grid_q, grid_kv, queues, st)
              : launch_bwd<Bf16>(dout, q, k, v, out, lse, sel, chunk_fid, delta, part_dq, dq, dk, dv, t, S, H, D, K,
-                                grid_q, grid_kv, st);
+                                grid_q, grid_kv, queues, st);
 }

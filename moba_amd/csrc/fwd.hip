@@ -541,8 +541,6 @@ __global__ __launch_bounds__(256) void moba_merge_kernel(const typename E::elem*
   if (c8 == 0) lse[row] = (mx + fast_log2(wsum)) * 0.6931471805599453f;
 }
 
-__global__ void zero_queues_kernel(int* queues) { queues[threadIdx.x] = 0; }
-
 }  // namespace moba
 
 using namespace moba;

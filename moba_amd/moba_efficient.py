@@ -242,12 +242,13 @@ def _backward(dout, q, k, v, out, lse, sel, seg_off, tile_off, seg_dest, tile_se
     dv = torch.empty(v.shape, dtype=v.dtype, device=dev)
     delta = torch.empty((2, S, H), dtype=torch.float32, device=dev)
     part_dq = torch.empty((S * H * (K + 1), D), dtype=torch.float32, device=dev)
+    queues = torch.empty(8, dtype=torch.int32, device=dev)  # the dK/dV kernel's tile counters (it zeroes them)
     _lib.check(lib.moba_bwd(_ptr(dout), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(sel), _ptr(seg_off),
                             _ptr(tile_off), _ptr(seg_dest), _ptr(t.get("fchunk_tok")), _ptr(t["chunk_tok"]),
                             _ptr(t["self_tile_prefix"]), _ptr(tile_seg), _ptr(t["self_tile_chunk"]),
                             _ptr(t.get("chunk_fid")), _ptr(delta), _ptr(part_dq), _ptr(dq), _ptr(dk), _ptr(dv),
                             S, H, k.shape[1], D, K, plan.F, plan.N, plan.chunk_size, plan.hist_tile_bound(H),
-                            plan.self_tiles, _strides(q, k), _dtype_code(q), _stream(dev)), "moba_bwd")
+                            plan.self_tiles, _strides(q, k), _ptr(queues), _dtype_code(q), _stream(dev)), "moba_bwd")
     return dq, dk, dv
 
 
