@@ -119,7 +119,7 @@ int moba_fwd(const void* q, const void* k, const void* v, void* part_o, float* p
  *   chunk_fid [N] int32: filtered id of each chunk, -1 for the last chunk of a sequence
  *   delta [2,S,H] fp32 scratch (rowsum(dO*O), then the LSE in the log2 domain); part_dq [S*H*(K+1), D] fp32 scratch
  *   dq, dk, dv: out; dk and dv of a key/value head sum over its query heads
- *   queues [8] int32 scratch: tile counters of the dK/dV kernel (as in moba_fwd_partials) */
+ *   queues [16] int32 scratch: tile counters of the dQ and dK/dV kernels (as in moba_fwd_partials) */
 int moba_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out, const float* lse,
              const int32_t* sel, const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest,
              const int32_t* fchunk_tok, const int32_t* chunk_tok, const int32_t* self_tile_prefix,

@@ -27,7 +27,8 @@ namespace moba {
 
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr int TQ = 64;                                  // query rows per step of the dK/dV kernel
-constexpr int kBwdDqLds = 4 * kTileBytes;               // K[2], V[2]
+constexpr int kDqIdSlot = 4 * kTileBytes;                // after K[2], V[2]: the tile id wave 0 drew
+constexpr int kBwdDqLds = kDqIdSlot + 16;
 constexpr int kQStage = 2 * TQ * kHeadDim * 2 + 2 * TQ * 4;  // Q tile, dO tile, lse, delta
 constexpr int kDkvStages = 3;
 constexpr int kDkvIdSlot = kDkvStages * kQStage;  // where wave 0 hands the tile id it drew to the other waves
@@ -51,7 +52,7 @@ struct BwdParams {
   float scale;
   uint32_t hk_magic;  // n / (H*K1) == (n * hk_magic) >> hk_shift for every n < 2^31
   uint32_t hk_shift;
-  int* queues;        // [8] tile counters of the dK/dV kernel, one per XCD, zero when it starts
+  int* queues;        // [16] tile counters, one per XCD, of the dQ kernel and of the dK/dV kernel; zero at the start
 };
 
 template <class E>
@@ -86,9 +87,33 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams<E> p) {
   const int n = lane & 31, hh = lane >> 5;
   const int H = p.t.H;
 
+  // The workgroups (two per CU, all resident) draw their tiles from eight queues, one per XCD: queue x
+  // hands out the ids (8i + x) * kXcdBlock + j in order, so that the tiles in flight on an XCD are
+  // consecutive ids (tiles that share a K/V chunk behind one L2), and a workgroup whose queue is empty
+  // goes on with the next XCD's: the XCDs differ in speed by a few percent and finish together this way.
+  // The draw for the next tile is in flight while the current one is computed.
+  int queue = blockIdx.x & 7, empty_queues = 0;
+  int drawn_next = 0;  // thread 0: the counter value drawn for the next tile
+  if (tid == 0) drawn_next = __hip_atomic_fetch_add(p.queues + queue, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  while (true) {
+  __syncthreads();  // the previous tile is done with LDS, and every wave has read the previous draw
+  if (tid == 0) *reinterpret_cast<int*>(smem + kDqIdSlot) = drawn_next;
+  __syncthreads();
+  const int drawn = __builtin_amdgcn_readfirstlane(*reinterpret_cast<const int*>(smem + kDqIdSlot));
+  const int64_t id = ((int64_t)(drawn / kXcdBlock) * 8 + queue) * kXcdBlock + (drawn % kXcdBlock);
+  const bool past_end = id >= (int64_t)p.t.hist_bound + p.t.self_total;
+  if (past_end) {
+    queue = (queue + 1) & 7;
+    if (++empty_queues == 8) break;
+  } else {
+    empty_queues = 0;
+  }
+  if (tid == 0) drawn_next = __hip_atomic_fetch_add(p.queues + queue, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (past_end) continue;
+
   Tile t;
   const int r = wave * 32 + n;
-  if (!decode_tile(p.t, logical_tile_id(), wave, r, t)) return;
+  if (!decode_tile(p.t, (int)id, wave, r, t)) continue;  // an unused id below hist_bound
   const int h = t.h, nkeys = t.nkeys, kv_tok0 = t.kv_tok0, limit = t.limit;
   const bool row_valid = r < t.row_count;
 
@@ -273,6 +298,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams<E> p) {
         *reinterpret_cast<f32x4*>(dst + 32 * db + 8 * g + 4 * hh) = w;
       }
   }
+  }  // tiles
 }
 
 // dq[row] = scale * sum over the row's valid slots of part_dq; 16 lanes per row
@@ -347,7 +373,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
   __syncthreads();  // every wave is done with the LDS of the previous tile and has read the previous draw
   if (tid == 0)
     *reinterpret_cast<int*>(smem + kDkvIdSlot) =
-        __hip_atomic_fetch_add(p.queues + queue, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_fetch_add(p.queues + 8 + queue, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   __syncthreads();
   const int drawn = __builtin_amdgcn_readfirstlane(*reinterpret_cast<const int*>(smem + kDkvIdSlot));
   const int64_t id = ((int64_t)(drawn / kXcdBlock) * 8 + queue) * kXcdBlock + (drawn % kXcdBlock);
@@ -691,10 +717,10 @@ static int launch_bwd(const void* dout, const void* q, const void* k, const void
   const int64_t rows = S * H;
   hipLaunchKernelGGL(bwd_delta_kernel<E>, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st, (const elem*)dout,
                      (const elem*)out, lse, delta, delta + S * H, rows);
+  hipLaunchKernelGGL(zero_queues_kernel, dim3(1), dim3(16), 0, st, queues);  // a kernel, not a memset: graph safe
   hipLaunchKernelGGL(bwd_dq_kernel<E>, dim3((unsigned)grid_q), dim3(256), kBwdDqLds, st, p);
   hipLaunchKernelGGL(bwd_dq_reduce_kernel<E>, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st,
                      (const float*)part_dq, sel, (elem*)dq, rows, K + 1, p.scale);
-  hipLaunchKernelGGL(zero_queues_kernel, dim3(1), dim3(8), 0, st, queues);  // a kernel, not a memset: graph safe
   hipLaunchKernelGGL(bwd_dkv_kernel<E>, dim3((unsigned)grid_kv), dim3(256), kBwdDkvLds, st, p);
   return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
 }
@@ -719,14 +745,13 @@ extern "C" int moba_bwd(const void* dout, const void* q, const void* k, const vo
   for (const void* x : ptrs)
     if ((uintptr_t)x & 15) return MOBA_ERR_ARG;
   if ((int64_t)S * H * (K + 1) >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
-  const int64_t per = 8 * kXcdBlock;
   const int64_t total_q = (K > 0 ? hist_bound : 0) + self_tiles * H;
-  const int64_t grid_q = (total_q + per - 1) / per * per;
   // the dK/dV kernel: one workgroup per CU, resident, drawing its tiles from the queues
   const int cus = compute_units();
   if (cus <= 0) return MOBA_ERR_LAUNCH;
   const int64_t grid_kv = ((int64_t)cus + 7) / 8 * 8;
-  if (grid_q >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
+  const int64_t grid_q = 2 * grid_kv;  // the dQ kernel fits two workgroups on a CU
+  if (total_q >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
   TileTables t;
   t.seg_off = seg_off; t.tile_off = tile_off; t.seg_dest = seg_dest; t.fchunk_tok = fchunk_tok;
   t.chunk_tok = chunk_tok; t.self_tile_prefix = self_tile_prefix;
