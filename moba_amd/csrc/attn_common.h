@@ -9,7 +9,11 @@ namespace moba {
 constexpr int TM = 128;  // query rows per workgroup (32 per wave)
 constexpr int TN = 64;   // keys per inner iteration
 constexpr int kTileBytes = TN * kHeadDim * 2;
-constexpr int kXcdBlock = 64;  // consecutive logical tiles that share an XCD
+constexpr int kXcdBlock = 64;  // consecutive logical tiles that share an XCD (one workgroup per tile id)
+// The same for kernels whose resident workgroups draw ids from per-XCD queues.  Longer runs there: an id is
+// computed a few tiles after it was drawn, by workgroups whose speeds differ, so the ids in flight on an XCD
+// span about two of its 64 slots' worth; with runs of 256 they still mostly belong to one K/V chunk.
+constexpr int kQueueRun = 256;
 
 // Index tables that define the tiles of one call.
 struct TileTables {

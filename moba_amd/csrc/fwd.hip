@@ -58,7 +58,7 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
   const int H = p.t.H;
 
   // The workgroups (two per CU, all resident) draw tiles from eight queues, one per XCD: queue x hands
-  // out the ids (8i + x) * kXcdBlock + j in order, so that the tiles in flight on an XCD are consecutive ids
+  // out the ids (8i + x) * kQueueRun + j in order, so that the tiles in flight on an XCD are consecutive ids
   // -- tiles that share a K/V chunk behind one L2 -- and an XCD that runs ahead (they differ by a few
   // percent) goes on with the next queue when its own is empty.  A tile's description takes dependent
   // lookups: the id (an atomic), the big table, the small tables, the gather-list entry of every row.
@@ -294,11 +294,11 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
   if (t.row_count > 0) scrub_v(key_tile(0), 0);
   __syncthreads();
   if constexpr (kQueued) {
-    // the id drawn: queue `queue` counts the ids (8i + queue) * kXcdBlock + j; past the last tile the
+    // the id drawn: queue `queue` counts the ids (8i + queue) * kQueueRun + j; past the last tile the
     // workgroup moves to the next queue, and after eight empty queues in a row there is nothing left
     const TileTables tt = kernarg_now<TileTables>(offsetof(FwdParams<E>, t));
     const int j = __builtin_amdgcn_readfirstlane(*reinterpret_cast<const int*>(smem + kFwdIdSlot));
-    const int64_t id = ((int64_t)(j / kXcdBlock) * 8 + queue) * kXcdBlock + (j % kXcdBlock);
+    const int64_t id = ((int64_t)(j / kQueueRun) * 8 + queue) * kQueueRun + (j % kQueueRun);
     if (id < (int64_t)tt.hist_bound + tt.self_total) {
       id3 = (int)id;
       empty_queues = 0;
