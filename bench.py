@@ -70,7 +70,7 @@ def make_inputs(name, device, gqa=False):
     return q, k, v, cu, max(lens), B, topk
 
 
-def cpu_baseline(q, k, v, B, topk, budget_tokens=32768, heads=4):
+def cpu_baseline(q, k, v, B, topk, budget_tokens=32768, heads=8):
     """Dense-mask oracle (restatement of moba_naive) on the first ``budget_tokens`` tokens of
     ``heads`` heads of the same data, one head at a time, on this host's cores."""
     from oracle import moba_oracle as O
@@ -226,8 +226,9 @@ def main():
         result["decode"] = bench_decode(dev, S if len(cu) == 2 else max_seqlen, H)
     if not args.no_cpu_baseline:
         rep = H // k.shape[1]
-        result["cpu_baseline"] = cpu_baseline(q, k[:, ::1] if rep == 1 else torch.repeat_interleave(k[:, :1], 4, dim=1),
-                                              v[:, ::1] if rep == 1 else torch.repeat_interleave(v[:, :1], 4, dim=1), B, topk)
+        nkv = (8 + rep - 1) // rep  # key/value heads behind the first 8 query heads
+        result["cpu_baseline"] = cpu_baseline(q, k if rep == 1 else torch.repeat_interleave(k[:, :nkv], rep, dim=1),
+                                              v if rep == 1 else torch.repeat_interleave(v[:, :nkv], rep, dim=1), B, topk)
     print(json.dumps(result))
 
 
