@@ -117,14 +117,14 @@ int moba_fwd(const void* q, const void* k, const void* v, void* part_o, float* p
  *   dout, q, out, dq [S,H,D] elem; k, v, dk, dv [S,Hkv,D] elem; lse [S,H] fp32 from the forward
  *   (`strides` applies to q, k, v; dout, out, dq, dk, dv are packed)
  *   chunk_fid [N] int32: filtered id of each chunk, -1 for the last chunk of a sequence
- *   delta [2,S,H] fp32 scratch (rowsum(dO*O), then the LSE in the log2 domain); part_dq [S*H*(K+1), D] fp32 scratch
+ *   delta [2,S,H] fp32 scratch (rowsum(dO*O), then the LSE in the log2 domain); part_dq [S*H*(K+1), D] elem scratch (the per-slot dQ, rounded as the per-chunk dQ that flash-attn returns to the reference is)
  *   dq, dk, dv: out; dk and dv of a key/value head sum over its query heads
  *   queues [16] int32 scratch: tile counters of the dQ and dK/dV kernels (as in moba_fwd_partials) */
 int moba_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out, const float* lse,
              const int32_t* sel, const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest,
              const int32_t* fchunk_tok, const int32_t* chunk_tok, const int32_t* self_tile_prefix,
              const int32_t* tile_seg, const int32_t* self_tile_chunk, const int32_t* chunk_fid, float* delta,
-             float* part_dq, void* dq, void* dk, void* dv, int64_t S, int H, int Hkv, int D, int K, int F, int N, int B,
+             void* part_dq, void* dq, void* dk, void* dv, int64_t S, int H, int Hkv, int D, int K, int F, int N, int B,
              int64_t hist_bound, int64_t self_tiles, const int64_t* strides, int32_t* queues, int dtype,
              void* stream);
 

@@ -43,7 +43,7 @@ struct BwdParams {
   const float* lse;    // [S*H] natural log
   const float* delta;  // [S*H]
   const float* lse2;   // [S*H] lse in the log2 domain
-  float* part_dq;      // [S*H*K1, D] fp32
+  typename E::elem* part_dq;  // [S*H*K1, D]: per-slot dQ before the softmax scale, in the element type
   typename E::elem* dk;
   typename E::elem* dv;
   const int* chunk_fid;  // [N] filtered id of a chunk, -1 for the last chunk of a sequence
@@ -286,24 +286,39 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams<E> p) {
     __syncthreads();
   }
 
-  if (row_valid) {
-    float* dst = p.part_dq + (int64_t)t.dest * kHeadDim;
+  // The accumulators hold dQ^T (a lane owns 4-element pieces of one row).  The partial is rounded to the
+  // element type, as the per-chunk dQ that flash-attn returns to the reference is, and goes through this
+  // wave's 8 KiB of LDS (free since the barrier that ended the last key tile) so that it leaves as whole
+  // 256-byte rows, four per store instruction.
+  {
+    char* stage = smem + wave_u * 8192;
+    char* wrow = stage + n * 256 + 8 * hh;
 #pragma unroll
     for (int db = 0; db < 4; ++db)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        f32x4 w;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) w[e] = dqacc[db][4 * g + e];
-        *reinterpret_cast<f32x4*>(dst + 32 * db + 8 * g + 4 * hh) = w;
+        u32x2 w;
+        w[0] = pack2<E>(dqacc[db][4 * g + 0], dqacc[db][4 * g + 1]);
+        w[1] = pack2<E>(dqacc[db][4 * g + 2], dqacc[db][4 * g + 3]);
+        // elements 32*db + 8*g + 4*hh .. +3 of row n: 16-byte column 4*db + g, swizzled by the row
+        *reinterpret_cast<u32x2*>(wrow + (((4 * db + g) ^ (n & 15)) << 4)) = w;
       }
+    const int c16 = lane & 15;
+    const int rows_here = t.row_count - wave_u * 32;  // rows of this wave that exist
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int row = 4 * i + (lane >> 4);
+      const int dest = __shfl(t.dest, row, 64);
+      const u32x4 x = *reinterpret_cast<const u32x4*>(stage + row * 256 + ((c16 ^ (row & 15)) << 4));
+      if (row < rows_here) *reinterpret_cast<u32x4*>(p.part_dq + (int64_t)dest * kHeadDim + c16 * 8) = x;
+    }
   }
   }  // tiles
 }
 
 // dq[row] = scale * sum over the row's valid slots of part_dq; 16 lanes per row
 template <class E>
-__global__ __launch_bounds__(256) void bwd_dq_reduce_kernel(const float* __restrict__ part_dq,
+__global__ __launch_bounds__(256) void bwd_dq_reduce_kernel(const typename E::elem* __restrict__ part_dq,
                                                             const int* __restrict__ sel,
                                                             typename E::elem* __restrict__ dq, int64_t rows, int K1,
                                                             float scale) {
@@ -317,33 +332,28 @@ __global__ __launch_bounds__(256) void bwd_dq_reduce_kernel(const float* __restr
   float acc[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.f;
-  const float* src = part_dq + row * K1 * kHeadDim + c8 * 8;
+  const elem* src = part_dq + row * K1 * kHeadDim + c8 * 8;
   // lane c8 fetches the presence of slot j0 + c8; absent slots are redirected to slot 0 and
-  // multiplied by 0, so the loads of four slots are unconditional and in flight together
+  // multiplied by 0, so the loads of eight slots are unconditional and in flight together
   for (int j0 = 0; j0 < K1; j0 += 16) {
     const int j = j0 + c8;
     const float present = (j < K1 && (j == 0 || ps[j - 1] >= 0)) ? 1.f : 0.f;
     const int nslot = min(16, K1 - j0);
-    for (int u0 = 0; u0 < nslot; u0 += 4) {
-      f32x4 a[4], b[4];
-      float w[4];
+    for (int u0 = 0; u0 < nslot; u0 += 8) {
+      elem8 a[8];
+      float w[8];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
+      for (int u = 0; u < 8; ++u) {
         w[u] = __shfl(present, u0 + u, 16);
         const int jj = w[u] > 0.f ? j0 + u0 + u : 0;
-        if (u0 + u < nslot) {  // uniform: no loads for slots that do not exist
-          a[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(src + (int64_t)jj * kHeadDim));
-          b[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(src + (int64_t)jj * kHeadDim + 4));
-        }
+        if (u0 + u < nslot)  // uniform: no loads for slots that do not exist
+          a[u] = __builtin_nontemporal_load(reinterpret_cast<const elem8*>(src + (int64_t)jj * kHeadDim));
       }
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
+      for (int u = 0; u < 8; ++u) {
         if (u0 + u >= nslot) break;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          acc[e] += w[u] * a[u][e];
-          acc[4 + e] += w[u] * b[u][e];
-        }
+        for (int e = 0; e < 8; ++e) acc[e] += w[u] * (float)a[u][e];
       }
     }
   }
@@ -690,13 +700,13 @@ using namespace moba;
 
 template <class E>
 static int launch_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out, const float* lse,
-                      const int32_t* sel, const int32_t* chunk_fid, float* delta, float* part_dq, void* dq, void* dk,
+                      const int32_t* sel, const int32_t* chunk_fid, float* delta, void* part_dq, void* dq, void* dk,
                       void* dv, const TileTables& t, int64_t S, int H, int D, int K, int64_t grid_q, int64_t grid_kv,
                       int* queues, hipStream_t st) {
   typedef typename E::elem elem;
   BwdParams<E> p;
   p.q = (const elem*)q; p.k = (const elem*)k; p.v = (const elem*)v; p.dout = (const elem*)dout;
-  p.lse = lse; p.delta = delta; p.lse2 = delta + S * H; p.part_dq = part_dq; p.dk = (elem*)dk; p.dv = (elem*)dv;
+  p.lse = lse; p.delta = delta; p.lse2 = delta + S * H; p.part_dq = (elem*)part_dq; p.dk = (elem*)dk; p.dv = (elem*)dv;
   p.chunk_fid = chunk_fid;
   p.queues = queues;
   p.t = t;
@@ -720,7 +730,7 @@ static int launch_bwd(const void* dout, const void* q, const void* k, const void
   hipLaunchKernelGGL(zero_queues_kernel, dim3(1), dim3(16), 0, st, queues);  // a kernel, not a memset: graph safe
   hipLaunchKernelGGL(bwd_dq_kernel<E>, dim3((unsigned)grid_q), dim3(256), kBwdDqLds, st, p);
   hipLaunchKernelGGL(bwd_dq_reduce_kernel<E>, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st,
-                     (const float*)part_dq, sel, (elem*)dq, rows, K + 1, p.scale);
+                     (const elem*)part_dq, sel, (elem*)dq, rows, K + 1, p.scale);
   hipLaunchKernelGGL(bwd_dkv_kernel<E>, dim3((unsigned)grid_kv), dim3(256), kBwdDkvLds, st, p);
   return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
 }
@@ -729,7 +739,7 @@ extern "C" int moba_bwd(const void* dout, const void* q, const void* k, const vo
                         const float* lse, const int32_t* sel, const int32_t* seg_off, const int32_t* tile_off,
                         const int32_t* seg_dest, const int32_t* fchunk_tok, const int32_t* chunk_tok,
                         const int32_t* self_tile_prefix, const int32_t* tile_seg, const int32_t* self_tile_chunk,
-                        const int32_t* chunk_fid, float* delta, float* part_dq,
+                        const int32_t* chunk_fid, float* delta, void* part_dq,
                         void* dq, void* dk, void* dv, int64_t S, int H, int Hkv, int D, int K, int F, int N, int B,
                         int64_t hist_bound, int64_t self_tiles, const int64_t* strides, int32_t* queues, int dtype,
                         void* stream) {

@@ -241,7 +241,7 @@ def _backward(dout, q, k, v, out, lse, sel, seg_off, tile_off, seg_dest, tile_se
     dk = torch.empty(k.shape, dtype=k.dtype, device=dev)
     dv = torch.empty(v.shape, dtype=v.dtype, device=dev)
     delta = torch.empty((2, S, H), dtype=torch.float32, device=dev)
-    part_dq = torch.empty((S * H * (K + 1), D), dtype=torch.float32, device=dev)
+    part_dq = torch.empty((S * H * (K + 1), D), dtype=q.dtype, device=dev)
     queues = torch.empty(16, dtype=torch.int32, device=dev)  # tile counters of the two backward kernels (zeroed there)
     _lib.check(lib.moba_bwd(_ptr(dout), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(sel), _ptr(seg_off),
                             _ptr(tile_off), _ptr(seg_dest), _ptr(t.get("fchunk_tok")), _ptr(t["chunk_tok"]),
