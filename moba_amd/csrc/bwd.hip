@@ -43,7 +43,7 @@ struct BwdParams {
   const float* lse;    // [S*H] natural log
   const float* delta;  // [S*H]
   const float* lse2;   // [S*H] lse in the log2 domain
-  typename E::elem* part_dq;  // [S*H*K1, D]: per-slot dQ before the softmax scale, in the element type
+  typename E::elem* part_dq;  // [S*H*K1, D]: per-slot dQ in the element type
   typename E::elem* dk;
   typename E::elem* dv;
   const int* chunk_fid;  // [N] filtered id of a chunk, -1 for the last chunk of a sequence
@@ -298,8 +298,9 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams<E> p) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         u32x2 w;
-        w[0] = pack2<E>(dqacc[db][4 * g + 0], dqacc[db][4 * g + 1]);
-        w[1] = pack2<E>(dqacc[db][4 * g + 2], dqacc[db][4 * g + 3]);
+        // (scaled before the rounding: a partial then overflows fp16 only where dQ itself would)
+        w[0] = pack2<E>(dqacc[db][4 * g + 0] * p.scale, dqacc[db][4 * g + 1] * p.scale);
+        w[1] = pack2<E>(dqacc[db][4 * g + 2] * p.scale, dqacc[db][4 * g + 3] * p.scale);
         // elements 32*db + 8*g + 4*hh .. +3 of row n: 16-byte column 4*db + g, swizzled by the row
         *reinterpret_cast<u32x2*>(wrow + (((4 * db + g) ^ (n & 15)) << 4)) = w;
       }
@@ -316,12 +317,11 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams<E> p) {
   }  // tiles
 }
 
-// dq[row] = scale * sum over the row's valid slots of part_dq; 16 lanes per row
+// dq[row] = sum over the row's valid slots of part_dq (in fp32); 16 lanes per row
 template <class E>
 __global__ __launch_bounds__(256) void bwd_dq_reduce_kernel(const typename E::elem* __restrict__ part_dq,
                                                             const int* __restrict__ sel,
-                                                            typename E::elem* __restrict__ dq, int64_t rows, int K1,
-                                                            float scale) {
+                                                            typename E::elem* __restrict__ dq, int64_t rows, int K1) {
   MOBA_ELEM_TYPES(E)
   const int64_t row_raw = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
   const bool row_ok = row_raw < rows;
@@ -360,7 +360,7 @@ __global__ __launch_bounds__(256) void bwd_dq_reduce_kernel(const typename E::el
   if (!row_ok) return;
   elem8 o;
 #pragma unroll
-  for (int e = 0; e < 8; ++e) o[e] = (elem)(acc[e] * scale);
+  for (int e = 0; e < 8; ++e) o[e] = (elem)acc[e];
   *reinterpret_cast<elem8*>(dq + row * kHeadDim + c8 * 8) = o;
 }
 
@@ -730,7 +730,7 @@ static int launch_bwd(const void* dout, const void* q, const void* k, const void
   hipLaunchKernelGGL(zero_queues_kernel, dim3(1), dim3(16), 0, st, queues);  // a kernel, not a memset: graph safe
   hipLaunchKernelGGL(bwd_dq_kernel<E>, dim3((unsigned)grid_q), dim3(256), kBwdDqLds, st, p);
   hipLaunchKernelGGL(bwd_dq_reduce_kernel<E>, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st,
-                     (const elem*)part_dq, sel, (elem*)dq, rows, K + 1, p.scale);
+                     (const elem*)part_dq, sel, (elem*)dq, rows, K + 1);
   hipLaunchKernelGGL(bwd_dkv_kernel<E>, dim3((unsigned)grid_kv), dim3(256), kBwdDkvLds, st, p);
   return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
 }
