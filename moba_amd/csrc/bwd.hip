@@ -536,37 +536,43 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
   auto phase_a = [&](f32x16& s_next, f32x16& dp_next, const f32x16& s_cur, const f32x16& dp_cur, auto masked_c,
                      int qb, int rows_ok, bool is_self, int qpos0, elem8 (&pb)[2], elem8 (&dsb)[2], auto dma)
                      __attribute__((always_inline)) {
-    f32x16 zero;
-#pragma unroll
-    for (int e = 0; e < 16; ++e) zero[e] = 0.f;
     __builtin_amdgcn_sched_barrier(0);
+    // The product of element e is formed in the slot of element e+1: an exponential followed at once by
+    // an instruction that uses it costs an idle issue cycle.
+    float pe[16], ds[16];
 #pragma unroll
     for (int k = 0; k < 16; k += 2) {
       const int s8 = k >> 1;
-      float pe[2], ds[2];
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
-        if (u == 0) s_next = mfma32(qa[s8], bk[s8], s8 == 0 ? zero : s_next);
-        else        dp_next = mfma32(oa[s8], bv[s8], s8 == 0 ? zero : dp_next);
+        if (u == 0) mfma32_into_vgprs(s_next, qa[s8], bk[s8], s8 == 0);
+        else        mfma32_into_vgprs(dp_next, oa[s8], bv[s8], s8 == 0);
         const int e = k + u, g = e >> 2, rr = e & 3;
-        pe[u] = fast_exp2(s_cur[e] * sl2 - l4[g][rr]);
+        pe[e] = fast_exp2(s_cur[e] * sl2 - l4[g][rr]);
+        if (e > 0) {
+          ds[e - 1] = pe[e - 1] * (dp_cur[e - 1] - d4[(e - 1) >> 2][(e - 1) & 3]);
+          MOBA_PIN(ds[e - 1]);
+        }
         if constexpr (decltype(masked_c)::value) {
           const int row = 32 * qb + 8 * g + 4 * hh + rr;
           const bool ok = (row < rows_ok) && (!is_self || qpos0 + row >= mykey);
-          pe[u] = ok ? pe[u] : 0.f;
+          pe[e] = ok ? pe[e] : 0.f;
         }
-        ds[u] = pe[u] * (dp_cur[e] - d4[g][rr]);
-        MOBA_PIN(pe[u]);
-        MOBA_PIN(ds[u]);
+        MOBA_PIN(pe[e]);
         __builtin_amdgcn_sched_barrier(0);
       }
-      pb[k >> 3][k & 7] = (elem)pe[0];
-      pb[k >> 3][(k & 7) + 1] = (elem)pe[1];
-      dsb[k >> 3][k & 7] = (elem)ds[0];
-      dsb[k >> 3][(k & 7) + 1] = (elem)ds[1];
+      pb[k >> 3][k & 7] = (elem)pe[k];
+      pb[k >> 3][(k & 7) + 1] = (elem)pe[k + 1];
+      if (k > 0) {
+        dsb[(k - 2) >> 3][(k - 2) & 7] = (elem)ds[k - 2];
+        dsb[(k - 2) >> 3][((k - 2) & 7) + 1] = (elem)ds[k - 1];
+      }
       dma(k >> 1);  // one global -> LDS copy (or nothing) per pair of MFMAs
       __builtin_amdgcn_sched_barrier(0);
     }
+    ds[15] = pe[15] * (dp_cur[15] - d4[3][3]);
+    dsb[1][6] = (elem)ds[14];
+    dsb[1][7] = (elem)ds[15];
     __builtin_amdgcn_sched_barrier(0);
   };
   // accumulate block (qs, qb); then fetch the fragments of (qs_f, qb_f) and the statistics of (qs_s, qb_s)

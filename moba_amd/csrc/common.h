@@ -60,6 +60,23 @@ __device__ __forceinline__ f32x16 mfma32(f16x8 a, f16x8 b, f32x16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
 }
 
+// The same product with the result in ordinary vector registers and the operands in accumulation
+// registers, for a kernel that needs the accumulation registers at all: there the compiler gives every
+// builtin MFMA the accumulation-register form, and a result that vector instructions consume is then
+// copied out one register at a time.  `first` (a constant once loops are unrolled) starts from zero
+// instead of from d.
+// The compiler does not see a matrix instruction here and inserts no wait states after it: the caller
+// keeps every other access to d at least two later matrix instructions away (they queue behind this
+// one), chained accumulations into the same d excepted, which the hardware orders itself.
+__device__ __forceinline__ void mfma32_into_vgprs(f32x16& d, bf16x8 a, bf16x8 b, bool first) {
+  if (first) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=v"(d) : "a"(a), "a"(b));
+  else                 asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "a"(a), "a"(b));
+}
+__device__ __forceinline__ void mfma32_into_vgprs(f32x16& d, f16x8 a, f16x8 b, bool first) {
+  if (first) asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=v"(d) : "a"(a), "a"(b));
+  else                 asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(d) : "a"(a), "a"(b));
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
