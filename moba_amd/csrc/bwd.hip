@@ -575,49 +575,56 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
     dsb[1][7] = (elem)ds[15];
     __builtin_amdgcn_sched_barrier(0);
   };
-  // accumulate block (qs, qb); then fetch the fragments of (qs_f, qb_f) and the statistics of (qs_s, qb_s)
+  // accumulate block (qs, qb); meanwhile fetch the fragments of (qs_f, qb_f) and the statistics of (qs_s, qb_s).
+  // Eight slots of two MFMAs; the four transposed reads of a slot are issued two slots ahead (an LDS read takes
+  // longer than a slot), the 24 prefetch reads ride along, three per slot.
   auto phase_b = [&](const char* qs, int qb, const elem8 (&pb)[2], const elem8 (&dsb)[2], const char* qs_f, int qb_f,
                      const char* qs_s, int qb_s) __attribute__((always_inline)) {
     const char* os = qs + TQ * kHeadDim * 2;
-#pragma unroll
-    for (int j2 = 0; j2 < 2; ++j2) {
+    const char* os_f = qs_f + TQ * kHeadDim * 2;
+    const float* lse_s = reinterpret_cast<const float*>(qs_s + 2 * TQ * kHeadDim * 2);
+    const float* del_s = lse_s + TQ;
+    elem4 ring[3][4];
+    auto issue = [&](int idx, int r) __attribute__((always_inline)) {
+      const int j2 = idx >> 2, db = idx & 3;
       const int rowA = 32 * qb + 16 * j2 + 4 * hh + i0;
       const int rowB = rowA + 8;
-#pragma unroll
-      for (int db = 0; db < 4; ++db) {
-        const int c16 = 4 * db + tr_c16;
-        const int offA = rowA * 256 + ((c16 ^ (i0 << 2) ^ hh) << 4) + tr_sub;
-        const int offB = rowB * 256 + ((c16 ^ (i0 << 2) ^ (hh + 2)) << 4) + tr_sub;
-        const elem4 oa4 = lds_read_tr<elem4>(os + offA);
-        const elem4 ob4 = lds_read_tr<elem4>(os + offB);
-        const elem4 qa4 = lds_read_tr<elem4>(qs + offA);
-        const elem4 qb4 = lds_read_tr<elem4>(qs + offB);
-        elem8 ao, aq;
-        ao[0] = oa4[0]; ao[1] = oa4[1]; ao[2] = oa4[2]; ao[3] = oa4[3];
-        ao[4] = ob4[0]; ao[5] = ob4[1]; ao[6] = ob4[2]; ao[7] = ob4[3];
-        aq[0] = qa4[0]; aq[1] = qa4[1]; aq[2] = qa4[2]; aq[3] = qa4[3];
-        aq[4] = qb4[0]; aq[5] = qb4[1]; aq[6] = qb4[2]; aq[7] = qb4[3];
-        dvacc[db] = mfma32(ao, pb[j2], dvacc[db]);
-        dkacc[db] = mfma32(aq, dsb[j2], dkacc[db]);
-      }
-    }
-    load_stats(qs_s, qb_s);
-    load_frags(qs_f, qb_f);
-    // 8 transposed reads ahead, then four reads per pair of MFMAs; the prefetches ride behind
-    __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
-#pragma unroll
-    for (int i = 0; i < 6; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-    }
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-    __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-    __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-    __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      const int c16 = 4 * db + tr_c16;
+      const int offA = rowA * 256 + ((c16 ^ (i0 << 2) ^ hh) << 4) + tr_sub;
+      const int offB = rowB * 256 + ((c16 ^ (i0 << 2) ^ (hh + 2)) << 4) + tr_sub;
+      ring[r][0] = lds_read_tr<elem4>(os + offA);
+      ring[r][1] = lds_read_tr<elem4>(os + offB);
+      ring[r][2] = lds_read_tr<elem4>(qs + offA);
+      ring[r][3] = lds_read_tr<elem4>(qs + offB);
+    };
     __builtin_amdgcn_sched_barrier(0);
+    issue(0, 0);
+    issue(1, 1);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int idx = 0; idx < 8; ++idx) {
+      const int r = idx % 3;
+      if (idx + 2 < 8) issue(idx + 2, (idx + 2) % 3);
+      // prefetches: statistics in the first four slots, two row fragments in every slot
+      if (idx < 4) {
+        l4[idx] = *reinterpret_cast<const f32x4*>(lse_s + 32 * qb_s + 8 * idx + 4 * hh);
+        d4[idx] = *reinterpret_cast<const f32x4*>(del_s + 32 * qb_s + 8 * idx + 4 * hh);
+      }
+      {
+        const int o = qb_f * 8192 + row_off + (((2 * idx + hh) ^ row_sw) << 4);
+        qa[idx] = *reinterpret_cast<const elem8*>(qs_f + o);
+        oa[idx] = *reinterpret_cast<const elem8*>(os_f + o);
+      }
+      elem8 ao, aq;
+      ao[0] = ring[r][0][0]; ao[1] = ring[r][0][1]; ao[2] = ring[r][0][2]; ao[3] = ring[r][0][3];
+      ao[4] = ring[r][1][0]; ao[5] = ring[r][1][1]; ao[6] = ring[r][1][2]; ao[7] = ring[r][1][3];
+      aq[0] = ring[r][2][0]; aq[1] = ring[r][2][1]; aq[2] = ring[r][2][2]; aq[3] = ring[r][2][3];
+      aq[4] = ring[r][3][0]; aq[5] = ring[r][3][1]; aq[6] = ring[r][3][2]; aq[7] = ring[r][3][3];
+      const int j2 = idx >> 2, db = idx & 3;
+      dvacc[db] = mfma32(ao, pb[j2], dvacc[db]);
+      dkacc[db] = mfma32(aq, dsb[j2], dkacc[db]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
   };
 
   for (int hq = hkv * rep; hq < (hkv + 1) * rep; ++hq) {
