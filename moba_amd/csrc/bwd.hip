@@ -247,6 +247,19 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams<E> p) {
         }
         __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
         __builtin_amdgcn_sched_barrier(0);
+        // the first K^T operands of the dQ product travel while the exponentials run
+        elem4 tr[8][2];
+        auto issue_tr = [&](int idx) __attribute__((always_inline)) {
+          const int j2 = idx >> 2, db = idx & 3;
+          const int keyA = 16 * (2 * kb + j2) + 4 * hh + i0;
+          const int keyB = keyA + 8;
+          const int c16 = 4 * db + tr_c16;
+          tr[idx][0] = lds_read_tr<elem4>(ks + keyA * 256 + ((c16 ^ (i0 << 2) ^ hh) << 4) + tr_sub);
+          tr[idx][1] = lds_read_tr<elem4>(ks + keyB * 256 + ((c16 ^ (i0 << 2) ^ (hh + 2)) << 4) + tr_sub);
+        };
+#pragma unroll
+        for (int idx = 0; idx < 4; ++idx) issue_tr(idx);
+        __builtin_amdgcn_sched_barrier(0);
         if (masked) {
 #pragma unroll
           for (int e = 0; e < 16; ++e) {
@@ -260,22 +273,16 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams<E> p) {
           const float pe = fast_exp2(sacc[e] * sl2 - lse2);
           dsb[e >> 3][e & 7] = (elem)(pe * (dpacc[e] - dl));
         }
+        __builtin_amdgcn_sched_barrier(0);
         // dQ^T += K^T dS^T
 #pragma unroll
-        for (int j2 = 0; j2 < 2; ++j2) {
-          const int j = 2 * kb + j2;
-          const int keyA = 16 * j + 4 * hh + i0;
-          const int keyB = keyA + 8;
-#pragma unroll
-          for (int db = 0; db < 4; ++db) {
-            const int c16 = 4 * db + tr_c16;
-            const elem4 xa = lds_read_tr<elem4>(ks + keyA * 256 + ((c16 ^ (i0 << 2) ^ hh) << 4) + tr_sub);
-            const elem4 xb = lds_read_tr<elem4>(ks + keyB * 256 + ((c16 ^ (i0 << 2) ^ (hh + 2)) << 4) + tr_sub);
-            elem8 a;
-            a[0] = xa[0]; a[1] = xa[1]; a[2] = xa[2]; a[3] = xa[3];
-            a[4] = xb[0]; a[5] = xb[1]; a[6] = xb[2]; a[7] = xb[3];
-            dqacc[db] = mfma32(a, dsb[j2], dqacc[db]);
-          }
+        for (int idx = 0; idx < 8; ++idx) {
+          if (idx + 4 < 8) issue_tr(idx + 4);
+          elem8 a;
+          a[0] = tr[idx][0][0]; a[1] = tr[idx][0][1]; a[2] = tr[idx][0][2]; a[3] = tr[idx][0][3];
+          a[4] = tr[idx][1][0]; a[5] = tr[idx][1][1]; a[6] = tr[idx][1][2]; a[7] = tr[idx][1][3];
+          dqacc[idx & 3] = mfma32(a, dsb[idx >> 2], dqacc[idx & 3]);
+          __builtin_amdgcn_sched_barrier(0);
         }
       }
     }
