@@ -9,8 +9,9 @@
 //
 //   bwd_delta_kernel     delta[token, head]
 //   bwd_dq_kernel        row-tile major, same tiling as the forward: each tile (128
-//                        query rows x the keys of one chunk) writes its fp32 partial dQ
-//                        into the row's slot; bwd_dq_reduce_kernel sums the K+1 slots
+//                        query rows x the keys of one chunk) writes its partial dQ, scaled
+//                        and rounded to the element type, into the row's slot;
+//                        bwd_dq_reduce_kernel sums the K+1 slots in fp32
 //   bwd_dkv_kernel       key-tile major: a workgroup owns 128 keys of (chunk, head) and
 //                        walks first the causal rows of the same chunk, then the gather
 //                        list of rows that selected the chunk; dK/dV accumulate in
