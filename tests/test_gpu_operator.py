@@ -247,6 +247,29 @@ def test_backward_is_deterministic():
         assert torch.equal(a, b)
 
 
+def test_float16_large_gradients_stay_finite():
+    """dQ = scale * dS K is summed from per-chunk partials kept in the element type.  The partials are
+    scaled before they are rounded, so they leave the fp16 range only where dQ itself would: here
+    dQ / scale reaches 2.5e5 (beyond fp16) while dQ stays near 2e4."""
+    from moba_amd import moba_efficient as E
+    q, k, v, do, cu, mx = make_case(1, 512, 2, seed=5, dtype=torch.float16)
+    q = (q.float() * 1e-3).half()
+    k = (k.float() * 300).half()
+    v = (v.float() * 30).half()
+    cu_t = torch.tensor(cu, dtype=torch.int32, device="cuda")
+    qg, kg, vg = (x.cuda().requires_grad_(True) for x in (q, k, v))
+    out = E.moba_attn_varlen(qg, kg, vg, cu_t, mx, moba_chunk_size=128, moba_topk=2)
+    out.backward(do.cuda())
+    qc, kc, vc = (x.float().clone().requires_grad_(True) for x in (q, k, v))
+    ref = O.moba_attn_varlen_oracle(qc, kc, vc, cu, mx, 128, 2)
+    ref.backward(do.float())
+    assert qc.grad.abs().max() * 128 ** 0.5 > 65504 > qc.grad.abs().max()   # the case is what it claims to be
+    for got, want in ((out, ref), (qg.grad, qc.grad), (kg.grad, kc.grad), (vg.grad, vc.grad)):
+        got = got.detach().cpu().float()
+        assert torch.isfinite(got).all()
+        assert (got - want.detach()).abs().max() <= 1e-2 * want.detach().abs().max()
+
+
 def test_argument_validation():
     from moba_amd import moba_attn_varlen
     q = torch.zeros((64, 2, 128), dtype=torch.bfloat16, device="cuda")
