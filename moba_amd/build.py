@@ -51,6 +51,11 @@ def build(force: bool = True, verbose: bool = True) -> str:
     srcs = [s for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
     with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as ex:
         objs = list(ex.map(lambda s: _compile(s, force), srcs))
+    # the hand-issued MFMAs of the dK/dV kernel: nothing touches their results too early in the generated code
+    from . import asm_check
+    report = asm_check.check_dkv_kernel(asm_check.device_assembly(HIPCC, FLAGS, os.path.join(CSRC, "bwd.hip")))
+    if verbose:
+        print(report)
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:

@@ -694,6 +694,9 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
     phase_b(qs, 1, pb, dsb, qs_next, 1, qs_next, 0);
     buf = buf1;
   }
+  // The last phase A left an S and a dO V^T that nobody reads: their registers may be reused at once on the way
+  // out of the loop, and the compiler puts no wait states behind the hand-issued MFMAs that wrote them.
+  asm volatile("s_nop 15");
   }  // query heads
 
   if (key_valid) {
