@@ -7,7 +7,8 @@
  * `stream` is a hipStream_t.
  * The library allocates nothing, frees nothing, and never synchronises the device:
  * every launch is enqueued on `stream`.  Return value: 0, or a negative code that
- * moba_strerror() explains.  head_dim 128; q, k, v and everything derived from them are
+ * moba_strerror() explains.  head_dim 128 (D below; narrower heads are padded with zeros by the
+ * caller, see softmax_scale); q, k, v and everything derived from them are
  * bf16 (dtype = MOBA_DTYPE_BF16) or fp16 (dtype = MOBA_DTYPE_F16, the dtype of the reference's
  * example, examples/llama.py:26); below, "elem" stands for that type.
  *
@@ -95,22 +96,25 @@ int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, const int32_t
  *   self_tiles: self_tile_prefix[N]
  *   queues [8] int32 scratch: the tile counters of the forward kernel, whose workgroups (two per CU) stay
  *              resident and draw tiles from one queue per XCD; the call zeroes them with a kernel of its own.
- *              Calls that overlap in time need their own eight counters each. */
+ *              Calls that overlap in time need their own eight counters each.
+ *   softmax_scale: the factor on q k^T; 0 (or less) stands for D^-0.5, the reference's only choice
+ *              (moba/moba_efficient.py:86).  A caller whose heads are narrower than D pads them with zeros
+ *              and passes its own head_dim^-0.5. */
 int moba_fwd_tile_rows(void);
 int moba_fwd_partials(const void* q, const void* k, const void* v, void* part_o, float* part_lse,
                       const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest,
                       const int32_t* fchunk_tok, const int32_t* chunk_tok, const int32_t* self_tile_prefix,
                       const int32_t* tile_seg, const int32_t* self_tile_chunk, int64_t S, int H, int Hkv, int D, int K,
                       int F, int N, int B, int64_t hist_bound, int64_t self_tiles, const int64_t* strides,
-                      int32_t* queues, int dtype, void* stream);
+                      int32_t* queues, float softmax_scale, int dtype, void* stream);
 int moba_fwd_merge(const void* part_o, const float* part_lse, const int32_t* sel, void* out, float* lse, int64_t S,
                    int H, int D, int K, int dtype, void* stream);
 int moba_fwd(const void* q, const void* k, const void* v, void* part_o, float* part_lse, const int32_t* sel,
              const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest, const int32_t* fchunk_tok,
              const int32_t* chunk_tok, const int32_t* self_tile_prefix, const int32_t* tile_seg,
              const int32_t* self_tile_chunk, void* out, float* lse, int64_t S, int H, int Hkv, int D, int K, int F,
-             int N, int B, int64_t hist_bound, int64_t self_tiles, const int64_t* strides, int32_t* queues, int dtype,
-             void* stream);
+             int N, int B, int64_t hist_bound, int64_t self_tiles, const int64_t* strides, int32_t* queues,
+             float softmax_scale, int dtype, void* stream);
 
 /* Backward.  Replaces MixedAttention.backward, moba/moba_efficient.py:185-267, and the
  * autograd scatter of its gathered gradients.  Deterministic (no floating-point atomics).
@@ -119,14 +123,15 @@ int moba_fwd(const void* q, const void* k, const void* v, void* part_o, float* p
  *   chunk_fid [N] int32: filtered id of each chunk, -1 for the last chunk of a sequence
  *   delta [2,S,H] fp32 scratch (rowsum(dO*O), then the LSE in the log2 domain); part_dq [S*H*(K+1), D] elem scratch (the per-slot dQ, rounded as the per-chunk dQ that flash-attn returns to the reference is)
  *   dq, dk, dv: out; dk and dv of a key/value head sum over its query heads
- *   queues [16] int32 scratch: tile counters of the dQ and dK/dV kernels (as in moba_fwd_partials) */
+ *   queues [16] int32 scratch: tile counters of the dQ and dK/dV kernels (as in moba_fwd_partials)
+ *   softmax_scale: as in the forward call */
 int moba_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out, const float* lse,
              const int32_t* sel, const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest,
              const int32_t* fchunk_tok, const int32_t* chunk_tok, const int32_t* self_tile_prefix,
              const int32_t* tile_seg, const int32_t* self_tile_chunk, const int32_t* chunk_fid, float* delta,
              void* part_dq, void* dq, void* dk, void* dv, int64_t S, int H, int Hkv, int D, int K, int F, int N, int B,
-             int64_t hist_bound, int64_t self_tiles, const int64_t* strides, int32_t* queues, int dtype,
-             void* stream);
+             int64_t hist_bound, int64_t self_tiles, const int64_t* strides, int32_t* queues, float softmax_scale,
+             int dtype, void* stream);
 
 /* Decode: one query token per sequence against the key/value cache.  Replaces the
  * flash_attn_func call of the adapter's decode branch, moba/wrapper.py:76-82 (full attention

@@ -725,8 +725,8 @@ using namespace moba;
 template <class E>
 static int launch_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out, const float* lse,
                       const int32_t* sel, const int32_t* chunk_fid, float* delta, void* part_dq, void* dq, void* dk,
-                      void* dv, const TileTables& t, int64_t S, int H, int D, int K, int64_t grid_q, int64_t grid_kv,
-                      int* queues, hipStream_t st) {
+                      void* dv, const TileTables& t, int64_t S, int H, int D, int K, float softmax_scale, int64_t grid_q,
+                      int64_t grid_kv, int* queues, hipStream_t st) {
   typedef typename E::elem elem;
   BwdParams<E> p;
   p.q = (const elem*)q; p.k = (const elem*)k; p.v = (const elem*)v; p.dout = (const elem*)dout;
@@ -734,8 +734,9 @@ static int launch_bwd(const void* dout, const void* q, const void* k, const void
   p.chunk_fid = chunk_fid;
   p.queues = queues;
   p.t = t;
-  p.scale = (float)(1.0 / sqrt((double)D));
-  p.scale_log2 = (float)(1.4426950408889634 / sqrt((double)D));
+  p.scale = softmax_scale > 0.f ? softmax_scale : (float)(1.0 / sqrt((double)D));
+  p.scale_log2 = softmax_scale > 0.f ? (float)(1.4426950408889634 * (double)softmax_scale)
+                                     : (float)(1.4426950408889634 / sqrt((double)D));
   // division by H*K1 as a multiplication: with s = 31 + ceil(log2 d) and m = floor(2^s / d) + 1 the
   // error m*d - 2^s is at most d <= 2^(s-31), so n*m >> s is the exact quotient for n < 2^31; m < 2^32
   const uint64_t hk = (uint64_t)H * (K + 1);
@@ -765,8 +766,8 @@ extern "C" int moba_bwd(const void* dout, const void* q, const void* k, const vo
                         const int32_t* self_tile_prefix, const int32_t* tile_seg, const int32_t* self_tile_chunk,
                         const int32_t* chunk_fid, float* delta, void* part_dq,
                         void* dq, void* dk, void* dv, int64_t S, int H, int Hkv, int D, int K, int F, int N, int B,
-                        int64_t hist_bound, int64_t self_tiles, const int64_t* strides, int32_t* queues, int dtype,
-                        void* stream) {
+                        int64_t hist_bound, int64_t self_tiles, const int64_t* strides, int32_t* queues,
+                        float softmax_scale, int dtype, void* stream) {
   if (!dout || !q || !k || !v || !out || !lse || !chunk_tok || !self_tile_prefix || !self_tile_chunk || !delta ||
       !part_dq || !dq || !dk || !dv || !queues)
     return MOBA_ERR_ARG;
@@ -798,7 +799,7 @@ extern "C" int moba_bwd(const void* dout, const void* q, const void* k, const vo
   hipStream_t st = (hipStream_t)stream;
   return dtype == MOBA_DTYPE_F16
              ? launch_bwd<F16>(dout, q, k, v, out, lse, sel, chunk_fid, delta, part_dq, dq, dk, dv, t, S, H, D, K,
-                               grid_q, grid_kv, queues, st)
+                               softmax_scale, grid_q, grid_kv, queues, st)
              : launch_bwd<Bf16>(dout, q, k, v, out, lse, sel, chunk_fid, delta, part_dq, dq, dk, dv, t, S, H, D, K,
-                                grid_q, grid_kv, queues, st);
+                                softmax_scale, grid_q, grid_kv, queues, st);
 }

@@ -549,12 +549,14 @@ extern "C" int moba_fwd_tile_rows(void) { return TM; }
 
 template <class E>
 static int launch_partials(const void* q, const void* k, const void* v, void* part_o, float* part_lse,
-                           const TileTables& t, int D, int64_t grid, int* queues, hipStream_t st) {
+                           const TileTables& t, int D, float softmax_scale, int64_t grid, int* queues,
+                           hipStream_t st) {
   FwdParams<E> p;
   p.q = (const typename E::elem*)q; p.k = (const typename E::elem*)k; p.v = (const typename E::elem*)v;
   p.part_o = (typename E::elem*)part_o; p.part_lse = part_lse;
   p.t = t;
-  p.scale_log2 = (float)(1.4426950408889634 / sqrt((double)D));
+  p.scale_log2 = softmax_scale > 0.f ? (float)(1.4426950408889634 * (double)softmax_scale)
+                                     : (float)(1.4426950408889634 / sqrt((double)D));
   p.queues = queues;
   static bool allowed[2][kMaxDevices];  // one pair of arrays per element type
   if (grid > 0) {  // resident workgroups drawing from the queues
@@ -575,7 +577,7 @@ extern "C" int moba_fwd_partials(const void* q, const void* k, const void* v, vo
                                  const int32_t* self_tile_prefix, const int32_t* tile_seg,
                                  const int32_t* self_tile_chunk, int64_t S, int H, int Hkv, int D, int K, int F,
                                  int N, int B, int64_t hist_bound, int64_t self_tiles, const int64_t* strides,
-                                 int32_t* queues, int dtype, void* stream) {
+                                 int32_t* queues, float softmax_scale, int dtype, void* stream) {
   if (!q || !k || !v || !part_o || !part_lse || !chunk_tok || !self_tile_prefix || !self_tile_chunk || !queues)
     return MOBA_ERR_ARG;
   if (Hkv <= 0 || H % Hkv != 0) return MOBA_ERR_ARG;
@@ -604,8 +606,9 @@ extern "C" int moba_fwd_partials(const void* q, const void* k, const void* v, vo
   t.self_total = (int)(self_tiles * H);
   if (!set_layout(t, strides)) return MOBA_ERR_ARG;
   hipStream_t st = (hipStream_t)stream;
-  return dtype == MOBA_DTYPE_F16 ? launch_partials<F16>(q, k, v, part_o, part_lse, t, D, grid, queues, st)
-                                 : launch_partials<Bf16>(q, k, v, part_o, part_lse, t, D, grid, queues, st);
+  return dtype == MOBA_DTYPE_F16
+             ? launch_partials<F16>(q, k, v, part_o, part_lse, t, D, softmax_scale, grid, queues, st)
+             : launch_partials<Bf16>(q, k, v, part_o, part_lse, t, D, softmax_scale, grid, queues, st);
 }
 
 extern "C" int moba_fwd_merge(const void* part_o, const float* part_lse, const int32_t* sel, void* out, float* lse,
@@ -630,11 +633,11 @@ extern "C" int moba_fwd(const void* q, const void* k, const void* v, void* part_
                         const int32_t* seg_dest, const int32_t* fchunk_tok, const int32_t* chunk_tok,
                         const int32_t* self_tile_prefix, const int32_t* tile_seg, const int32_t* self_tile_chunk,
                         void* out, float* lse, int64_t S, int H, int Hkv, int D, int K, int F, int N, int B,
-                        int64_t hist_bound, int64_t self_tiles, const int64_t* strides, int32_t* queues, int dtype,
-                        void* stream) {
+                        int64_t hist_bound, int64_t self_tiles, const int64_t* strides, int32_t* queues,
+                        float softmax_scale, int dtype, void* stream) {
   int rc = moba_fwd_partials(q, k, v, part_o, part_lse, seg_off, tile_off, seg_dest, fchunk_tok, chunk_tok,
                              self_tile_prefix, tile_seg, self_tile_chunk, S, H, Hkv, D, K, F, N, B, hist_bound,
-                             self_tiles, strides, queues, dtype, stream);
+                             self_tiles, strides, queues, softmax_scale, dtype, stream);
   if (rc != MOBA_OK) return rc;
   return moba_fwd_merge(part_o, part_lse, sel, out, lse, S, H, D, K, dtype, stream);
 }

@@ -91,8 +91,8 @@ def _check_qkv(q, k, v, gqa=False):
             raise ValueError("the number of query heads must be a multiple of the number of key/value heads")
     elif q.shape != k.shape:
         raise ValueError("q, k, v must all be [seqlen, heads, head_dim] with the same number of heads")
-    if q.shape[2] != HEAD_DIM:
-        raise ValueError(f"head_dim must be {HEAD_DIM}")
+    if not 0 < q.shape[2] <= HEAD_DIM:
+        raise ValueError(f"head_dim must be at most {HEAD_DIM} (narrower heads are padded with zeros)")
 
 
 # ----------------------------------------------------------------------------- stages
@@ -197,7 +197,7 @@ class _NoSpan:
         return False
 
 
-def _forward(q, k, v, plan: MobaPlan, timer: Optional[StageTimer] = None):
+def _forward(q, k, v, plan: MobaPlan, timer: Optional[StageTimer] = None, scale: float = 0.0):
     lib = _lib.load()
     S, H, D = q.shape
     dev = q.device
@@ -224,14 +224,14 @@ def _forward(q, k, v, plan: MobaPlan, timer: Optional[StageTimer] = None):
                                          _ptr(t["chunk_tok"]), _ptr(t["self_tile_prefix"]), _ptr(tile_seg),
                                          _ptr(t["self_tile_chunk"]), S, H, k.shape[1], D, K, plan.F, plan.N,
                                          plan.chunk_size, plan.hist_tile_bound(H), plan.self_tiles, _strides(q, k),
-                                         _ptr(queues), _dtype_code(q), _stream(dev)), "moba_fwd_partials")
+                                         _ptr(queues), scale, _dtype_code(q), _stream(dev)), "moba_fwd_partials")
     with span("fwd_merge"):
         _lib.check(lib.moba_fwd_merge(_ptr(part_o), _ptr(part_lse), _ptr(sel), _ptr(out), _ptr(lse), S, H, D, K,
                                       _dtype_code(q), _stream(dev)), "moba_fwd_merge")
     return out, lse, sel, seg_off, tile_off, seg_dest, tile_seg
 
 
-def _backward(dout, q, k, v, out, lse, sel, seg_off, tile_off, seg_dest, tile_seg, plan: MobaPlan):
+def _backward(dout, q, k, v, out, lse, sel, seg_off, tile_off, seg_dest, tile_seg, plan: MobaPlan, scale: float = 0.0):
     lib = _lib.load()
     S, H, D = q.shape
     dev = q.device
@@ -248,7 +248,8 @@ def _backward(dout, q, k, v, out, lse, sel, seg_off, tile_off, seg_dest, tile_se
                             _ptr(t["self_tile_prefix"]), _ptr(tile_seg), _ptr(t["self_tile_chunk"]),
                             _ptr(t.get("chunk_fid")), _ptr(delta), _ptr(part_dq), _ptr(dq), _ptr(dk), _ptr(dv),
                             S, H, k.shape[1], D, K, plan.F, plan.N, plan.chunk_size, plan.hist_tile_bound(H),
-                            plan.self_tiles, _strides(q, k), _ptr(queues), _dtype_code(q), _stream(dev)), "moba_bwd")
+                            plan.self_tiles, _strides(q, k), _ptr(queues), scale, _dtype_code(q), _stream(dev)),
+               "moba_bwd")
     return dq, dk, dv
 
 
@@ -256,9 +257,10 @@ class _MobaAttention(torch.autograd.Function):
     """Counterpart of ``MixedAttention`` (moba/moba_efficient.py:67-267)."""
 
     @staticmethod
-    def forward(ctx, q, k, v, plan, timer=None):
-        out, lse, sel, seg_off, tile_off, seg_dest, tile_seg = _forward(q, k, v, plan, timer)
+    def forward(ctx, q, k, v, plan, timer=None, scale=0.0):
+        out, lse, sel, seg_off, tile_off, seg_dest, tile_seg = _forward(q, k, v, plan, timer, scale)
         ctx.plan = plan
+        ctx.scale = scale
         ctx.aux = (sel, seg_off, tile_off, seg_dest, tile_seg)
         ctx.save_for_backward(q, k, v, out, lse)
         ctx.mark_non_differentiable(lse)
@@ -269,8 +271,8 @@ class _MobaAttention(torch.autograd.Function):
         q, k, v, out, lse = ctx.saved_tensors
         sel, seg_off, tile_off, seg_dest, tile_seg = ctx.aux
         dq, dk, dv = _backward(_aligned(dout.to(q.dtype)), q, k, v, out, lse, sel, seg_off, tile_off, seg_dest, tile_seg,
-                               ctx.plan)
-        return dq, dk, dv, None, None
+                               ctx.plan, ctx.scale)
+        return dq, dk, dv, None, None, None
 
 
 def moba_attn_varlen(
@@ -291,6 +293,10 @@ def moba_attn_varlen(
         moba_chunk_size, moba_topk: block size and number of attended blocks (the current one included)
     Returns:
         [seqlen, heads, head_dim] in q's dtype.  Softmax scale is head_dim ** -0.5.
+
+    The kernels are built for head_dim 128.  Narrower heads are padded with zeros to 128 (the scores, the
+    gate and the softmax scale head_dim ** -0.5 are those of the narrow heads; the padding costs the work
+    and memory of 128); wider heads are refused.
     """
     return moba_attn_varlen_with_lse(q, k, v, cu_seqlens, max_seqlen, moba_chunk_size, moba_topk)[0]
 
@@ -318,5 +324,11 @@ def moba_attn_varlen_with_lse(q, k, v, cu_seqlens, max_seqlen, moba_chunk_size, 
     plan = make_plan(cu_seqlens, moba_chunk_size, moba_topk, device=q.device)
     if plan.S != q.shape[0]:
         raise ValueError(f"cu_seqlens ends at {plan.S} but q has {q.shape[0]} tokens")
+    head_dim = q.shape[2]
+    if head_dim < HEAD_DIM:
+        pad = (0, HEAD_DIM - head_dim)
+        q, k, v = (torch.nn.functional.pad(x, pad) for x in (q, k, v))
+        out, lse = _MobaAttention.apply(q, k, v, plan, timer, head_dim ** -0.5)
+        return out[..., :head_dim].contiguous(), lse
     q, k, v = _in_place(q, k, v)
     return _MobaAttention.apply(q, k, v, plan, timer)

@@ -270,6 +270,45 @@ def test_float16_large_gradients_stay_finite():
         assert (got - want.detach()).abs().max() <= 1e-2 * want.detach().abs().max()
 
 
+@pytest.mark.parametrize("head_dim,dtype", [(64, torch.bfloat16), (96, torch.float16), (40, torch.bfloat16)])
+def test_narrow_heads_are_padded(head_dim, dtype):
+    """head_dim below 128: zero padding inside the operator, softmax scale head_dim ** -0.5 (the oracle's
+    scale for these inputs), outputs and gradients of the narrow shape."""
+    from moba_amd import moba_efficient as E
+    from moba_amd.plan import make_plan
+    q, k, v, do, cu, mx = make_case(3, 1500, 4, head_dim=head_dim, seed=21, dtype=dtype)
+    cu_t = torch.tensor(cu, dtype=torch.int32, device="cuda")
+    qg, kg, vg = (x.cuda().requires_grad_(True) for x in (q, k, v))
+    out = E.moba_attn_varlen(qg, kg, vg, cu_t, mx, moba_chunk_size=128, moba_topk=3)
+    assert out.shape == q.shape and out.is_contiguous()
+    out.backward(do.cuda())
+    # the selection the GPU made on the padded tensors (the gate does not see the zeros)
+    plan = make_plan(cu_t, 128, 3)
+    pad = (0, 128 - head_dim)
+    qp, kp = (torch.nn.functional.pad(x.cuda(), pad) for x in (q, k))
+    sel = E.gate_topk(qp, E.chunk_mean(kp, plan), plan).cpu()
+    qc, kc, vc = (x.clone().requires_grad_(True) for x in (q, k, v))
+    ref = O.moba_attn_varlen_oracle(qc, kc, vc, cu, mx, 128, 3, sel=sel)
+    ref.backward(do.float())
+    for name, got, want in (("out", out, ref), ("dq", qg.grad, qc.grad), ("dk", kg.grad, kc.grad), ("dv", vg.grad, vc.grad)):
+        assert got.shape == want.shape
+        err = (got.detach().cpu().float() - want.detach().float()).abs()
+        assert err.max() < MAX_ABS and err.mean() < MEAN_ABS, (name, err.max().item(), err.mean().item())
+    # and the selection itself is the oracle's on the narrow tensors, up to near-ties of the fp32 scores
+    want = O.select_topk(O.gate_scores(q, O.chunk_mean(k, cu, 128), cu, 128), plan.K)
+    got = torch.sort(torch.where(sel < 0, torch.full_like(sel, 1 << 30), sel), dim=-1).values
+    got = torch.where(got == 1 << 30, torch.full_like(got, -1), got)
+    assert (got != want).any(dim=-1).float().mean() < 1e-3
+
+
+def test_heads_wider_than_128_are_refused():
+    from moba_amd import moba_attn_varlen
+    q, k, v, _, cu, mx = make_case(1, 256, 1, head_dim=192, seed=3)
+    cu_t = torch.tensor(cu, dtype=torch.int32, device="cuda")
+    with pytest.raises(ValueError, match="head_dim"):
+        moba_attn_varlen(q.cuda(), k.cuda(), v.cuda(), cu_t, mx, 64, 2)
+
+
 def test_argument_validation():
     from moba_amd import moba_attn_varlen
     q = torch.zeros((64, 2, 128), dtype=torch.bfloat16, device="cuda")
