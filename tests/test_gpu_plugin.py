@@ -8,10 +8,10 @@ import torch
 pytestmark = pytest.mark.gpu
 
 
-def _model(dtype):
+def _model(dtype, head_dim=128):
     from transformers import LlamaConfig, LlamaForCausalLM
-    cfg = LlamaConfig(vocab_size=128, hidden_size=512, intermediate_size=512, num_hidden_layers=2,
-                      num_attention_heads=4, num_key_value_heads=2, head_dim=128, max_position_embeddings=2048)
+    cfg = LlamaConfig(vocab_size=128, hidden_size=4 * head_dim, intermediate_size=512, num_hidden_layers=2,
+                      num_attention_heads=4, num_key_value_heads=2, head_dim=head_dim, max_position_embeddings=2048)
     cfg._attn_implementation = "eager"
     torch.manual_seed(0)
     return LlamaForCausalLM(cfg).to(dtype).cuda().eval()
@@ -95,3 +95,21 @@ def test_generate_runs_prefill_then_decode():
     assert out.shape == (1, 304)
     # every decode step of every layer went through the HIP decode kernel, over a growing cache
     assert len(calls) == 3 * model.config.num_hidden_layers and calls[0] == 301 and calls[-1] == 303
+
+
+def test_narrow_head_model_prefill_and_generate():
+    """A model with head_dim 64: the prefill runs the HIP operator on zero-padded heads (full selection, so it
+    must reproduce eager attention), decoding goes through PyTorch SDPA (the decode kernel is built for 128)."""
+    from moba_amd import MoBAConfig, register_moba
+    register_moba(MoBAConfig(moba_chunk_size=128, moba_topk=16))
+    model = _model(torch.bfloat16, head_dim=64)
+    ids = torch.randint(0, 128, (2, 1024), device="cuda")
+    with torch.no_grad():
+        model.config._attn_implementation = "eager"
+        ref = model(ids).logits.float()
+        model.config._attn_implementation = "moba"
+        got = model(ids).logits.float()
+        out = model.generate(ids[:1, :300], max_new_tokens=3, do_sample=False)
+    err = (got - ref).abs()
+    assert err.max() < 6e-2 and err.mean() < 4e-3, (err.max().item(), err.mean().item())
+    assert out.shape == (1, 303)
