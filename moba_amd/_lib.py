@@ -40,6 +40,7 @@ _SIGNATURES = {
     "moba_decode": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_int64] * 4 + [c_float, c_int, c_void_p]),
 }
 OPTIONAL = set()
+ABI_VERSION = 101  # MOBA_ABI_VERSION of include/moba_hip.h, the signatures above
 DTYPE_BF16, DTYPE_F16 = 0, 1
 
 
@@ -63,6 +64,9 @@ def load():
             raise
         fn.restype = res
         fn.argtypes = args
+    if lib.moba_version() != ABI_VERSION:
+        raise RuntimeError(f"{LIB_PATH} was built for version {lib.moba_version()} of the C ABI, this binding is for "
+                           f"{ABI_VERSION}: rebuild it with `python -m moba_amd.build`")
     _lib = lib
     return lib
 

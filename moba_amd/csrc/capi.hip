@@ -1,7 +1,8 @@
 // Library-level entry points of the C ABI.
 #include "common.h"
 
-extern "C" int moba_version(void) { return 100; }
+// changes whenever a signature of the C ABI does: a binding made for another number must not call this library
+extern "C" int moba_version(void) { return 101; }
 
 extern "C" const char* moba_strerror(int code) {
   switch (code) {

@@ -38,8 +38,11 @@ def test_binding_covers_header():
 
 
 def test_version_and_strerror(lib):
+    from moba_amd import _lib
     lib.moba_version.restype = ctypes.c_int
-    assert lib.moba_version() >= 100
+    header = open(os.path.join(os.path.dirname(__file__), "..", "include", "moba_hip.h")).read()
+    assert f"#define MOBA_ABI_VERSION {_lib.ABI_VERSION} " in header
+    assert lib.moba_version() == _lib.ABI_VERSION
     lib.moba_strerror.restype = ctypes.c_char_p
     assert lib.moba_strerror(0) == b"ok"
     assert b"argument" in lib.moba_strerror(-1)
