@@ -369,7 +369,7 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
         sn = mfma32(ka[s8], bq[s8], sn);
       }
       pf[s8] = fast_exp2(sc[8 + s8] * sl2 - m_run);
-      rs += pf[s8];
+      if (s8 > 0) rs += pf[s8 - 1];  // one slot late: an instruction that uses a fresh exponential waits a cycle
       MOBA_PIN(pf[s8]);
       MOBA_PIN(rs);
       if (s8 >= 6) {  // first V^T fragments of phase 2
@@ -378,7 +378,7 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
       }
       __builtin_amdgcn_sched_barrier(0);
     }
-    l_run += rs;
+    l_run += rs + pf[7];
 #pragma unroll
     for (int e = 0; e < 8; ++e) pb[1][e] = (elem)pf[e];
 
