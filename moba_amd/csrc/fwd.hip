@@ -372,9 +372,9 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
       if (s8 > 0) rs += pf[s8 - 1];  // one slot late: an instruction that uses a fresh exponential waits a cycle
       MOBA_PIN(pf[s8]);
       MOBA_PIN(rs);
-      if (s8 >= 6) {  // first V^T fragments of phase 2
-        va[2 * (s8 - 6)] = v_frag(vs, kb, 0, 2 * (s8 - 6));
-        va[2 * (s8 - 6) + 1] = v_frag(vs, kb, 0, 2 * (s8 - 6) + 1);
+      if (s8 >= 4 && s8 < 6) {  // first V^T fragments of phase 2, four slots before their MFMAs
+        va[2 * (s8 - 4)] = v_frag(vs, kb, 0, 2 * (s8 - 4));
+        va[2 * (s8 - 4) + 1] = v_frag(vs, kb, 0, 2 * (s8 - 4) + 1);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
