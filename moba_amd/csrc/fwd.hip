@@ -197,6 +197,10 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
 #define MOBA_PIN(x) asm volatile("" : "+v"(x))
 
   bool have_partial = false;  // the accumulators hold a finished tile whose partial is not written yet
+  // The drawn id travels through one of two LDS words, alternating per pass: a pass without a tile has no
+  // barrier after the waves read the word, so wave 0 may already be writing the next pass's id -- into the
+  // other word.  The word of pass i is rewritten in pass i + 2, behind the barrier of pass i + 1.
+  int id_word = 0;
   int dest_done = 0, rows_done = 0;
   bool valid_done = false;
   while (true) {
@@ -289,7 +293,7 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
   // every copy of this wave has landed, and wave 0 has its draw
   wait_vmem();
   if constexpr (kQueued) {
-    if (tid == 0) *reinterpret_cast<int*>(smem + kFwdIdSlot) = drawn;
+    if (tid == 0) *reinterpret_cast<int*>(smem + kFwdIdSlot + 4 * id_word) = drawn;
   }
   if (t.row_count > 0) scrub_v(key_tile(0), 0);
   __syncthreads();
@@ -297,7 +301,8 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
     // the id drawn: queue `queue` counts the ids (8i + queue) * kQueueRun + j; past the last tile the
     // workgroup moves to the next queue, and after eight empty queues in a row there is nothing left
     const TileTables tt = kernarg_now<TileTables>(offsetof(FwdParams<E>, t));
-    const int j = __builtin_amdgcn_readfirstlane(*reinterpret_cast<const int*>(smem + kFwdIdSlot));
+    const int j = __builtin_amdgcn_readfirstlane(*reinterpret_cast<const int*>(smem + kFwdIdSlot + 4 * id_word));
+    id_word ^= 1;
     const int64_t id = ((int64_t)(j / kQueueRun) * 8 + queue) * kQueueRun + (j % kQueueRun);
     if (id < (int64_t)tt.hist_bound + tt.self_total) {
       id3 = (int)id;

@@ -149,6 +149,15 @@ def make_plan(cu_seqlens, chunk_size: int, moba_topk: int, device=None, host_len
     if not torch.is_tensor(cu_seqlens):
         return _build(np.asarray(list(cu_seqlens), dtype=np.int64), chunk_size, moba_topk, device)
     device = cu_seqlens.device if device is None else device
+    # An inference tensor (made under torch.inference_mode()) has no version counter, so an in-place update
+    # could not be noticed: such a tensor is never remembered by identity.  It costs one small device-to-host
+    # read per call unless the caller supplies host_lengths (the transformers adapter does).
+    if cu_seqlens.is_inference():
+        if host_lengths is not None:
+            cu = np.asarray(list(host_lengths), dtype=np.int64)
+        else:
+            cu = cu_seqlens.detach().to("cpu", torch.int64).numpy()
+        return _build(cu, chunk_size, moba_topk, device)
     tkey = (id(cu_seqlens), cu_seqlens._version, str(device), int(chunk_size), int(moba_topk))
     hit = _BY_TENSOR.get(tkey)
     if hit is not None and hit[1] is cu_seqlens:

@@ -149,6 +149,63 @@ def test_grouped_query(batch, seqlen, heads, kv_heads, B, topk, dtype):
         moba_attn_varlen(qa, ka, va, cu_t, mx, B, topk)       # the 7-argument operator keeps the reference's contract
 
 
+@pytest.mark.parametrize("batch,seqlen,heads,kv_heads,B,topk,dtype", [
+    (1, 1024, 4, 1, 128, 3, torch.bfloat16),
+    (3, 2048, 8, 2, 256, 3, torch.bfloat16),
+    (2, 1500, 6, 3, 100, 4, torch.float16),
+    (4, 2048, 8, 2, 128, 2, torch.float16),
+    (1, 2048, 4, 2, 128, 1, torch.bfloat16),     # fallback: full causal attention
+])
+def test_grouped_query_vs_oracle(batch, seqlen, heads, kv_heads, B, topk, dtype):
+    """The grouped-query operator against the oracle run on key/value heads expanded with repeat_interleave
+    (the reference's semantics, moba/wrapper.py:59-61): out and dq as they are, dk and dv against the
+    oracle's gradients summed over the query heads of each group."""
+    from moba_amd import moba_attn_varlen_gqa
+    from moba_amd import moba_efficient as E
+    from moba_amd.plan import make_plan
+    rep = heads // kv_heads
+    q, _, _, do, cu, mx = make_case(batch, seqlen, heads, seed=5, dtype=dtype)
+    _, k, v, _, _, _ = make_case(batch, seqlen, kv_heads, seed=6, dtype=dtype)
+    cu_t = torch.tensor(cu, dtype=torch.int32, device="cuda")
+    qg, kg, vg = (x.cuda().requires_grad_(True) for x in (q, k, v))
+    out = moba_attn_varlen_gqa(qg, kg, vg, cu_t, mx, B, topk)
+    out.backward(do.cuda())
+    plan = make_plan(cu_t, B, topk)
+    sel = None
+    if not plan.fallback:
+        sel = E.gate_topk(qg.detach(), E.chunk_mean(kg.detach(), plan), plan).cpu()
+        # the selection itself: the oracle's on the expanded heads, up to near-ties of the fp32 scores
+        kx = torch.repeat_interleave(k, rep, dim=1)
+        want = O.select_topk(O.gate_scores(q, O.chunk_mean(kx, cu, B), cu, B), plan.K)
+        got = torch.sort(torch.where(sel < 0, torch.full_like(sel, 1 << 30), sel), dim=-1).values
+        got = torch.where(got == 1 << 30, torch.full_like(got, -1), got)
+        assert (got != want).any(dim=-1).float().mean() < 1e-3
+    qc = q.clone().requires_grad_(True)
+    kc, vc = (x.clone().requires_grad_(True) for x in (k, v))
+    ref = O.moba_attn_varlen_oracle(qc, torch.repeat_interleave(kc, rep, dim=1), torch.repeat_interleave(vc, rep, dim=1),
+                                    cu, mx, B, topk, sel=sel)
+    ref.backward(do.float())       # autograd of repeat_interleave sums each group's gradients into kc, vc
+    err = (out.detach().cpu().float() - ref.detach()).abs()
+    assert err.max() < MAX_ABS and err.mean() < MEAN_ABS, ("out", err.max().item(), err.mean().item())
+    for name, got_g, want_g in (("dq", qg.grad, qc.grad), ("dk", kg.grad, kc.grad), ("dv", vg.grad, vc.grad)):
+        assert got_g.shape == want_g.shape
+        e = (got_g.cpu().float() - want_g.float()).abs()
+        scale = want_g.abs().max().clamp_min(1.0)
+        assert e.max() < MAX_ABS * scale and e.mean() < MEAN_ABS * rep, (name, e.max().item(), e.mean().item(), scale.item())
+
+
+def test_baseline_config_1():
+    """One sequence of 4096 tokens, 4 heads, chunk 512, top-k 3, bf16 N(0,1) from a seed: forward against
+    the dense oracle (the configuration the reference's naive path runs on a CPU)."""
+    run_case(1, 4096, 4, 512, 3, seed=0, check_grad=False)
+
+
+def test_baseline_config_2():
+    """The reference's own speed-test shape (tests/test_moba_speedup.py:84, README.md:62): one sequence of
+    32768 tokens, 1 head, chunk 2048, top-k 3; forward and backward with dO ~ N(0,1) against the dense oracle."""
+    run_case(1, 32768, 1, 2048, 3, seed=0, check_grad=True)
+
+
 @pytest.mark.parametrize("seed", range(4))
 def test_random_shapes(seed):
     """Seeded random shapes: odd sequence lengths, chunk sizes that divide nothing, one to many

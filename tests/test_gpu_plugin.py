@@ -113,3 +113,46 @@ def test_narrow_head_model_prefill_and_generate():
     err = (got - ref).abs()
     assert err.max() < 6e-2 and err.mean() < 4e-3, (err.max().item(), err.mean().item())
     assert out.shape == (1, 303)
+
+
+def test_full_attention_layers_through_the_hip_operator():
+    """Layer-wise hybrid: layers named in full_attention_layers run the HIP operator with one chunk per
+    sequence (plain causal attention), the others keep MoBA.  With both layers full the model must reproduce
+    eager attention; with one of them full it must agree with the dense "moba_naive" plugin under the same
+    configuration, and differ from the all-MoBA run (the switch really changes a layer)."""
+    from moba_amd import MoBAConfig, register_moba
+    model = _model(torch.bfloat16)
+    ids = torch.randint(0, 128, (2, 1024), device="cuda")
+    import moba_amd.moba_efficient as E
+    chunk_sizes, real = [], E.moba_attn_varlen_with_lse
+
+    def spying(q, k, v, cu_seqlens, max_seqlen, moba_chunk_size, moba_topk, **kw):
+        chunk_sizes.append(moba_chunk_size)
+        return real(q, k, v, cu_seqlens, max_seqlen, moba_chunk_size, moba_topk, **kw)
+
+    E.moba_attn_varlen_with_lse = spying
+    try:
+        with torch.no_grad():
+            model.config._attn_implementation = "eager"
+            eager = model(ids).logits.float()
+            register_moba(MoBAConfig(moba_chunk_size=128, moba_topk=3, full_attention_layers=(0, 1)))
+            model.config._attn_implementation = "moba"
+            both_full = model(ids).logits.float()
+            assert chunk_sizes == [1024, 1024]
+            register_moba(MoBAConfig(moba_chunk_size=128, moba_topk=3, full_attention_layers=(-1,)))
+            del chunk_sizes[:]
+            last_full = model(ids).logits.float()
+            assert chunk_sizes == [128, 1024]
+            model.config._attn_implementation = "moba_naive"
+            last_full_naive = model(ids).logits.float()
+            register_moba(MoBAConfig(moba_chunk_size=128, moba_topk=3))
+            model.config._attn_implementation = "moba"
+            none_full = model(ids).logits.float()
+    finally:
+        E.moba_attn_varlen_with_lse = real
+        register_moba(MoBAConfig(moba_chunk_size=128, moba_topk=3))
+    err = (both_full - eager).abs()
+    assert err.max() < 6e-2 and err.mean() < 4e-3, (err.max().item(), err.mean().item())
+    err = (last_full - last_full_naive).abs()
+    assert err.median() < 4e-3 and err.mean() < 8e-3, (err.median().item(), err.mean().item())
+    assert (last_full - none_full).abs().max() > 1e-2

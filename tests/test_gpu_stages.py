@@ -173,3 +173,40 @@ def test_merge_of_random_partials(K, dtype):
     want, want_lse = O.merge_partials(part_o.float().view(S * H, K1, 128).permute(1, 0, 2), lses.t())
     assert (out.float().cpu().view(S * H, 128) - want).abs().max() < 2e-2
     assert (lse.cpu().view(-1) - want_lse).abs().max() < 1e-3
+
+
+# ------------------------------------------------------------------ the one-call attention entry point
+@pytest.mark.parametrize("batch,seqlen,heads,B,topk,dtype", [(3, 3000, 3, 100, 3, torch.bfloat16),
+                                                              (2, 4096, 2, 256, 4, torch.float16),
+                                                              (1, 2048, 2, 128, 1, torch.bfloat16)])
+def test_moba_fwd_entry_point(batch, seqlen, heads, B, topk, dtype):
+    """moba_fwd (partial attentions + merge behind one call): bit for bit what moba_fwd_partials followed by
+    moba_fwd_merge give, and within the tolerances of the oracle run on the same selection."""
+    from moba_amd import _lib
+    from moba_amd import moba_efficient as E
+    _note("moba_fwd", batch, seqlen, heads, B, topk, dtype)
+    q, k, v, _, cu, mx = make_case(batch, seqlen, heads, seed=9, dtype=dtype)
+    plan = _plan(cu, B, topk)
+    qg, kg, vg = q.cuda(), k.cuda(), v.cuda()
+    want_out, want_lse, sel, seg_off, tile_off, seg_dest, tile_seg = E._forward(qg, kg, vg, plan)
+    lib = _lib.load()
+    S, H, D = q.shape
+    K, t, dev = plan.K, plan.tables, qg.device
+    part_o = torch.empty((S * H * (K + 1), D), dtype=dtype, device=dev)
+    part_lse = torch.empty((S * H * (K + 1),), dtype=torch.float32, device=dev)
+    out = torch.zeros((S, H, D), dtype=dtype, device=dev)
+    lse = torch.zeros((S, H), dtype=torch.float32, device=dev)
+    queues = torch.empty(8, dtype=torch.int32, device=dev)
+    p = E._ptr
+    _lib.check(lib.moba_fwd(p(qg), p(kg), p(vg), p(part_o), p(part_lse), p(sel), p(seg_off), p(tile_off), p(seg_dest),
+                            p(t.get("fchunk_tok")), p(t["chunk_tok"]), p(t["self_tile_prefix"]), p(tile_seg),
+                            p(t["self_tile_chunk"]), p(out), p(lse), S, H, H, D, K, plan.F, plan.N, plan.chunk_size,
+                            plan.hist_tile_bound(H), plan.self_tiles, None, p(queues), 0.0, E._dtype_code(qg),
+                            E._stream(dev)), "moba_fwd")
+    torch.cuda.synchronize()
+    assert torch.equal(out, want_out) and torch.equal(lse, want_lse)
+    ref, ref_lse, _ = O.moba_attn_varlen_oracle(q, k, v, cu, mx, B, topk, sel=None if sel is None else sel.cpu(),
+                                                return_aux=True)
+    err = (out.cpu().float() - ref).abs()
+    assert err.max() < 2e-2 and err.mean() < 2e-3, (err.max().item(), err.mean().item())
+    assert (lse.cpu() - ref_lse).abs().max() < 2e-3

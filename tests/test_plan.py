@@ -72,3 +72,18 @@ def test_plan_cache_follows_the_tensor_contents():
     assert c.cu == [0, 7, 9]
     # different chunk size or top-k: different plan
     assert make_plan(cu, 16, 3) is not b and make_plan(cu, 32, 2) is not b
+
+
+def test_plan_accepts_inference_tensors():
+    """A cu_seqlens made under torch.inference_mode() has no version counter: it is planned by value on
+    every call (never remembered by identity), so an in-place update inside that mode is seen too."""
+    import torch
+    with torch.inference_mode():
+        cu = torch.tensor([0, 100, 260], dtype=torch.int32)
+        assert cu.is_inference()
+        a = make_plan(cu, 32, 3)
+        assert a.cu == [0, 100, 260] and make_plan(cu, 32, 3) is a
+        cu[1] = 120
+        assert make_plan(cu, 32, 3).cu == [0, 120, 260]
+        assert make_plan(cu, 32, 3, host_lengths=[0, 120, 260]).cu == [0, 120, 260]
+    assert make_plan(cu, 32, 3).cu == [0, 120, 260]      # and outside the mode as well

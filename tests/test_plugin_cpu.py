@@ -110,6 +110,32 @@ def test_moba_layer_hands_grouped_heads_to_an_impl_that_takes_them():
     assert seen["k"].shape == (b * s, hkv, d) and torch.equal(seen["k"][1 * s + 2, 1], key[1, 1, 2])
 
 
+def test_moba_layer_prefill_under_inference_mode():
+    """Under torch.inference_mode() the adapter's cu_seqlens is an inference tensor; an operator that plans
+    from host lengths (as the HIP operator does) must get through make_plan with it."""
+    from moba_amd import MoBAConfig
+    from moba_amd.plan import make_plan
+    from moba_amd.wrapper import moba_layer
+
+    seen = {}
+
+    def impl(q, k, v, cu_seqlens, max_seqlen, moba_chunk_size, moba_topk):
+        seen["plan"] = make_plan(cu_seqlens, moba_chunk_size, moba_topk, device="cpu")
+        seen["inference"] = cu_seqlens.is_inference()
+        return q
+
+    impl.takes_host_lengths = True
+
+    class Mod(torch.nn.Module):
+        is_causal = True
+
+    b, h, s, d = 2, 2, 7, 8     # a shape no other test uses: the adapter makes a fresh cu_seqlens for it
+    with torch.inference_mode():
+        x = torch.randn(b, h, s, d)
+        out, _ = moba_layer(impl, MoBAConfig(4, 3), Mod(), x, x, x, None)
+    assert seen["inference"] and seen["plan"].cu == [0, 7, 14] and out.shape == (b * s, h, d)
+
+
 def test_full_attention_layers_switch():
     """Layers named in full_attention_layers get one chunk per sequence (= causal attention in every
     implementation); the others keep the configured chunk size.  Negative indices count from the end."""
