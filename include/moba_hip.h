@@ -39,7 +39,7 @@ extern "C" {
 
 enum { MOBA_DTYPE_BF16 = 0, MOBA_DTYPE_F16 = 1 };
 
-#define MOBA_ABI_VERSION 101 /* the signatures below; moba_version() returns the number the library was built with */
+#define MOBA_ABI_VERSION 102 /* the signatures below; moba_version() returns the number the library was built with */
 int moba_version(void);
 const char* moba_strerror(int code);
 
@@ -52,6 +52,18 @@ const char* moba_strerror(int code);
 size_t moba_chunk_mean_workspace_bytes(int H, int D, int F, int B);
 int moba_chunk_mean(const void* k, const int32_t* fchunk_tok, void* kbar, void* workspace, int64_t S, int H, int D,
                     int F, int B, const int64_t* strides, int dtype, void* stream);
+
+/* moba_chunk_mean for callers that cannot allocate or bring a workspace (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and
+ * bit for bit the same kbar as moba_chunk_mean (the sums are exact in fp64 whatever the token split), but
+ * the partial sums live in a fixed array inside the library, moba_chunk_mean_static_capacity() bytes (32 MiB)
+ * per GPU, held until the process ends.  The call allocates and frees nothing.  Limit: F * H * D * 8 bytes
+ * must fit the array (MOBA_ERR_LIMIT otherwise; F * H <= 32768 at D = 128).  All calls on one GPU share the
+ * array: calls that overlap in time on one GPU (two streams) race.  The first call on a GPU looks the
+ * array's address up (hipGetSymbolAddress); make that call outside any stream capture. */
+size_t moba_chunk_mean_static_capacity(void);
+int moba_chunk_mean_static(const void* k, const int32_t* fchunk_tok, void* kbar, int64_t S, int H, int D, int F, int B,
+                           const int64_t* strides, int dtype, void* stream);
 
 /* Gate scores + causal top-k.  Replaces moba/moba_efficient.py:341-371 (fp32 einsum,
  * -inf mask, torch.topk, dropping -inf picks).

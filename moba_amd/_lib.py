@@ -24,6 +24,9 @@ _SIGNATURES = {
     "moba_chunk_mean_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "moba_chunk_mean": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_strides,
                                 c_int, c_void_p]),
+    "moba_chunk_mean_static_capacity": (c_size_t, []),
+    "moba_chunk_mean_static": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_strides,
+                                       c_int, c_void_p]),
     "moba_gate_topk": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_strides, c_int, c_void_p]),
     "moba_topk_from_scores": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_void_p]),
@@ -40,7 +43,7 @@ _SIGNATURES = {
     "moba_decode": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_int64] * 4 + [c_float, c_int, c_void_p]),
 }
 OPTIONAL = set()
-ABI_VERSION = 101  # MOBA_ABI_VERSION of include/moba_hip.h, the signatures above
+ABI_VERSION = 102  # MOBA_ABI_VERSION of include/moba_hip.h, the signatures above
 DTYPE_BF16, DTYPE_F16 = 0, 1
 
 

@@ -10,6 +10,7 @@
 // Stage 1: grid (F, token splits, column blocks); each thread owns 8 adjacent
 //          columns of the [H*D] token row and sums its token split.
 // Stage 2: sums the splits in order, divides by B, rounds.
+#include <mutex>
 #include "common.h"
 
 namespace moba {
@@ -98,34 +99,91 @@ extern "C" size_t moba_chunk_mean_workspace_bytes(int H, int D, int F, int B) {
   return (size_t)F * pick_nsplit(HD8, F, B) * HD8 * 8 * sizeof(double);
 }
 
-extern "C" int moba_chunk_mean(const void* k, const int32_t* fchunk_tok, void* kbar, void* workspace,
-                               int64_t S, int H, int D, int F, int B, const int64_t* strides, int dtype,
-                               void* stream) {
-  if (F == 0) return MOBA_OK;
-  if (dtype != MOBA_DTYPE_BF16 && dtype != MOBA_DTYPE_F16) return MOBA_ERR_UNSUPPORTED;
-  if (!k || !fchunk_tok || !kbar || !workspace || S <= 0 || H <= 0 || D <= 0 || F < 0 || B <= 0) return MOBA_ERR_ARG;
-  if ((H * D) % 8 != 0 || ((uintptr_t)k & 15) || ((uintptr_t)kbar & 15) || ((uintptr_t)workspace & 7)) return MOBA_ERR_ARG;
-  if (D % 8 != 0) return MOBA_ERR_ARG;
-  // strides (elements): {., ., k token, k head}; null = packed [S, H, D]
-  const int64_t kts = strides ? strides[2] : (int64_t)H * D, khs = strides ? strides[3] : D;
-  if (kts <= 0 || khs <= 0 || (kts & 7) || (khs & 7)) return MOBA_ERR_ARG;
+static int launch_chunk_mean(const void* k, const int32_t* fchunk_tok, void* kbar, double* partial, int H, int D,
+                             int F, int B, int nsplit, int64_t kts, int64_t khs, int dtype, hipStream_t st) {
   const int HD8 = H * D / 8;
-  const int nsplit = pick_nsplit(HD8, F, B);
   const int tps = (B + nsplit - 1) / nsplit;
-  hipStream_t st = (hipStream_t)stream;
   dim3 grid(F, nsplit, (HD8 + 255) / 256);
   const int64_t n = (int64_t)F * HD8;
   const dim3 fgrid((unsigned)((n + 255) / 256));
   if (dtype == MOBA_DTYPE_F16) {
-    hipLaunchKernelGGL(chunk_mean_partial_kernel<F16>, grid, dim3(256), 0, st, (const f16*)k, fchunk_tok,
-                       (double*)workspace, HD8, D / 8, B, nsplit, tps, kts, khs);
-    hipLaunchKernelGGL(chunk_mean_finish_kernel<F16>, fgrid, dim3(256), 0, st, (const double*)workspace, (f16*)kbar,
+    hipLaunchKernelGGL(chunk_mean_partial_kernel<F16>, grid, dim3(256), 0, st, (const f16*)k, fchunk_tok, partial,
+                       HD8, D / 8, B, nsplit, tps, kts, khs);
+    hipLaunchKernelGGL(chunk_mean_finish_kernel<F16>, fgrid, dim3(256), 0, st, (const double*)partial, (f16*)kbar,
                        HD8, B, nsplit, F);
   } else {
-    hipLaunchKernelGGL(chunk_mean_partial_kernel<Bf16>, grid, dim3(256), 0, st, (const bf16*)k, fchunk_tok,
-                       (double*)workspace, HD8, D / 8, B, nsplit, tps, kts, khs);
-    hipLaunchKernelGGL(chunk_mean_finish_kernel<Bf16>, fgrid, dim3(256), 0, st, (const double*)workspace,
-                       (bf16*)kbar, HD8, B, nsplit, F);
+    hipLaunchKernelGGL(chunk_mean_partial_kernel<Bf16>, grid, dim3(256), 0, st, (const bf16*)k, fchunk_tok, partial,
+                       HD8, D / 8, B, nsplit, tps, kts, khs);
+    hipLaunchKernelGGL(chunk_mean_finish_kernel<Bf16>, fgrid, dim3(256), 0, st, (const double*)partial, (bf16*)kbar,
+                       HD8, B, nsplit, F);
   }
   return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
+}
+
+// argument checks shared by the two entry points; kts, khs receive the key token and head strides (elements)
+static int check_chunk_mean_args(const void* k, const int32_t* fchunk_tok, void* kbar, int64_t S, int H, int D, int F,
+                                 int B, const int64_t* strides, int dtype, int64_t& kts, int64_t& khs) {
+  if (dtype != MOBA_DTYPE_BF16 && dtype != MOBA_DTYPE_F16) return MOBA_ERR_UNSUPPORTED;
+  if (!k || !fchunk_tok || !kbar || S <= 0 || H <= 0 || D <= 0 || F < 0 || B <= 0) return MOBA_ERR_ARG;
+  if ((H * D) % 8 != 0 || ((uintptr_t)k & 15) || ((uintptr_t)kbar & 15)) return MOBA_ERR_ARG;
+  if (D % 8 != 0) return MOBA_ERR_ARG;
+  // strides (elements): {., ., k token, k head}; null = packed [S, H, D]
+  kts = strides ? strides[2] : (int64_t)H * D;
+  khs = strides ? strides[3] : D;
+  if (kts <= 0 || khs <= 0 || (kts & 7) || (khs & 7)) return MOBA_ERR_ARG;
+  return MOBA_OK;
+}
+
+extern "C" int moba_chunk_mean(const void* k, const int32_t* fchunk_tok, void* kbar, void* workspace,
+                               int64_t S, int H, int D, int F, int B, const int64_t* strides, int dtype,
+                               void* stream) {
+  if (F == 0) return MOBA_OK;
+  int64_t kts = 0, khs = 0;
+  const int rc = check_chunk_mean_args(k, fchunk_tok, kbar, S, H, D, F, B, strides, dtype, kts, khs);
+  if (rc != MOBA_OK) return rc;
+  if (!workspace || ((uintptr_t)workspace & 7)) return MOBA_ERR_ARG;
+  return launch_chunk_mean(k, fchunk_tok, kbar, (double*)workspace, H, D, F, B, pick_nsplit(H * D / 8, F, B), kts, khs,
+                           dtype, (hipStream_t)stream);
+}
+
+// ---- the same stage for callers that cannot allocate: the partial sums live in a fixed array of the library ----
+// Every GPU the library runs on holds its own copy of this array, at its own address, until the process
+// ends.  The name below is a host-side stand-in, not a device address: host code only ever uses the
+// address that hipGetSymbolAddress returned for the current device.
+constexpr size_t kStaticPartialBytes = (size_t)32 << 20;
+static __device__ __align__(256) double scratch[kStaticPartialBytes / sizeof(double)];
+
+static std::mutex scratch_lock;
+static double* scratch_of_device[kMaxDevices];   // guarded by scratch_lock
+
+// device address of `scratch` on the current device (null on error), asked once per device
+static double* static_partials() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0) return nullptr;
+  std::lock_guard<std::mutex> hold(scratch_lock);
+  if (dev < kMaxDevices && scratch_of_device[dev]) return scratch_of_device[dev];
+  double* ptr = nullptr;
+  if (hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return nullptr;
+  if (dev < kMaxDevices) scratch_of_device[dev] = ptr;
+  return ptr;
+}
+
+extern "C" size_t moba_chunk_mean_static_capacity(void) { return kStaticPartialBytes; }
+
+extern "C" int moba_chunk_mean_static(const void* k, const int32_t* fchunk_tok, void* kbar, int64_t S, int H, int D,
+                                      int F, int B, const int64_t* strides, int dtype, void* stream) {
+  if (F == 0) return MOBA_OK;
+  int64_t kts = 0, khs = 0;
+  const int rc = check_chunk_mean_args(k, fchunk_tok, kbar, S, H, D, F, B, strides, dtype, kts, khs);
+  if (rc != MOBA_OK) return rc;
+  // The sums are exact in fp64, so the mean does not depend on the number of token splits: take the
+  // widest split (up to the one moba_chunk_mean would use) whose partial sums fit the array.
+  const int HD8 = H * D / 8;
+  const size_t per_split = (size_t)F * HD8 * 8 * sizeof(double);
+  if (per_split > kStaticPartialBytes) return MOBA_ERR_LIMIT;   // F * H * D * 8 bytes exceed the array
+  int nsplit = pick_nsplit(HD8, F, B);
+  while (nsplit > 1 && per_split * nsplit > kStaticPartialBytes) nsplit /= 2;
+  double* partial = static_partials();
+  if (!partial) return MOBA_ERR_LAUNCH;
+  return launch_chunk_mean(k, fchunk_tok, kbar, partial, H, D, F, B, nsplit, kts, khs, dtype, (hipStream_t)stream);
 }
