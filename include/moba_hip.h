@@ -39,7 +39,7 @@ extern "C" {
 
 enum { MOBA_DTYPE_BF16 = 0, MOBA_DTYPE_F16 = 1 };
 
-#define MOBA_ABI_VERSION 102 /* the signatures below; moba_version() returns the number the library was built with */
+#define MOBA_ABI_VERSION 103 /* the signatures below; moba_version() returns the number the library was built with */
 int moba_version(void);
 const char* moba_strerror(int code);
 
@@ -110,6 +110,12 @@ int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, const int32_t
  *   queues [8] int32 scratch: the tile counters of the forward kernel, whose workgroups (two per CU) stay
  *              resident and draw tiles from one queue per XCD; the call zeroes them with a kernel of its own.
  *              Calls that overlap in time need their own eight counters each.
+ *   redo   [1 + hist_bound + self_tiles * H] int32 scratch, or NULL.  With it, bf16 problems large enough for the
+ *              resident-workgroup kernel take each tile's softmax relative to one fixed reference per row (the row
+ *              maximum of the tile's first 32 keys) instead of a running maximum; a tile in which a row's scores rise
+ *              more than 96 powers of two above that reference is entered in this list and computed again by the
+ *              kernel that tracks the maximum (redo[0] = number of such tiles after the call, normally 0).  The result
+ *              is within rounding of the other path's either way.  NULL, fp16 and small problems: running maximum only.
  *   softmax_scale: the factor on q k^T; 0 (or less) stands for D^-0.5, the reference's only choice
  *              (moba/moba_efficient.py:86).  A caller whose heads are narrower than D pads them with zeros
  *              and passes its own head_dim^-0.5. */
@@ -119,7 +125,7 @@ int moba_fwd_partials(const void* q, const void* k, const void* v, void* part_o,
                       const int32_t* fchunk_tok, const int32_t* chunk_tok, const int32_t* self_tile_prefix,
                       const int32_t* tile_seg, const int32_t* self_tile_chunk, int64_t S, int H, int Hkv, int D, int K,
                       int F, int N, int B, int64_t hist_bound, int64_t self_tiles, const int64_t* strides,
-                      int32_t* queues, float softmax_scale, int dtype, void* stream);
+                      int32_t* queues, int32_t* redo, float softmax_scale, int dtype, void* stream);
 int moba_fwd_merge(const void* part_o, const float* part_lse, const int32_t* sel, void* out, float* lse, int64_t S,
                    int H, int D, int K, int dtype, void* stream);
 int moba_fwd(const void* q, const void* k, const void* v, void* part_o, float* part_lse, const int32_t* sel,
@@ -127,7 +133,7 @@ int moba_fwd(const void* q, const void* k, const void* v, void* part_o, float* p
              const int32_t* chunk_tok, const int32_t* self_tile_prefix, const int32_t* tile_seg,
              const int32_t* self_tile_chunk, void* out, float* lse, int64_t S, int H, int Hkv, int D, int K, int F,
              int N, int B, int64_t hist_bound, int64_t self_tiles, const int64_t* strides, int32_t* queues,
-             float softmax_scale, int dtype, void* stream);
+             int32_t* redo, float softmax_scale, int dtype, void* stream);
 
 /* Backward.  Replaces MixedAttention.backward, moba/moba_efficient.py:185-267, and the
  * autograd scatter of its gathered gradients.  Deterministic (no floating-point atomics).

@@ -33,17 +33,17 @@ _SIGNATURES = {
     "moba_build_lists": (c_int, [c_void_p] * 10 + [c_int64] + [c_int] * 7 + [c_int64, c_void_p]),
     "moba_fwd_tile_rows": (c_int, []),
     "moba_fwd_partials": (c_int, [c_void_p] * 13 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int64,
-                                                   c_int64, c_strides, c_void_p, c_float, c_int, c_void_p]),
+                                                   c_int64, c_strides, c_void_p, c_void_p, c_float, c_int, c_void_p]),
     "moba_fwd_merge": (c_int, [c_void_p] * 5 + [c_int64, c_int, c_int, c_int, c_int, c_void_p]),
     "moba_fwd": (c_int, [c_void_p] * 16 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_int64,
-                                          c_strides, c_void_p, c_float, c_int, c_void_p]),
+                                          c_strides, c_void_p, c_void_p, c_float, c_int, c_void_p]),
     "moba_bwd": (c_int, [c_void_p] * 21 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_int64,
                                           c_strides, c_void_p, c_float, c_int, c_void_p]),
     "moba_decode_splits": (c_int, [c_int, c_int, c_int]),
     "moba_decode": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_int64] * 4 + [c_float, c_int, c_void_p]),
 }
 OPTIONAL = set()
-ABI_VERSION = 102  # MOBA_ABI_VERSION of include/moba_hip.h, the signatures above
+ABI_VERSION = 103  # MOBA_ABI_VERSION of include/moba_hip.h, the signatures above
 DTYPE_BF16, DTYPE_F16 = 0, 1
 
 

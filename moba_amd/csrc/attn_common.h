@@ -54,6 +54,7 @@ inline bool set_layout(TileTables& t, const int64_t* strides) {
 
 // One tile of up to TM query rows of one head, as seen by a lane.
 struct Tile {
+  int id;         // logical tile id
   int h;          // head
   int kv_tok0;    // token of key 0
   int nkeys;      // keys the tile attends (before masking)
@@ -68,7 +69,11 @@ struct Tile {
 
 // the tile counters of a kernel whose resident workgroups draw their tiles from per-XCD queues start at zero
 // (a kernel, not a memset: safe to record into a graph)
-static __global__ void zero_queues_kernel(int* queues) { queues[threadIdx.x] = 0; }
+// (`also`, if not null, is one more counter to clear)
+static __global__ void zero_queues_kernel(int* queues, int* also) {
+  queues[threadIdx.x] = 0;
+  if (also && threadIdx.x == 0) *also = 0;
+}
 
 // Workgroup ids are dealt round-robin to the 8 XCDs; give each XCD runs of kXcdBlock
 // consecutive logical tiles so that tiles sharing a K/V chunk share an L2.
@@ -94,6 +99,7 @@ __device__ __forceinline__ int decode_tile_code(const TileTables& p, int logical
 // Returns false (and row_count = 0) for a code that is not a tile.
 __device__ __forceinline__ bool decode_tile_head(const TileTables& p, int logical, int code, Tile& t) {
   const int H = p.H;
+  t.id = logical;
   t.row_count = 0;
   t.base = -1;
   if (code < 0) return false;
@@ -188,6 +194,24 @@ template <class V4>
 __device__ __forceinline__ V4 lds_read_tr(const char* p) {
   V4 r;
   lds_read_tr(p, r);
+  return r;
+}
+// the same reads at an LDS byte address held as a number
+template <class T>
+__device__ __forceinline__ __attribute__((address_space(3))) T* lds_ptr(uint32_t addr) {
+  return (__attribute__((address_space(3))) T*)(uintptr_t)addr;
+}
+__device__ __forceinline__ void lds_read_tr(uint32_t addr, bf16x4& out) {
+  out = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(lds_ptr<bf16x4>(addr));
+}
+__device__ __forceinline__ void lds_read_tr(uint32_t addr, f16x4& out) {
+  typedef __attribute__((ext_vector_type(4))) short i16x4;
+  out = __builtin_bit_cast(f16x4, __builtin_amdgcn_ds_read_tr16_b64_v4i16(lds_ptr<i16x4>(addr)));
+}
+template <class V4>
+__device__ __forceinline__ V4 lds_read_tr(uint32_t addr) {
+  V4 r;
+  lds_read_tr(addr, r);
   return r;
 }
 

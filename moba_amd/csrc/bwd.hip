@@ -752,7 +752,7 @@ static int launch_bwd(const void* dout, const void* q, const void* k, const void
   const int64_t rows = S * H;
   hipLaunchKernelGGL(bwd_delta_kernel<E>, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st, (const elem*)dout,
                      (const elem*)out, lse, delta, delta + S * H, rows);
-  hipLaunchKernelGGL(zero_queues_kernel, dim3(1), dim3(16), 0, st, queues);  // a kernel, not a memset: graph safe
+  hipLaunchKernelGGL(zero_queues_kernel, dim3(1), dim3(16), 0, st, queues, (int*)nullptr);  // a kernel, not a memset: graph safe
   hipLaunchKernelGGL(bwd_dq_kernel<E>, dim3((unsigned)grid_q), dim3(256), kBwdDqLds, st, p);
   hipLaunchKernelGGL(bwd_dq_reduce_kernel<E>, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st,
                      (const elem*)part_dq, sel, (elem*)dq, rows, K + 1);

@@ -24,6 +24,7 @@ namespace moba {
 // LDS: K[2], V[2] stages, then 256 bytes per wave for the gather-list entries of the next tile's rows,
 // then the slot through which wave 0 hands the tile id it drew to the other waves
 constexpr int kFwdEntries = 4 * kTileBytes, kFwdIdSlot = kFwdEntries + 4 * 256;
+constexpr int kFwdRedoWord = kFwdIdSlot + 8;  // set by a wave whose rows left the range of the fixed-reference softmax
 constexpr int kFwdLds = kFwdIdSlot + 16;
 
 template <class E>
@@ -36,9 +37,21 @@ struct FwdParams {
   TileTables t;
   float scale_log2;  // D^-0.5 * log2(e)
   int* queues;       // [8] tile counters, one per XCD, zero when the kernel starts
+  int* redo;         // [1 + tiles] count and ids of the tiles to be computed again (see kFixedRef); count zero at the start
 };
 
 constexpr float kRescaleThreshold = 8.f;  // log2 units: the running max may lag the true max by this much
+// Fixed-reference softmax: a row's sum of exponentials (relative to the row maximum of the tile's first key
+// block) at or beyond this, or not a number, sends the tile to the kernel that tracks the maximum.  Below it
+// every probability is a finite bf16 and the accumulators stay finite for |v| < 2^31.
+constexpr float kFixedRefMaxSum = 0x1p96f;
+
+// how a workgroup comes by its tiles
+enum : int {
+  kTilePerGroup = 0,  // one tile, the id from the workgroup id (small problems)
+  kTilesQueued = 1,   // resident workgroups drawing ids from the per-XCD queues
+  kTilesListed = 2,   // resident workgroups walking the list FwdParams::redo
+};
 
 // The loop is software pipelined by hand at the granularity of a 32-key block u:
 //     phase 1:  S^T(u+1)      8 MFMA   with   exponentials 8..15 of block u, packing of P(u)
@@ -46,12 +59,21 @@ constexpr float kRescaleThreshold = 8.f;  // log2 units: the running max may lag
 // so the vector work of one block executes under the MFMAs of its neighbours, and the
 // fragment reads from LDS run a few MFMAs ahead.  K and V tiles (64 keys) are double
 // buffered separately: K(t+1) must be resident half a tile before V(t+1).
-// kQueued: resident workgroups that draw tiles from the queues (large problems).  Otherwise one tile per
-// workgroup, the id from the workgroup id: with few tiles the queue protocol's start-up and wind-down
-// (three passes to fill the look-ahead, eight empty draws to know that nothing is left) would dominate.
-template <class E, bool kQueued>
+// kMode: resident workgroups that draw tiles from the queues (large problems), or one tile per workgroup,
+// the id from the workgroup id: with few tiles the queue protocol's start-up and wind-down (three passes
+// to fill the look-ahead, eight empty draws to know that nothing is left) would dominate.
+// kFixedRef (bf16, queued): the softmax of a tile is taken relative to one fixed reference per row, the row
+// maximum of the tile's first 32-key block, instead of a running maximum.  A bf16 probability has the
+// exponent range of fp32, so later scores may exceed the reference by almost 2^7 before anything overflows:
+// the per-block row maximum, its exchange between the lane halves, the comparison with the running maximum
+// and the rescale branch all go (22 of 88 vector instructions per key block).  A row whose sum leaves the
+// safe range -- scores that rise by more than 96 powers of two within one tile -- marks its tile in
+// FwdParams::redo, and the kTilesListed kernel, which tracks the maximum, computes those tiles again.
+template <class E, int kMode, bool kFixedRef>
 __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) {
   MOBA_ELEM_TYPES(E)
+  constexpr bool kQueued = kMode == kTilesQueued;
+  static_assert(!kFixedRef || (kQueued && std::is_same<E, Bf16>::value), "the fixed reference needs bf16's exponent range");
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int n = lane & 31, hh = lane >> 5;
@@ -139,33 +161,38 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
   int nkt = 1, rot = 0;
   auto key_tile = [&](int it) __attribute__((always_inline)) { const int x = it + rot; return x >= nkt ? x - nkt : x; };
 
-  // ---- fragment addressing: per-lane byte offsets inside a tile, everything else is an immediate ----
+  // ---- fragment addressing: per-lane LDS byte addresses inside a tile (numbers, not pointers into smem:
+  // the address of a read is then one register plus an immediate, with no base left to add) ----
   const int g16 = lane >> 4, i0 = (lane & 15) >> 2, i1 = lane & 3;
   // K row fragment (row 32*kb + n, 16-byte column 2*s8 + hh)
-  int koff[8];
+  uint32_t koff[8];
   {
     const int k_sw = ((n & 3) << 2) ^ ((n >> 2) & 3);
 #pragma unroll
-    for (int s8 = 0; s8 < 8; ++s8) koff[s8] = n * 256 + (((2 * s8 + hh) ^ k_sw) << 4);
+    for (int s8 = 0; s8 < 8; ++s8) koff[s8] = lds_base + n * 256 + (((2 * s8 + hh) ^ k_sw) << 4);
   }
   // V^T quads: rows 32*kb + 16*j2 + 4*hh + i0 (A) and +8 (B), 8 bytes at d = 32*db + 16*(g16&1) + 4*i1
-  int voffA[4], voffB[4];
+  uint32_t voffA[4], voffB[4];
   {
     const int v_c16 = 2 * (g16 & 1) + (i1 >> 1);
     const int v_sub = (i1 & 1) * 8;
 #pragma unroll
     for (int db = 0; db < 4; ++db) {
       const int c16 = 4 * db + v_c16;
-      voffA[db] = (4 * hh + i0) * 256 + ((c16 ^ (i0 << 2) ^ hh) << 4) + v_sub;
-      voffB[db] = (4 * hh + i0 + 8) * 256 + ((c16 ^ (i0 << 2) ^ (hh + 2)) << 4) + v_sub;
+      voffA[db] = lds_base + (4 * hh + i0) * 256 + ((c16 ^ (i0 << 2) ^ hh) << 4) + v_sub;
+      voffB[db] = lds_base + (4 * hh + i0 + 8) * 256 + ((c16 ^ (i0 << 2) ^ (hh + 2)) << 4) + v_sub;
+      // finished addresses, kept as they are: the compiler otherwise holds their summands and adds them
+      // again at every use (eight additions per key block)
+      asm volatile("" : "+v"(voffA[db]));
+      asm volatile("" : "+v"(voffB[db]));
     }
   }
   auto k_frag = [&](int tile_off, int kb, int s8) __attribute__((always_inline)) {
-    return *reinterpret_cast<const elem8*>(smem + koff[s8] + (tile_off + kb * 8192));
+    return *lds_ptr<const elem8>(koff[s8] + (uint32_t)(tile_off + kb * 8192));
   };
   auto v_frag = [&](int tile_off, int kb, int j2, int db) __attribute__((always_inline)) {
-    const elem4 va = lds_read_tr<elem4>(smem + voffA[db] + (tile_off + (32 * kb + 16 * j2) * 256));
-    const elem4 vb = lds_read_tr<elem4>(smem + voffB[db] + (tile_off + (32 * kb + 16 * j2) * 256));
+    const elem4 va = lds_read_tr<elem4>(voffA[db] + (uint32_t)(tile_off + (32 * kb + 16 * j2) * 256));
+    const elem4 vb = lds_read_tr<elem4>(voffB[db] + (uint32_t)(tile_off + (32 * kb + 16 * j2) * 256));
     elem8 a;
     a[0] = va[0]; a[1] = va[1]; a[2] = va[2]; a[3] = va[3];
     a[4] = vb[0]; a[5] = vb[1]; a[6] = vb[2]; a[7] = vb[3];
@@ -201,8 +228,12 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
   // barrier after the waves read the word, so wave 0 may already be writing the next pass's id -- into the
   // other word.  The word of pass i is rewritten in pass i + 2, behind the barrier of pass i + 1.
   int id_word = 0;
-  int dest_done = 0, rows_done = 0;
+  int dest_done = 0, rows_done = 0, id_done = 0;
   bool valid_done = false;
+  int list_pos = blockIdx.x;  // kTilesListed: position in the list of the next tile
+  if constexpr (kFixedRef) {
+    if (tid == 0) *reinterpret_cast<int*>(smem + kFwdRedoWord) = 0;  // first read many barriers from here
+  }
   while (true) {
   // ================= tile switch =================
   wait_vmem();  // nothing of this wave is in flight any more: the next tile's row entries are in LDS
@@ -217,6 +248,11 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
     const int en = ln & 31, ehh = ln >> 5;
     const float l_tot = sum_xhalf(l_run);
     const float inv = 1.f / l_tot;
+    if constexpr (kFixedRef) {
+      // compared as bit patterns: infinities, every NaN and negative values all read as "too large"
+      const bool bad = valid_done && __builtin_bit_cast(uint32_t, l_tot) >= __builtin_bit_cast(uint32_t, kFixedRefMaxSum);
+      if (__any(bad) && ln == 0) *reinterpret_cast<volatile int*>(smem + kFwdRedoWord) = 1;
+    }
     char* stage = smem + wave_u * 8192;
     char* wrow = stage + en * 256 + 8 * ehh;
 #pragma unroll
@@ -242,10 +278,19 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
     for (int db = 0; db < 4; ++db)
 #pragma unroll
       for (int e = 0; e < 16; ++e) oacc[db][e] = 0.f;
-    if constexpr (!kQueued) return;
+    if constexpr (kMode == kTilePerGroup) return;
     m_run = -INFINITY;
     l_run = 0.f;
     __syncthreads();  // the K stages take the next tile's copies only after every wave has read its rows back
+    if constexpr (kFixedRef) {
+      // one thread enters the tile in the list if any wave marked it (the word is next written by a later
+      // tile's epilogue, several barriers from here)
+      if (tid == 0 && *reinterpret_cast<volatile int*>(smem + kFwdRedoWord) != 0) {
+        *reinterpret_cast<volatile int*>(smem + kFwdRedoWord) = 0;
+        const int at = __hip_atomic_fetch_add(pn.redo, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        pn.redo[1 + at] = id_done;
+      }
+    }
   }
   int drawn = 0;  // wave 0, lane 0: the value of the queue's counter
   {
@@ -255,6 +300,11 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
     const int er = (tx >> 6) * 32 + (tx & 31);
     if constexpr (kQueued) {
       t = t1;  // the next tile becomes the current one: its rows' gather-list entries are in LDS by now
+    } else if constexpr (kMode == kTilesListed) {
+      if (list_pos >= pn.redo[0]) return;  // (uniform; the count is final: the kernel that wrote it has ended)
+      const int listed = pn.redo[1 + list_pos];
+      list_pos += gridDim.x;
+      if (!decode_tile_head(pn.t, listed, t)) return;  // (cannot happen: listed ids are tiles)
     } else {
       if (!decode_tile_head(pn.t, logical_tile_id(), t)) return;
     }
@@ -324,6 +374,7 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
   have_partial = t.row_count > 0;
   if (!have_partial) continue;
   dest_done = t.dest;
+  id_done = t.id;
   valid_done = row_valid;
   rows_done = t.row_count - wave_u * 32;  // rows of this wave that exist
 
@@ -338,7 +389,10 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
     float mx = s0[0];
 #pragma unroll
     for (int e = 1; e < 16; ++e) mx = fmaxf(mx, s0[e]);
-    update_max(max_xhalf(mx) * sl2);  // nothing accumulated yet: the factor is not needed
+    // the row maximum of the first block: where the running maximum starts, or the tile's fixed reference
+    // (every row has a key in this block: key 0 of a causal tile, any key of a history tile)
+    if constexpr (kFixedRef) m_run = max_xhalf(mx) * sl2;
+    else update_max(max_xhalf(mx) * sl2);  // nothing accumulated yet: the factor is not needed
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const float pe = fast_exp2(s0[e] * sl2 - m_run);
@@ -391,8 +445,38 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
     if constexpr (has_next) {
       if (masked) mask_block(sn, next_key0);
     }
-    float mx = -INFINITY, alpha = 1.f, rn = 0.f;
     float pg[8];
+    if constexpr (kFixedRef) {
+      // no row maximum: the eight exponentials spread over slots 1..7 (slot 0 is left to the packing above
+      // and to the last S^T MFMA's result), each sum one slot behind its exponential
+      float rn = 0.f;
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const int j2 = k >> 2, db = k & 3;
+        if (k + 4 < 8) va[k + 4] = v_frag(vs, kb, 1, db);
+        oacc[db] = mfma32(va[k], pb[j2], oacc[db]);
+        if constexpr (has_next) {
+          if (k == 1) {
+            pg[0] = fast_exp2(sn[0] * sl2 - m_run);
+            pg[1] = fast_exp2(sn[1] * sl2 - m_run);
+            MOBA_PIN(pg[0]);
+            MOBA_PIN(pg[1]);
+          } else if (k >= 2) {
+            pg[k] = fast_exp2(sn[k] * sl2 - m_run);
+            rn = (k == 2) ? pg[0] + pg[1] : rn + pg[k - 1];
+            MOBA_PIN(pg[k]);
+            MOBA_PIN(rn);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if constexpr (has_next) {
+        l_run += rn + pg[7];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) pb[0][e] = (elem)pg[e];
+      }
+    } else {
+    float mx = -INFINITY, alpha = 1.f, rn = 0.f;
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
       const int j2 = k >> 2, db = k & 3;
@@ -432,6 +516,7 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
       l_run = l_run * alpha + rn;
 #pragma unroll
       for (int e = 0; e < 8; ++e) pb[0][e] = (elem)pg[e];
+    }
     }
   };
 
@@ -554,7 +639,7 @@ extern "C" int moba_fwd_tile_rows(void) { return TM; }
 
 template <class E>
 static int launch_partials(const void* q, const void* k, const void* v, void* part_o, float* part_lse,
-                           const TileTables& t, int D, float softmax_scale, int64_t grid, int* queues,
+                           const TileTables& t, int D, float softmax_scale, int64_t grid, int* queues, int* redo,
                            hipStream_t st) {
   FwdParams<E> p;
   p.q = (const typename E::elem*)q; p.k = (const typename E::elem*)k; p.v = (const typename E::elem*)v;
@@ -563,14 +648,26 @@ static int launch_partials(const void* q, const void* k, const void* v, void* pa
   p.scale_log2 = softmax_scale > 0.f ? (float)(1.4426950408889634 * (double)softmax_scale)
                                      : (float)(1.4426950408889634 / sqrt((double)D));
   p.queues = queues;
-  static bool allowed[2][kMaxDevices];  // one pair of arrays per element type
+  p.redo = redo;
+  static bool allowed[4][kMaxDevices];  // one set of arrays per element type
   if (grid > 0) {  // resident workgroups drawing from the queues
-    if (!allow_dynamic_lds((const void*)moba_fwd_kernel<E, true>, kFwdLds, allowed[1])) return MOBA_ERR_LAUNCH;
-    hipLaunchKernelGGL(zero_queues_kernel, dim3(1), dim3(8), 0, st, queues);  // a kernel, not a memset: graph safe
-    hipLaunchKernelGGL((moba_fwd_kernel<E, true>), dim3((unsigned)grid), dim3(256), kFwdLds, st, p);
+    hipLaunchKernelGGL(zero_queues_kernel, dim3(1), dim3(8), 0, st, queues, redo);  // a kernel, not a memset: graph safe
+    if constexpr (std::is_same<E, Bf16>::value) {
+      if (redo) {
+        // fixed-reference softmax, then the tiles it could not serve (normally none) with the tracked maximum
+        if (!allow_dynamic_lds((const void*)moba_fwd_kernel<E, kTilesQueued, true>, kFwdLds, allowed[2]) ||
+            !allow_dynamic_lds((const void*)moba_fwd_kernel<E, kTilesListed, false>, kFwdLds, allowed[3]))
+          return MOBA_ERR_LAUNCH;
+        hipLaunchKernelGGL((moba_fwd_kernel<E, kTilesQueued, true>), dim3((unsigned)grid), dim3(256), kFwdLds, st, p);
+        hipLaunchKernelGGL((moba_fwd_kernel<E, kTilesListed, false>), dim3((unsigned)grid), dim3(256), kFwdLds, st, p);
+        return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
+      }
+    }
+    if (!allow_dynamic_lds((const void*)moba_fwd_kernel<E, kTilesQueued, false>, kFwdLds, allowed[1])) return MOBA_ERR_LAUNCH;
+    hipLaunchKernelGGL((moba_fwd_kernel<E, kTilesQueued, false>), dim3((unsigned)grid), dim3(256), kFwdLds, st, p);
   } else {         // one workgroup per tile id
-    if (!allow_dynamic_lds((const void*)moba_fwd_kernel<E, false>, kFwdLds, allowed[0])) return MOBA_ERR_LAUNCH;
-    hipLaunchKernelGGL((moba_fwd_kernel<E, false>), dim3((unsigned)-grid), dim3(256), kFwdLds, st, p);
+    if (!allow_dynamic_lds((const void*)moba_fwd_kernel<E, kTilePerGroup, false>, kFwdLds, allowed[0])) return MOBA_ERR_LAUNCH;
+    hipLaunchKernelGGL((moba_fwd_kernel<E, kTilePerGroup, false>), dim3((unsigned)-grid), dim3(256), kFwdLds, st, p);
   }
   return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
 }
@@ -582,7 +679,7 @@ extern "C" int moba_fwd_partials(const void* q, const void* k, const void* v, vo
                                  const int32_t* self_tile_prefix, const int32_t* tile_seg,
                                  const int32_t* self_tile_chunk, int64_t S, int H, int Hkv, int D, int K, int F,
                                  int N, int B, int64_t hist_bound, int64_t self_tiles, const int64_t* strides,
-                                 int32_t* queues, float softmax_scale, int dtype, void* stream) {
+                                 int32_t* queues, int32_t* redo, float softmax_scale, int dtype, void* stream) {
   if (!q || !k || !v || !part_o || !part_lse || !chunk_tok || !self_tile_prefix || !self_tile_chunk || !queues)
     return MOBA_ERR_ARG;
   if (Hkv <= 0 || H % Hkv != 0) return MOBA_ERR_ARG;
@@ -612,8 +709,8 @@ extern "C" int moba_fwd_partials(const void* q, const void* k, const void* v, vo
   if (!set_layout(t, strides)) return MOBA_ERR_ARG;
   hipStream_t st = (hipStream_t)stream;
   return dtype == MOBA_DTYPE_F16
-             ? launch_partials<F16>(q, k, v, part_o, part_lse, t, D, softmax_scale, grid, queues, st)
-             : launch_partials<Bf16>(q, k, v, part_o, part_lse, t, D, softmax_scale, grid, queues, st);
+             ? launch_partials<F16>(q, k, v, part_o, part_lse, t, D, softmax_scale, grid, queues, redo, st)
+             : launch_partials<Bf16>(q, k, v, part_o, part_lse, t, D, softmax_scale, grid, queues, redo, st);
 }
 
 extern "C" int moba_fwd_merge(const void* part_o, const float* part_lse, const int32_t* sel, void* out, float* lse,
@@ -639,10 +736,10 @@ extern "C" int moba_fwd(const void* q, const void* k, const void* v, void* part_
                         const int32_t* self_tile_prefix, const int32_t* tile_seg, const int32_t* self_tile_chunk,
                         void* out, float* lse, int64_t S, int H, int Hkv, int D, int K, int F, int N, int B,
                         int64_t hist_bound, int64_t self_tiles, const int64_t* strides, int32_t* queues,
-                        float softmax_scale, int dtype, void* stream) {
+                        int32_t* redo, float softmax_scale, int dtype, void* stream) {
   int rc = moba_fwd_partials(q, k, v, part_o, part_lse, seg_off, tile_off, seg_dest, fchunk_tok, chunk_tok,
                              self_tile_prefix, tile_seg, self_tile_chunk, S, H, Hkv, D, K, F, N, B, hist_bound,
-                             self_tiles, strides, queues, softmax_scale, dtype, stream);
+                             self_tiles, strides, queues, redo, softmax_scale, dtype, stream);
   if (rc != MOBA_OK) return rc;
   return moba_fwd_merge(part_o, part_lse, sel, out, lse, S, H, D, K, dtype, stream);
 }

@@ -14,6 +14,7 @@ Stages (each also callable on its own, which is how the tests reach them):
 from __future__ import annotations
 
 import ctypes
+import os
 from typing import Optional
 
 import torch
@@ -22,6 +23,9 @@ from . import _lib
 from .plan import MobaPlan, TILE_ROWS, make_plan
 
 HEAD_DIM = 128
+# MOBA_FIXED_REFERENCE=0 keeps the forward kernel on its running-maximum softmax for every problem (the
+# fixed-reference form, with its redo list, is otherwise used where the C ABI's `redo` argument says)
+FIXED_REFERENCE = os.environ.get("MOBA_FIXED_REFERENCE", "1") != "0"
 
 
 def _ptr(t: Optional[torch.Tensor]):
@@ -217,14 +221,18 @@ def _forward(q, k, v, plan: MobaPlan, timer: Optional[StageTimer] = None, scale:
     part_lse = torch.empty((S * H * (K + 1),), dtype=torch.float32, device=dev)
     out = torch.empty((S, H, D), dtype=q.dtype, device=dev)
     lse = torch.empty((S, H), dtype=torch.float32, device=dev)
-    queues = torch.empty(8, dtype=torch.int32, device=dev)  # the forward kernel's tile counters (it zeroes them)
+    # the forward kernel's tile counters, then the list of tiles its fixed-reference softmax hands to the kernel
+    # that tracks the running maximum (count first; the call zeroes the counters and the count)
+    scratch = torch.empty(8 + 1 + plan.hist_tile_bound(H) + plan.self_tiles * H, dtype=torch.int32, device=dev)
+    queues, redo = scratch[:8], (scratch[8:] if FIXED_REFERENCE else None)
     with span("fwd_partials"):
         _lib.check(lib.moba_fwd_partials(_ptr(q), _ptr(k), _ptr(v), _ptr(part_o), _ptr(part_lse), _ptr(seg_off),
                                          _ptr(tile_off), _ptr(seg_dest), _ptr(t.get("fchunk_tok")),
                                          _ptr(t["chunk_tok"]), _ptr(t["self_tile_prefix"]), _ptr(tile_seg),
                                          _ptr(t["self_tile_chunk"]), S, H, k.shape[1], D, K, plan.F, plan.N,
                                          plan.chunk_size, plan.hist_tile_bound(H), plan.self_tiles, _strides(q, k),
-                                         _ptr(queues), scale, _dtype_code(q), _stream(dev)), "moba_fwd_partials")
+                                         _ptr(queues), _ptr(redo), scale, _dtype_code(q), _stream(dev)),
+                   "moba_fwd_partials")
     with span("fwd_merge"):
         _lib.check(lib.moba_fwd_merge(_ptr(part_o), _ptr(part_lse), _ptr(sel), _ptr(out), _ptr(lse), S, H, D, K,
                                       _dtype_code(q), _stream(dev)), "moba_fwd_merge")
