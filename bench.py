@@ -40,6 +40,9 @@ WORKLOADS = {
     "cfg3_varlen8_h32_c2048_k3": (None, 32, 32, 2048, 3, False, True),
     "cfg4_L131072_h32_c4096_k12": ([131072], 32, 8, 4096, 12, True, False),
     "cfg5_L1048576_h32_c4096_k12": ([1048576], 32, 8, 4096, 12, False, False),
+    # not BASELINE configurations: the headline shape with longer and shorter chunks (per-tile overhead)
+    "x16k_L131072_h32_c16384_k4": ([131072], 32, 8, 16384, 4, True, False),
+    "x1k_L131072_h32_c1024_k48": ([131072], 32, 8, 1024, 48, True, False),
 }
 DEFAULT = "cfg4_L131072_h32_c4096_k12"
 

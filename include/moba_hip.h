@@ -39,7 +39,7 @@ extern "C" {
 
 enum { MOBA_DTYPE_BF16 = 0, MOBA_DTYPE_F16 = 1 };
 
-#define MOBA_ABI_VERSION 103 /* the signatures below; moba_version() returns the number the library was built with */
+#define MOBA_ABI_VERSION 104 /* the signatures below; moba_version() returns the number the library was built with */
 int moba_version(void);
 const char* moba_strerror(int code);
 
@@ -91,10 +91,19 @@ int moba_topk_from_scores(const float* scores, int32_t* sel, int64_t S, int H, i
  *            sum of ceil(rows/tile_rows);  seg_dest [M] out, entries
  *            (token*H + h)*(K+1) + 1 + slot
  *   tile_seg [hist_bound] out: segment f*H + h of every history tile id, -1 past the last tile
- * cmax = most chunks in a sequence minus one; hist_bound as in moba_fwd_partials. */
+ * cmax = most chunks in a sequence minus one; tile_rows = rows per tile of the kernel that will read tile_off and
+ * tile_seg (moba_fwd_tile_rows() or moba_bwd_tile_rows()); hist_bound: an upper bound on the number of tiles,
+ * e.g. M / tile_rows + F * H. */
 int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, const int32_t* chunk_fb, const int32_t* chunk_local,
                      const int32_t* pair_off, int32_t* cnt, int32_t* seg_off, int32_t* tile_off, int32_t* seg_dest,
                      int32_t* tile_seg, int64_t S, int H, int K, int N, int F, int P, int cmax, int tile_rows,
+                     int64_t hist_bound, void* stream);
+
+/* The tile tables of moba_build_lists alone, for another tile height: the forward and the backward kernels cut
+ * the same gather lists into tiles of moba_fwd_tile_rows() and moba_bwd_tile_rows() rows.  No counterpart in the
+ * reference (flash-attn tiles its varlen batches internally).
+ *   seg_off [F*H+1] from moba_build_lists; tile_off [F*H+1] out; tile_seg [hist_bound] out */
+int moba_tile_tables(const int32_t* seg_off, int32_t* tile_off, int32_t* tile_seg, int H, int F, int tile_rows,
                      int64_t hist_bound, void* stream);
 
 /* Attention.  Replaces MixedAttention.forward, moba/moba_efficient.py:69-183 (two
@@ -103,11 +112,12 @@ int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, const int32_t
  *   part_o [S*H*(K+1), D] elem and part_lse [S*H*(K+1)] fp32: per-slot partial results
  *   self_tile_prefix [N+1] int32: prefix sum of ceil(chunk_len / moba_fwd_tile_rows())
  *   self_tile_chunk [self_tile_prefix[N]] int32: the chunk of each of those tiles
- *   tile_seg: from moba_build_lists (may be NULL when K = 0)
+ *   tile_off, tile_seg: from moba_build_lists or moba_tile_tables with tile_rows = moba_fwd_tile_rows()
+ *              (may be NULL when K = 0)
  *   out [S,H,D] elem, lse [S,H] fp32 (natural log)
- *   hist_bound: upper bound on the number of history tiles, e.g. M/tile_rows + F*H
+ *   hist_bound: upper bound on the number of history tiles, e.g. M / moba_fwd_tile_rows() + F*H
  *   self_tiles: self_tile_prefix[N]
- *   queues [8] int32 scratch: the tile counters of the forward kernel, whose workgroups (two per CU) stay
+ *   queues [8] int32 scratch: the tile counters of the forward kernel, whose workgroups (one per CU) stay
  *              resident and draw tiles from one queue per XCD; the call zeroes them with a kernel of its own.
  *              Calls that overlap in time need their own eight counters each.
  *   redo   [1 + hist_bound + self_tiles * H] int32 scratch, or NULL.  With it, bf16 problems large enough for the
@@ -120,6 +130,7 @@ int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, const int32_t
  *              (moba/moba_efficient.py:86).  A caller whose heads are narrower than D pads them with zeros
  *              and passes its own head_dim^-0.5. */
 int moba_fwd_tile_rows(void);
+int moba_bwd_tile_rows(void);
 int moba_fwd_partials(const void* q, const void* k, const void* v, void* part_o, float* part_lse,
                       const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest,
                       const int32_t* fchunk_tok, const int32_t* chunk_tok, const int32_t* self_tile_prefix,
@@ -139,6 +150,8 @@ int moba_fwd(const void* q, const void* k, const void* v, void* part_o, float* p
  * autograd scatter of its gathered gradients.  Deterministic (no floating-point atomics).
  *   dout, q, out, dq [S,H,D] elem; k, v, dk, dv [S,Hkv,D] elem; lse [S,H] fp32 from the forward
  *   (`strides` applies to q, k, v; dout, out, dq, dk, dv are packed)
+ *   tile_off, tile_seg, self_tile_prefix, self_tile_chunk, hist_bound, self_tiles: as in moba_fwd_partials, but for
+ *   tiles of moba_bwd_tile_rows() rows (moba_tile_tables makes the first two from seg_off)
  *   chunk_fid [N] int32: filtered id of each chunk, -1 for the last chunk of a sequence
  *   delta [2,S,H] fp32 scratch (rowsum(dO*O), then the LSE in the log2 domain); part_dq [S*H*(K+1), D] elem scratch (the per-slot dQ, rounded as the per-chunk dQ that flash-attn returns to the reference is)
  *   dq, dk, dv: out; dk and dv of a key/value head sum over its query heads

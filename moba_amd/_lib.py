@@ -31,7 +31,9 @@ _SIGNATURES = {
                                c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_strides, c_int, c_void_p]),
     "moba_topk_from_scores": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_void_p]),
     "moba_build_lists": (c_int, [c_void_p] * 10 + [c_int64] + [c_int] * 7 + [c_int64, c_void_p]),
+    "moba_tile_tables": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int64, c_void_p]),
     "moba_fwd_tile_rows": (c_int, []),
+    "moba_bwd_tile_rows": (c_int, []),
     "moba_fwd_partials": (c_int, [c_void_p] * 13 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int64,
                                                    c_int64, c_strides, c_void_p, c_void_p, c_float, c_int, c_void_p]),
     "moba_fwd_merge": (c_int, [c_void_p] * 5 + [c_int64, c_int, c_int, c_int, c_int, c_void_p]),
@@ -43,7 +45,7 @@ _SIGNATURES = {
     "moba_decode": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_int64] * 4 + [c_float, c_int, c_void_p]),
 }
 OPTIONAL = set()
-ABI_VERSION = 103  # MOBA_ABI_VERSION of include/moba_hip.h, the signatures above
+ABI_VERSION = 104  # MOBA_ABI_VERSION of include/moba_hip.h, the signatures above
 DTYPE_BF16, DTYPE_F16 = 0, 1
 
 

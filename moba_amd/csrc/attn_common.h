@@ -6,7 +6,8 @@
 
 namespace moba {
 
-constexpr int TM = 128;  // query rows per workgroup (32 per wave)
+constexpr int TM = 128;  // query rows per workgroup of the backward kernels (32 per wave)
+constexpr int kFwdTileRows = 256;  // ... and of the forward kernel (8 waves)
 constexpr int TN = 64;   // keys per inner iteration
 constexpr int kTileBytes = TN * kHeadDim * 2;
 constexpr int kXcdBlock = 64;  // consecutive logical tiles that share an XCD (one workgroup per tile id)
@@ -97,7 +98,8 @@ __device__ __forceinline__ int decode_tile_code(const TileTables& p, int logical
 }
 // Step 1, wave-uniform: head, key range, number of rows, from the small per-segment / per-chunk tables.
 // Returns false (and row_count = 0) for a code that is not a tile.
-__device__ __forceinline__ bool decode_tile_head(const TileTables& p, int logical, int code, Tile& t) {
+// (tm: rows per tile of the tables in p)
+__device__ __forceinline__ bool decode_tile_head(const TileTables& p, int logical, int code, Tile& t, int tm = TM) {
   const int H = p.H;
   t.id = logical;
   t.row_count = 0;
@@ -108,8 +110,8 @@ __device__ __forceinline__ bool decode_tile_head(const TileTables& p, int logica
     const int tile = logical - p.tile_off[seg];
     const int f = seg / H;
     t.h = seg - f * H;
-    t.base = p.seg_off[seg] + tile * TM;
-    t.row_count = min(TM, p.seg_off[seg + 1] - t.base);
+    t.base = p.seg_off[seg] + tile * tm;
+    t.row_count = min(tm, p.seg_off[seg + 1] - t.base);
     t.kv_tok0 = p.fchunk_tok[f];
     t.nkeys = p.B;
     t.rot = tile;
@@ -123,15 +125,15 @@ __device__ __forceinline__ bool decode_tile_head(const TileTables& p, int logica
   const int tin = nt - 1 - (rem - t.h * nt);  // longest tiles first
   const int c0 = p.chunk_tok[c];
   const int len = p.chunk_tok[c + 1] - c0;
-  t.base = -1 - tin * TM;                   // self tile: -(first row of the tile inside its chunk) - 1
-  t.row_count = min(TM, len - tin * TM);
+  t.base = -1 - tin * tm;                   // self tile: -(first row of the tile inside its chunk) - 1
+  t.row_count = min(tm, len - tin * tm);
   t.kv_tok0 = c0;
-  t.nkeys = min(len, tin * TM + TM);
+  t.nkeys = min(len, tin * tm + tm);
   t.rot = 0;
   return true;
 }
-__device__ __forceinline__ bool decode_tile_head(const TileTables& p, int logical, Tile& t) {
-  return decode_tile_head(p, logical, decode_tile_code(p, logical), t);
+__device__ __forceinline__ bool decode_tile_head(const TileTables& p, int logical, Tile& t, int tm = TM) {
+  return decode_tile_head(p, logical, decode_tile_code(p, logical), t, tm);
 }
 // Step 2a, per row: the gather-list entry of row r (history tiles; self tiles need no lookup).
 __device__ __forceinline__ int decode_tile_row_entry(const TileTables& p, int r, const Tile& t) {

@@ -760,6 +760,8 @@ static int launch_bwd(const void* dout, const void* q, const void* k, const void
   return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
 }
 
+extern "C" int moba_bwd_tile_rows(void) { return TM; }
+
 extern "C" int moba_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out,
                         const float* lse, const int32_t* sel, const int32_t* seg_off, const int32_t* tile_off,
                         const int32_t* seg_dest, const int32_t* fchunk_tok, const int32_t* chunk_tok,

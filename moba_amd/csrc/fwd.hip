@@ -1,13 +1,15 @@
 // Fused MoBA forward for gfx950.
 //
-// One kernel covers both kinds of work, as tiles of 128 query rows of one head:
-//   history tile : 128 rows of the gather list of segment (filtered chunk f, head h),
+// One kernel covers both kinds of work, as tiles of 256 query rows of one head (eight waves of 32 rows:
+// one workgroup per CU, so that a K/V tile is copied into the CU's LDS once for 256 rows -- the copies
+// global -> LDS are the second largest cost of the kernel after the matrix instructions):
+//   history tile : 256 rows of the gather list of segment (filtered chunk f, head h),
 //                  against the B keys of chunk f, no mask
-//   self tile    : 128 consecutive rows of one chunk against the keys of the same
+//   self tile    : 256 consecutive rows of one chunk against the keys of the same
 //                  chunk up to the diagonal (causal); with the chunk table set to whole
 //                  sequences this is plain causal attention (the k <= 0 case)
 // Each tile runs a flash-style loop over 64-key tiles: K and V tiles are staged in LDS
-// (double buffered, bank-conflict-free swizzles), S^T = K Q^T and O^T += V^T P^T use
+// (a ring of three stages, bank-conflict-free swizzles), S^T = K Q^T and O^T += V^T P^T use
 // v_mfma_f32_32x32x16_bf16 with the query index in the lane dimension, so a row's
 // softmax statistics live in one lane pair; V^T fragments come from ds_read_b64_tr_b16.
 // A tile writes a normalised partial output (bf16) and its log2-sum-exp into the
@@ -21,9 +23,13 @@
 
 namespace moba {
 
-// LDS: K[2], V[2] stages, then 256 bytes per wave for the gather-list entries of the next tile's rows,
-// then the slot through which wave 0 hands the tile id it drew to the other waves
-constexpr int kFwdEntries = 4 * kTileBytes, kFwdIdSlot = kFwdEntries + 4 * 256;
+// LDS: three K stages, three V stages (a ring: key tile t lives in stage t % 3), then 256 bytes per wave for the
+// gather-list entries of the next tile's rows, then the slot through which wave 0 hands the tile id it drew to
+// the other waves
+constexpr int kFwdWaves = 8;
+constexpr int kFwdStages = 3;
+constexpr int kFwdVBase = kFwdStages * kTileBytes;
+constexpr int kFwdEntries = 2 * kFwdStages * kTileBytes, kFwdIdSlot = kFwdEntries + kFwdWaves * 256;
 constexpr int kFwdRedoWord = kFwdIdSlot + 8;  // set by a wave whose rows left the range of the fixed-reference softmax
 constexpr int kFwdLds = kFwdIdSlot + 16;
 
@@ -57,8 +63,12 @@ enum : int {
 //     phase 1:  S^T(u+1)      8 MFMA   with   exponentials 8..15 of block u, packing of P(u)
 //     phase 2:  O^T += V^T P^T(u)  8 MFMA   with   row max of block u+1 and its exponentials 0..7
 // so the vector work of one block executes under the MFMAs of its neighbours, and the
-// fragment reads from LDS run a few MFMAs ahead.  K and V tiles (64 keys) are double
-// buffered separately: K(t+1) must be resident half a tile before V(t+1).
+// fragment reads from LDS run a few MFMAs ahead.
+//
+// K and V tiles (64 keys) travel through a ring of three LDS stages; every wave copies an eighth of each tile.
+// One barrier per key tile, at its top: a wave first waits for its own copies of tile t+1 (issued a whole tile
+// earlier), and once all eight waves have passed the barrier tile t+1 is complete in LDS and nobody reads tile
+// t-1 any more, so its stage takes tile t+2.
 // kMode: resident workgroups that draw tiles from the queues (large problems), or one tile per workgroup,
 // the id from the workgroup id: with few tiles the queue protocol's start-up and wind-down (three passes
 // to fill the look-ahead, eight empty draws to know that nothing is left) would dominate.
@@ -70,7 +80,7 @@ enum : int {
 // safe range -- scores that rise by more than 96 powers of two within one tile -- marks its tile in
 // FwdParams::redo, and the kTilesListed kernel, which tracks the maximum, computes those tiles again.
 template <class E, int kMode, bool kFixedRef>
-__global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) {
+__global__ __launch_bounds__(512, 2) void moba_fwd_kernel(const FwdParams<E> p) {
   MOBA_ELEM_TYPES(E)
   constexpr bool kQueued = kMode == kTilesQueued;
   static_assert(!kFixedRef || (kQueued && std::is_same<E, Bf16>::value), "the fixed reference needs bf16's exponent range");
@@ -99,18 +109,18 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
   elem8 bq[8];
 
   // ---- K/V tile loader: global -> LDS without passing through registers.
-  // A wave copy fills 1 KiB = 4 keys x 16 columns of 16 bytes; wave w issues slabs
-  // w, w+4, w+8, w+12.  Lane i lands at slab + 16*i, so the lane picks the global column
-  // whose swizzled LDS position is i.  LDS: K stages at 0 and 16 KiB, V stages at 32 and 48 KiB.
+  // A wave copy fills 1 KiB = 4 keys x 16 columns of 16 bytes; wave w issues slabs w and w+8 of the
+  // tile's 16.  Lane i lands at slab + 16*i, so the lane picks the global column whose swizzled LDS
+  // position is i.  LDS: K stages at 0, 16, 32 KiB, V stages at 48, 64, 80 KiB.
   const int64_t row_bytes = p.t.kv_tok_b;                        // from one K or V token to the next
   const uint32_t lds_base = lds_addr(smem);
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   const int ld_kin = lane >> 4;  // key within the slab
   const int ld_pc = lane & 15;   // physical 16-byte column
-  uint32_t ld_off[4];
+  uint32_t ld_off[2];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int key = 4 * (4 * i + wave_u) + ld_kin;
+  for (int i = 0; i < 2; ++i) {
+    const int key = 4 * (8 * i + wave_u) + ld_kin;
     ld_off[i] = (uint32_t)(key * row_bytes + sw_col16(key, ld_pc) * 16);  // the swizzle is an involution
   }
   const char* k_head = nullptr;  // key 0 of the current tile's key range, this tile's key/value head
@@ -121,15 +131,15 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
     if (full) {  // uniform tile base in SGPRs + constant per-lane offsets: no address arithmetic
       const char* base = head + (int64_t)key0 * row_bytes;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) async_copy16_sv(base, ld_off[i], dst + (4 * i + wave_u) * 1024);
+      for (int i = 0; i < 2; ++i) async_copy16_sv(base, ld_off[i], dst + (8 * i + wave_u) * 1024);
     } else {
       // (rare path: its per-lane constants are derived here, from a value the compiler cannot trace, so
       // that they are not computed ahead of the tile loop and carried through it in registers)
       int kin = ld_kin;
       asm volatile("" : "+v"(kin));
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int slab = 4 * i + wave_u;
+      for (int i = 0; i < 2; ++i) {
+        const int slab = 8 * i + wave_u;
         const int key = 4 * slab + kin;
         const int64_t tk = min((int64_t)kv_tok0 + key0 + key, (int64_t)p.t.S - 1);
         async_copy16(tensor + tk * row_bytes + hkv * p.t.kv_head_b + sw_col16(key, ld_pc) * 16, dst + slab * 1024);
@@ -137,25 +147,21 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
     }
   };
   auto issue_k = [&](int kt, int stage) __attribute__((always_inline)) { issue(k_head, (const char*)p.k, kt, lds_base + stage * kTileBytes); };
-  auto issue_v = [&](int kt, int stage) __attribute__((always_inline)) { issue(v_head, (const char*)p.v, kt, lds_base + (2 + stage) * kTileBytes); };
+  auto issue_v = [&](int kt, int stage) __attribute__((always_inline)) { issue(v_head, (const char*)p.v, kt, lds_base + kFwdVBase + stage * kTileBytes); };
   // rows of V past the end of the key range must not reach the MFMA (0 * NaN): clear them
   auto scrub_v = [&](int kt, int stage) __attribute__((always_inline)) {
     const int key0 = kt * TN;
     if (key0 + TN <= nkeys) return;
-    char* vdst = smem + (2 + stage) * kTileBytes;
+    char* vdst = smem + kFwdVBase + stage * kTileBytes;
     int ln = lane;  // rare path: see the remark in the loader
     asm volatile("" : "+v"(ln));
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int slab = 4 * i + wave_u;
+    for (int i = 0; i < 2; ++i) {
+      const int slab = 8 * i + wave_u;
       const int key = 4 * slab + (ln >> 4);
       if (key0 + key >= nkeys) *reinterpret_cast<u32x4*>(vdst + slab * 1024 + ln * 16) = u32x4{0, 0, 0, 0};
     }
   };
-  auto wait_newer4 = [&](bool newer_issued) __attribute__((always_inline)) {  // all copies landed except the newest group of 4
-    if (newer_issued) __builtin_amdgcn_s_waitcnt(0x0F74); else wait_vmem();
-  };
-
   // Tiles that run side by side on an XCD work on the same chunk; starting each at a
   // different key tile spreads their first touches of the chunk over all of it.
   int nkt = 1, rot = 0;
@@ -172,6 +178,7 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
     for (int s8 = 0; s8 < 8; ++s8) koff[s8] = lds_base + n * 256 + (((2 * s8 + hh) ^ k_sw) << 4);
   }
   // V^T quads: rows 32*kb + 16*j2 + 4*hh + i0 (A) and +8 (B), 8 bytes at d = 32*db + 16*(g16&1) + 4*i1
+  // (addresses inside V stage 0: the immediate of a read spans 64 KiB, not the whole ring)
   uint32_t voffA[4], voffB[4];
   {
     const int v_c16 = 2 * (g16 & 1) + (i1 >> 1);
@@ -179,8 +186,8 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
 #pragma unroll
     for (int db = 0; db < 4; ++db) {
       const int c16 = 4 * db + v_c16;
-      voffA[db] = lds_base + (4 * hh + i0) * 256 + ((c16 ^ (i0 << 2) ^ hh) << 4) + v_sub;
-      voffB[db] = lds_base + (4 * hh + i0 + 8) * 256 + ((c16 ^ (i0 << 2) ^ (hh + 2)) << 4) + v_sub;
+      voffA[db] = lds_base + kFwdVBase + (4 * hh + i0) * 256 + ((c16 ^ (i0 << 2) ^ hh) << 4) + v_sub;
+      voffB[db] = lds_base + kFwdVBase + (4 * hh + i0 + 8) * 256 + ((c16 ^ (i0 << 2) ^ (hh + 2)) << 4) + v_sub;
       // finished addresses, kept as they are: the compiler otherwise holds their summands and adds them
       // again at every use (eight additions per key block)
       asm volatile("" : "+v"(voffA[db]));
@@ -222,6 +229,7 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
   };
 // keeps a value, and therefore the instructions that produce it, at this point of the program
 #define MOBA_PIN(x) asm volatile("" : "+v"(x))
+
 
   bool have_partial = false;  // the accumulators hold a finished tile whose partial is not written yet
   // The drawn id travels through one of two LDS words, alternating per pass: a pass without a tile has no
@@ -304,13 +312,13 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
       if (list_pos >= pn.redo[0]) return;  // (uniform; the count is final: the kernel that wrote it has ended)
       const int listed = pn.redo[1 + list_pos];
       list_pos += gridDim.x;
-      if (!decode_tile_head(pn.t, listed, t)) return;  // (cannot happen: listed ids are tiles)
+      if (!decode_tile_head(pn.t, listed, t, kFwdTileRows)) return;  // (cannot happen: listed ids are tiles)
     } else {
-      if (!decode_tile_head(pn.t, logical_tile_id(), t)) return;
+      if (!decode_tile_head(pn.t, logical_tile_id(), t, kFwdTileRows)) return;
     }
     if (t.row_count > 0) {
-      // the wave-uniform half of the description is enough to start the first copies: the first K and V
-      // tiles and the second K tile (global -> LDS)
+      // the wave-uniform half of the description is enough to start the first copies: the first two K
+      // and V tiles (global -> LDS)
       h = t.h; nkeys = t.nkeys; kv_tok0 = t.kv_tok0;
       hkv = h / pn.t.rep;  // key/value head of this query head
       k_head = (const char*)pn.k + (int64_t)kv_tok0 * row_bytes + hkv * pn.t.kv_head_b;
@@ -319,7 +327,11 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
       rot = t.rot % nkt;
       issue_k(key_tile(0), 0);
       issue_v(key_tile(0), 0);
-      if (nkt > 1) issue_k(key_tile(1), 1);
+      if (nkt > 1) {
+        issue_k(key_tile(1), 1);
+        issue_v(key_tile(1), 1);
+      }
+
       // the per-row half, then the Q rows.  Q^T operand: lane (n, hh) holds q[tok][16*ks + 8*hh .. +7]
       const int entry = kQueued ? *reinterpret_cast<const int*>(smem + kFwdEntries + 4 * tx)
                                 : decode_tile_row_entry(pn.t, er, t);
@@ -333,7 +345,7 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
     }
     if constexpr (kQueued) {
       // look-ahead: small-table lookups of the tile after, big-table lookup of the one after that, a new id
-      if (!decode_tile_head(pn.t, id2, code2, t1)) t1.nkeys = (code2 == kTilePastEnd) ? -1 : 0;
+      if (!decode_tile_head(pn.t, id2, code2, t1, kFwdTileRows)) t1.nkeys = (code2 == kTilePastEnd) ? -1 : 0;
       id2 = id3;
       code2 = decode_tile_code(pn.t, id2);
       if (tx == 0) drawn = __hip_atomic_fetch_add(pn.queues + queue, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -345,7 +357,10 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
   if constexpr (kQueued) {
     if (tid == 0) *reinterpret_cast<int*>(smem + kFwdIdSlot + 4 * id_word) = drawn;
   }
-  if (t.row_count > 0) scrub_v(key_tile(0), 0);
+  if (t.row_count > 0) {
+    scrub_v(key_tile(0), 0);
+    if (nkt > 1) scrub_v(key_tile(1), 1);
+  }
   __syncthreads();
   if constexpr (kQueued) {
     // the id drawn: queue `queue` counts the ids (8i + queue) * kQueueRun + j; past the last tile the
@@ -520,47 +535,54 @@ __global__ __launch_bounds__(256, 2) void moba_fwd_kernel(const FwdParams<E> p) 
     }
   };
 
-  // st: LDS stage of this tile (= parity of it), compile-time so that every LDS address is
-  // a per-lane register plus an immediate
+  // st: LDS stage of this key tile (it % 3): a constant in the three copies of the hot loop, so that every
+  // LDS address is a per-lane register plus an immediate, a number in the copies that finish a query tile.
   auto tile_body = [&](int it, auto st_c, auto more_c) __attribute__((always_inline)) {
-    constexpr int st = decltype(st_c)::value;
-    constexpr bool more = decltype(more_c)::value;  // a tile follows this one
-    constexpr int kcur = st * kTileBytes, knext = (st ^ 1) * kTileBytes, vcur = (2 + st) * kTileBytes;
+    const int st = static_cast<int>(st_c);
+    constexpr bool more = decltype(more_c)::value;  // a key tile follows this one
+    const int st1 = (st + 1) % kFwdStages, st2 = (st + 2) % kFwdStages;
+    const int kcur = st * kTileBytes, knext = st1 * kTileBytes, vcur = st * kTileBytes;
     const int key0 = key_tile(it) * TN;
     const int key0n = more ? key_tile(it + 1) * TN : 0;
     // the mask is needed once a key block reaches past the smallest row limit of the wave
     const bool mask_a = key0 + 63 > min_limit;
     const bool mask_b = more && (key0n + 31 > min_limit);
-    if constexpr (more) issue_v(key_tile(it + 1), st ^ 1);  // V(it-1) is dead since the barrier that ended tile it-1
-
-    step(s0, s1, kcur, 1, key0 + 32, std::true_type{}, mask_a, vcur, 0);
-
-    // K(it) is dead; K(it+1) must be visible for the second half of this tile
-    if constexpr (more) wait_newer4(true);
-    __syncthreads();
-    if (it + 2 < nkt) issue_k(key_tile(it + 2), st);
-
-    step(s1, s0, knext, 0, key0n, more_c, mask_b, vcur, 1);
-
     if constexpr (more) {
-      wait_newer4(it + 2 < nkt);
-      scrub_v(key_tile(it + 1), st ^ 1);
+      wait_vmem();
+      scrub_v(key_tile(it + 1), st1);
+      __syncthreads();
+      if (it + 2 < nkt) {
+        issue_k(key_tile(it + 2), st2);
+        issue_v(key_tile(it + 2), st2);
+      }
     }
-    __syncthreads();
+    step(s0, s1, kcur, 1, key0 + 32, std::true_type{}, mask_a, vcur, 0);
+    step(s1, s0, knext, 0, key0n, more_c, mask_b, vcur, 1);
   };
   using St0 = std::integral_constant<int, 0>;
   using St1 = std::integral_constant<int, 1>;
+  using St2 = std::integral_constant<int, 2>;
+  // Three copies of the body, one per stage, make the hot loop.  The up to two key tiles left before the
+  // last one, and the last one (no tile follows it), run through a fourth and a fifth copy that take the
+  // stage as a number: with more copies, or a loop with several exits, the compiler's register allocation
+  // degrades for the whole kernel (a thousand bytes of spills).
   int it = 0;
-  for (; it + 2 < nkt; it += 2) {
+  for (; it + 3 < nkt; it += 3) {
     tile_body(it, St0{}, std::true_type{});
     tile_body(it + 1, St1{}, std::true_type{});
+    tile_body(it + 2, St2{}, std::true_type{});
   }
-  if (it + 2 == nkt) {
-    tile_body(it, St0{}, std::true_type{});
-    tile_body(it + 1, St1{}, std::false_type{});
-  } else {
-    tile_body(it, St0{}, std::false_type{});
+  for (; it + 1 < nkt; ++it) {
+    int st = it % kFwdStages;
+    asm volatile("" : "+s"(st));  // a number, not one of three constants
+    tile_body(it, st, std::true_type{});
   }
+  {
+    int st = it % kFwdStages;
+    asm volatile("" : "+s"(st));
+    tile_body(it, st, std::false_type{});
+  }
+  __syncthreads();  // every wave has read its last fragments: the stages may take the partial's rows
   }  // tiles
 #undef MOBA_PIN
 }
@@ -635,7 +657,7 @@ __global__ __launch_bounds__(256) void moba_merge_kernel(const typename E::elem*
 
 using namespace moba;
 
-extern "C" int moba_fwd_tile_rows(void) { return TM; }
+extern "C" int moba_fwd_tile_rows(void) { return kFwdTileRows; }
 
 template <class E>
 static int launch_partials(const void* q, const void* k, const void* v, void* part_o, float* part_lse,
@@ -658,16 +680,16 @@ static int launch_partials(const void* q, const void* k, const void* v, void* pa
         if (!allow_dynamic_lds((const void*)moba_fwd_kernel<E, kTilesQueued, true>, kFwdLds, allowed[2]) ||
             !allow_dynamic_lds((const void*)moba_fwd_kernel<E, kTilesListed, false>, kFwdLds, allowed[3]))
           return MOBA_ERR_LAUNCH;
-        hipLaunchKernelGGL((moba_fwd_kernel<E, kTilesQueued, true>), dim3((unsigned)grid), dim3(256), kFwdLds, st, p);
-        hipLaunchKernelGGL((moba_fwd_kernel<E, kTilesListed, false>), dim3((unsigned)grid), dim3(256), kFwdLds, st, p);
+        hipLaunchKernelGGL((moba_fwd_kernel<E, kTilesQueued, true>), dim3((unsigned)grid), dim3(512), kFwdLds, st, p);
+        hipLaunchKernelGGL((moba_fwd_kernel<E, kTilesListed, false>), dim3((unsigned)grid), dim3(512), kFwdLds, st, p);
         return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
       }
     }
     if (!allow_dynamic_lds((const void*)moba_fwd_kernel<E, kTilesQueued, false>, kFwdLds, allowed[1])) return MOBA_ERR_LAUNCH;
-    hipLaunchKernelGGL((moba_fwd_kernel<E, kTilesQueued, false>), dim3((unsigned)grid), dim3(256), kFwdLds, st, p);
+    hipLaunchKernelGGL((moba_fwd_kernel<E, kTilesQueued, false>), dim3((unsigned)grid), dim3(512), kFwdLds, st, p);
   } else {         // one workgroup per tile id
     if (!allow_dynamic_lds((const void*)moba_fwd_kernel<E, kTilePerGroup, false>, kFwdLds, allowed[0])) return MOBA_ERR_LAUNCH;
-    hipLaunchKernelGGL((moba_fwd_kernel<E, kTilePerGroup, false>), dim3((unsigned)-grid), dim3(256), kFwdLds, st, p);
+    hipLaunchKernelGGL((moba_fwd_kernel<E, kTilePerGroup, false>), dim3((unsigned)-grid), dim3(512), kFwdLds, st, p);
   }
   return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
 }
@@ -690,11 +712,11 @@ extern "C" int moba_fwd_partials(const void* q, const void* k, const void* v, vo
   if ((int64_t)S * H * (K + 1) >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
   const int64_t total = (K > 0 ? hist_bound : 0) + self_tiles * H;
   if (total >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
-  // two workgroups per CU (what the kernel's registers and LDS allow), all resident at once and drawing
+  // one workgroup of eight waves per CU (what the kernel's registers allow), all resident at once and drawing
   // tiles from the queues; a multiple of 8 so that every XCD starts on its own queue with as many
   const int cus = compute_units();
   if (cus <= 0) return MOBA_ERR_LAUNCH;
-  int64_t grid = (2 * (int64_t)cus + 7) / 8 * 8;
+  int64_t grid = ((int64_t)cus + 7) / 8 * 8;
   // with fewer than a few tiles per resident workgroup the queues do not pay: one workgroup per id then
   // (a negative grid tells the launcher)
   if (total < 8 * grid) grid = -((total + 8 * kXcdBlock - 1) / (8 * kXcdBlock) * (8 * kXcdBlock));

@@ -202,6 +202,13 @@ __global__ __launch_bounds__(256) void lists_segments_kernel(const int* __restri
   tile_off[fh] = (end - start + tile_rows - 1) / tile_rows;
 }
 
+// number of row tiles per (f, h) from the list starts
+__global__ __launch_bounds__(256) void lists_tile_counts_kernel(const int* __restrict__ seg_off,
+                                                                int* __restrict__ tile_off, int FH, int tile_rows) {
+  const int fh = blockIdx.x * 256 + threadIdx.x;
+  if (fh < FH) tile_off[fh] = (seg_off[fh + 1] - seg_off[fh] + tile_rows - 1) / tile_rows;
+}
+
 // segment of every history tile id below `bound` (-1 past the last tile): the attention
 // kernels then find their tile with one load instead of a search in tile_off
 __global__ __launch_bounds__(256) void lists_tile_seg_kernel(const int* __restrict__ tile_off,
@@ -251,6 +258,22 @@ extern "C" int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, co
 #undef MOBA_FILL
   hipLaunchKernelGGL(lists_segments_kernel, dim3((F * H + 1 + 255) / 256), dim3(256), 0, st, (const int*)cnt,
                      pair_off, seg_off, tile_off, F, H, tile_rows);
+  hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(1024), 0, st, tile_off, F * H);
+  hipLaunchKernelGGL(lists_tile_seg_kernel, dim3((unsigned)((hist_bound + 255) / 256)), dim3(256), 0, st,
+                     (const int*)tile_off, tile_seg, F * H, (int)hist_bound);
+  return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
+}
+
+// The tile tables alone, for another number of rows per tile, from the list starts moba_build_lists wrote
+// (the forward and the backward kernels cut the same lists into tiles of different heights).
+extern "C" int moba_tile_tables(const int32_t* seg_off, int32_t* tile_off, int32_t* tile_seg, int H, int F,
+                                int tile_rows, int64_t hist_bound, void* stream) {
+  if (!seg_off || !tile_off || !tile_seg) return MOBA_ERR_ARG;
+  if (H <= 0 || F <= 0 || tile_rows <= 0 || hist_bound <= 0 || hist_bound >= 0x7fffffffLL) return MOBA_ERR_ARG;
+  if ((int64_t)F * H >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
+  hipStream_t st = (hipStream_t)stream;
+  hipLaunchKernelGGL(lists_tile_counts_kernel, dim3((F * H + 255) / 256), dim3(256), 0, st, seg_off, tile_off, F * H,
+                     tile_rows);
   hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(1024), 0, st, tile_off, F * H);
   hipLaunchKernelGGL(lists_tile_seg_kernel, dim3((unsigned)((hist_bound + 255) / 256)), dim3(256), 0, st,
                      (const int*)tile_off, tile_seg, F * H, (int)hist_bound);

@@ -20,7 +20,7 @@ from typing import Optional
 import torch
 
 from . import _lib
-from .plan import MobaPlan, TILE_ROWS, make_plan
+from .plan import FWD_TILE_ROWS, MobaPlan, TILE_ROWS, make_plan
 
 HEAD_DIM = 128
 # MOBA_FIXED_REFERENCE=0 keeps the forward kernel on its running-maximum softmax for every problem (the
@@ -144,8 +144,9 @@ def topk_from_scores(scores: torch.Tensor, K: int) -> torch.Tensor:
     return sel
 
 
-def build_lists(sel: torch.Tensor, plan: MobaPlan):
-    """(seg_off [F*H+1], tile_off [F*H+1], seg_dest [M], tile_seg [tile bound]) int32 -- see csrc/lists.hip."""
+def build_lists(sel: torch.Tensor, plan: MobaPlan, tile_rows: int = FWD_TILE_ROWS):
+    """(seg_off [F*H+1], tile_off [F*H+1], seg_dest [M], tile_seg [tile bound]) int32 -- see csrc/lists.hip.
+    The tile tables cut the lists into tiles of `tile_rows` rows (the forward kernel's by default)."""
     lib = _lib.load()
     S, H, K = sel.shape
     dev = sel.device
@@ -154,14 +155,26 @@ def build_lists(sel: torch.Tensor, plan: MobaPlan):
     seg_off = torch.empty(plan.F * H + 1, dtype=torch.int32, device=dev)
     tile_off = torch.empty(plan.F * H + 1, dtype=torch.int32, device=dev)
     seg_dest = torch.empty(max(M, 1), dtype=torch.int32, device=dev)
-    bound = plan.hist_tile_bound(H)
+    bound = plan.hist_tile_bound(H, tile_rows)
     tile_seg = torch.empty(bound, dtype=torch.int32, device=dev)
     t = plan.tables
     _lib.check(lib.moba_build_lists(_ptr(sel), _ptr(t["chunk_tok"]), _ptr(t["chunk_fb"]), _ptr(t["chunk_local"]),
                                     _ptr(t["pair_off"]), _ptr(cnt), _ptr(seg_off), _ptr(tile_off), _ptr(seg_dest),
-                                    _ptr(tile_seg), S, H, K, plan.N, plan.F, plan.P, plan.cmax, TILE_ROWS, bound,
+                                    _ptr(tile_seg), S, H, K, plan.N, plan.F, plan.P, plan.cmax, tile_rows, bound,
                                     _stream(dev)), "moba_build_lists")
     return seg_off, tile_off, seg_dest, tile_seg
+
+
+def tile_tables(seg_off: torch.Tensor, plan: MobaPlan, H: int, tile_rows: int):
+    """(tile_off [F*H+1], tile_seg [tile bound]) for tiles of `tile_rows` rows, from the list starts."""
+    lib = _lib.load()
+    dev = seg_off.device
+    tile_off = torch.empty(plan.F * H + 1, dtype=torch.int32, device=dev)
+    bound = plan.hist_tile_bound(H, tile_rows)
+    tile_seg = torch.empty(bound, dtype=torch.int32, device=dev)
+    _lib.check(lib.moba_tile_tables(_ptr(seg_off), _ptr(tile_off), _ptr(tile_seg), H, plan.F, tile_rows, bound,
+                                    _stream(dev)), "moba_tile_tables")
+    return tile_off, tile_seg
 
 
 class StageTimer:
@@ -223,14 +236,15 @@ def _forward(q, k, v, plan: MobaPlan, timer: Optional[StageTimer] = None, scale:
     lse = torch.empty((S, H), dtype=torch.float32, device=dev)
     # the forward kernel's tile counters, then the list of tiles its fixed-reference softmax hands to the kernel
     # that tracks the running maximum (count first; the call zeroes the counters and the count)
-    scratch = torch.empty(8 + 1 + plan.hist_tile_bound(H) + plan.self_tiles * H, dtype=torch.int32, device=dev)
+    bound = plan.hist_tile_bound(H, FWD_TILE_ROWS)
+    scratch = torch.empty(8 + 1 + bound + plan.fwd_self_tiles * H, dtype=torch.int32, device=dev)
     queues, redo = scratch[:8], (scratch[8:] if FIXED_REFERENCE else None)
     with span("fwd_partials"):
         _lib.check(lib.moba_fwd_partials(_ptr(q), _ptr(k), _ptr(v), _ptr(part_o), _ptr(part_lse), _ptr(seg_off),
                                          _ptr(tile_off), _ptr(seg_dest), _ptr(t.get("fchunk_tok")),
-                                         _ptr(t["chunk_tok"]), _ptr(t["self_tile_prefix"]), _ptr(tile_seg),
-                                         _ptr(t["self_tile_chunk"]), S, H, k.shape[1], D, K, plan.F, plan.N,
-                                         plan.chunk_size, plan.hist_tile_bound(H), plan.self_tiles, _strides(q, k),
+                                         _ptr(t["chunk_tok"]), _ptr(t["fwd_self_tile_prefix"]), _ptr(tile_seg),
+                                         _ptr(t["fwd_self_tile_chunk"]), S, H, k.shape[1], D, K, plan.F, plan.N,
+                                         plan.chunk_size, bound, plan.fwd_self_tiles, _strides(q, k),
                                          _ptr(queues), _ptr(redo), scale, _dtype_code(q), _stream(dev)),
                    "moba_fwd_partials")
     with span("fwd_merge"):
@@ -239,12 +253,14 @@ def _forward(q, k, v, plan: MobaPlan, timer: Optional[StageTimer] = None, scale:
     return out, lse, sel, seg_off, tile_off, seg_dest, tile_seg
 
 
-def _backward(dout, q, k, v, out, lse, sel, seg_off, tile_off, seg_dest, tile_seg, plan: MobaPlan, scale: float = 0.0):
+def _backward(dout, q, k, v, out, lse, sel, seg_off, seg_dest, plan: MobaPlan, scale: float = 0.0):
     lib = _lib.load()
     S, H, D = q.shape
     dev = q.device
     K = plan.K
     t = plan.tables
+    # the backward kernels cut the gather lists into tiles of their own height
+    tile_off, tile_seg = (None, None) if plan.fallback else tile_tables(seg_off, plan, H, TILE_ROWS)
     dq = torch.empty(q.shape, dtype=q.dtype, device=dev)  # packed, whatever the strides of q, k, v
     dk = torch.empty(k.shape, dtype=k.dtype, device=dev)
     dv = torch.empty(v.shape, dtype=v.dtype, device=dev)
@@ -266,10 +282,10 @@ class _MobaAttention(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q, k, v, plan, timer=None, scale=0.0):
-        out, lse, sel, seg_off, tile_off, seg_dest, tile_seg = _forward(q, k, v, plan, timer, scale)
+        out, lse, sel, seg_off, _, seg_dest, _ = _forward(q, k, v, plan, timer, scale)
         ctx.plan = plan
         ctx.scale = scale
-        ctx.aux = (sel, seg_off, tile_off, seg_dest, tile_seg)
+        ctx.aux = (sel, seg_off, seg_dest)
         ctx.save_for_backward(q, k, v, out, lse)
         ctx.mark_non_differentiable(lse)
         return out, lse
@@ -277,9 +293,8 @@ class _MobaAttention(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dout, _dlse):
         q, k, v, out, lse = ctx.saved_tensors
-        sel, seg_off, tile_off, seg_dest, tile_seg = ctx.aux
-        dq, dk, dv = _backward(_aligned(dout.to(q.dtype)), q, k, v, out, lse, sel, seg_off, tile_off, seg_dest, tile_seg,
-                               ctx.plan, ctx.scale)
+        sel, seg_off, seg_dest = ctx.aux
+        dq, dk, dv = _backward(_aligned(dout.to(q.dtype)), q, k, v, out, lse, sel, seg_off, seg_dest, ctx.plan, ctx.scale)
         return dq, dk, dv, None, None, None
 
 

@@ -17,7 +17,8 @@ from typing import Dict, List, Tuple
 import numpy as np
 import torch
 
-TILE_ROWS = 128  # query rows per workgroup of the attention kernels
+TILE_ROWS = 128      # query rows per workgroup of the backward kernels
+FWD_TILE_ROWS = 256  # ... and of the forward kernel
 
 
 @dataclass
@@ -35,13 +36,15 @@ class MobaPlan:
     P: int              # (filtered chunk, later chunk of the same sequence) pairs
     cmax: int           # max chunks per sequence minus one
     pairs_per_head: int  # selected (token, chunk) pairs per head  (M / H)
-    self_tiles: int     # row tiles of the self part, per head
+    self_tiles: int     # row tiles of the self part, per head (TILE_ROWS rows each; tables self_tile_*)
+    fwd_self_tiles: int  # the same in tiles of FWD_TILE_ROWS rows (tables fwd_self_tile_*)
     flops_per_head: float
     tables: Dict[str, torch.Tensor] = field(default_factory=dict)
     host: Dict[str, np.ndarray] = field(default_factory=dict)
 
-    def hist_tile_bound(self, H: int) -> int:
-        return (self.pairs_per_head * H) // TILE_ROWS + self.F * H
+    def hist_tile_bound(self, H: int, rows: int = TILE_ROWS) -> int:
+        """Upper bound on the number of history tiles of `rows` rows (every segment may end in a partial tile)."""
+        return (self.pairs_per_head * H) // rows + self.F * H
 
 
 def _host_tables(cu: np.ndarray, B: int, topk: int):
@@ -65,11 +68,13 @@ def _host_tables(cu: np.ndarray, B: int, topk: int):
         chunk_tok = np.concatenate([chunk_start, [cu[-1]]])
     N = int(n_chunks.sum())
     tiles = (chunk_len + TILE_ROWS - 1) // TILE_ROWS
-    self_tile_prefix = np.concatenate([[0], np.cumsum(tiles)])
-    out = dict(chunk_tok=chunk_tok, self_tile_prefix=self_tile_prefix,
-               self_tile_chunk=np.repeat(np.arange(N), tiles))
+    ftiles = (chunk_len + FWD_TILE_ROWS - 1) // FWD_TILE_ROWS
+    out = dict(chunk_tok=chunk_tok, self_tile_prefix=np.concatenate([[0], np.cumsum(tiles)]),
+               self_tile_chunk=np.repeat(np.arange(N), tiles),
+               fwd_self_tile_prefix=np.concatenate([[0], np.cumsum(ftiles)]),
+               fwd_self_tile_chunk=np.repeat(np.arange(N), ftiles))
     info = dict(nseq=nseq, N=N, F=0 if fallback else F, k_eff=k_eff, fallback=fallback, K=0, P=0, cmax=0,
-                pairs_per_head=0, self_tiles=int(tiles.sum()))
+                pairs_per_head=0, self_tiles=int(tiles.sum()), fwd_self_tiles=int(ftiles.sum()))
     pairs_self = int((chunk_len.astype(np.int64) * (chunk_len + 1) // 2).sum())
     if not fallback:
         seq_fbase = np.concatenate([[0], np.cumsum(n_chunks - 1)])
@@ -129,7 +134,7 @@ def _build(cu: np.ndarray, chunk_size: int, moba_topk: int, device) -> MobaPlan:
     plan = MobaPlan(cu=cu.tolist(), chunk_size=int(chunk_size), moba_topk=int(moba_topk), S=int(cu[-1]),
                     nseq=info["nseq"], N=info["N"], F=info["F"], k_eff=info["k_eff"], K=info["K"],
                     fallback=info["fallback"], P=info["P"], cmax=info["cmax"], pairs_per_head=info["pairs_per_head"],
-                    self_tiles=info["self_tiles"], flops_per_head=info["flops_per_head_per_d"], host=host)
+                    self_tiles=info["self_tiles"], fwd_self_tiles=info["fwd_self_tiles"], flops_per_head=info["flops_per_head_per_d"], host=host)
     if on_device:
         names = list(host)
         flat = np.concatenate([host[n_].astype(np.int32) for n_ in names])

@@ -107,12 +107,19 @@ def test_gather_lists(batch, seqlen, heads, B, topk):
     heads_of = np.repeat(np.arange(plan.F * H) % H, counts)
     want_dest = (rows * H + heads_of) * K1 + 1 + slots
     assert np.array_equal(seg_dest[:offs[-1]], want_dest)
-    tiles = (counts + 127) // 128
-    assert np.array_equal(tile_off, np.concatenate([[0], np.cumsum(tiles)]))
-    # every history tile id names its segment; ids past the last tile are marked
-    want_seg = np.repeat(np.arange(plan.F * H), tiles)
-    assert tile_seg.size == plan.hist_tile_bound(H) >= want_seg.size
-    assert np.array_equal(tile_seg[:want_seg.size], want_seg) and (tile_seg[want_seg.size:] == -1).all()
+    from moba_amd import _lib
+    lib = _lib.load()
+    fwd_rows, bwd_rows = lib.moba_fwd_tile_rows(), lib.moba_bwd_tile_rows()
+    assert (fwd_rows, bwd_rows) == (256, 128)
+    # the tile tables: the forward kernel's from moba_build_lists, the backward kernels' from moba_tile_tables
+    bwd_off, bwd_seg = (x.cpu().numpy() for x in E.tile_tables(torch.from_numpy(seg_off).cuda(), plan, H, bwd_rows))
+    for rows_per_tile, toff, tseg in ((fwd_rows, tile_off, tile_seg), (bwd_rows, bwd_off, bwd_seg)):
+        tiles = (counts + rows_per_tile - 1) // rows_per_tile
+        assert np.array_equal(toff, np.concatenate([[0], np.cumsum(tiles)]))
+        # every history tile id names its segment; ids past the last tile are marked
+        want_seg = np.repeat(np.arange(plan.F * H), tiles)
+        assert tseg.size == plan.hist_tile_bound(H, rows_per_tile) >= want_seg.size
+        assert np.array_equal(tseg[:want_seg.size], want_seg) and (tseg[want_seg.size:] == -1).all()
 
 
 # ------------------------------------------------------------------ forward
@@ -199,9 +206,9 @@ def test_moba_fwd_entry_point(batch, seqlen, heads, B, topk, dtype):
     queues = torch.empty(8, dtype=torch.int32, device=dev)
     p = E._ptr
     _lib.check(lib.moba_fwd(p(qg), p(kg), p(vg), p(part_o), p(part_lse), p(sel), p(seg_off), p(tile_off), p(seg_dest),
-                            p(t.get("fchunk_tok")), p(t["chunk_tok"]), p(t["self_tile_prefix"]), p(tile_seg),
-                            p(t["self_tile_chunk"]), p(out), p(lse), S, H, H, D, K, plan.F, plan.N, plan.chunk_size,
-                            plan.hist_tile_bound(H), plan.self_tiles, None, p(queues), None, 0.0, E._dtype_code(qg),
+                            p(t.get("fchunk_tok")), p(t["chunk_tok"]), p(t["fwd_self_tile_prefix"]), p(tile_seg),
+                            p(t["fwd_self_tile_chunk"]), p(out), p(lse), S, H, H, D, K, plan.F, plan.N, plan.chunk_size,
+                            plan.hist_tile_bound(H, 256), plan.fwd_self_tiles, None, p(queues), None, 0.0, E._dtype_code(qg),
                             E._stream(dev)), "moba_fwd")
     torch.cuda.synchronize()
     assert torch.equal(out, want_out) and torch.equal(lse, want_lse)
@@ -226,13 +233,13 @@ def _attention_stage(q, k, v, plan, aux, with_redo):
     out = torch.zeros((S, H, D), dtype=q.dtype, device=dev)
     lse = torch.zeros((S, H), dtype=torch.float32, device=dev)
     queues = torch.empty(8, dtype=torch.int32, device=dev)
-    tiles = plan.hist_tile_bound(H) + plan.self_tiles * H
+    tiles = plan.hist_tile_bound(H, 256) + plan.fwd_self_tiles * H
     redo = torch.full((1 + tiles,), -7, dtype=torch.int32, device=dev) if with_redo else None
     p = E._ptr
     _lib.check(lib.moba_fwd(p(q), p(k), p(v), p(part_o), p(part_lse), p(sel), p(seg_off), p(tile_off), p(seg_dest),
-                            p(t.get("fchunk_tok")), p(t["chunk_tok"]), p(t["self_tile_prefix"]), p(tile_seg),
-                            p(t["self_tile_chunk"]), p(out), p(lse), S, H, H, D, K, plan.F, plan.N, plan.chunk_size,
-                            plan.hist_tile_bound(H), plan.self_tiles, None, p(queues), p(redo), 0.0,
+                            p(t.get("fchunk_tok")), p(t["chunk_tok"]), p(t["fwd_self_tile_prefix"]), p(tile_seg),
+                            p(t["fwd_self_tile_chunk"]), p(out), p(lse), S, H, H, D, K, plan.F, plan.N, plan.chunk_size,
+                            plan.hist_tile_bound(H, 256), plan.fwd_self_tiles, None, p(queues), p(redo), 0.0,
                             E._dtype_code(q), E._stream(dev)), "moba_fwd")
     torch.cuda.synchronize()
     if redo is None:

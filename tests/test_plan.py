@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 from oracle import moba_oracle as O
-from moba_amd.plan import make_plan, TILE_ROWS
+from moba_amd.plan import make_plan, FWD_TILE_ROWS, TILE_ROWS
 
 
 def rand_cu(rng, nseq, lo, hi):
@@ -39,6 +39,12 @@ def test_plan_tables_match_oracle(seed):
     # every per-head self tile names its chunk: prefix[c] <= t < prefix[c+1]
     stc, pre = plan.host["self_tile_chunk"], plan.host["self_tile_prefix"]
     assert stc.size == plan.self_tiles
+    assert all(pre[c] <= t < pre[c + 1] for t, c in enumerate(stc.tolist()))
+    # the same for the forward kernel's taller tiles
+    assert (TILE_ROWS, FWD_TILE_ROWS) == (128, 256)
+    assert plan.fwd_self_tiles == int(((lens + FWD_TILE_ROWS - 1) // FWD_TILE_ROWS).sum())
+    stc, pre = plan.host["fwd_self_tile_chunk"], plan.host["fwd_self_tile_prefix"]
+    assert stc.size == plan.fwd_self_tiles
     assert all(pre[c] <= t < pre[c + 1] for t, c in enumerate(stc.tolist()))
 
 
