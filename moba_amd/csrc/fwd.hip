@@ -395,6 +395,8 @@ __global__ __launch_bounds__(512, 2) void moba_fwd_kernel(const FwdParams<E> p) 
 
   f32x16 s0, s1;   // S^T, then P^T, of the current and the next key block
   elem8 pb[2];    // P^T operand of the current block: elements 0..7 and 8..15
+  constexpr int kPre = 4;
+  elem8 kpre[kPre > 0 ? kPre : 1];  // the first K fragments of the next step's S^T, read one step ahead
   {
 #pragma unroll
     for (int e = 0; e < 16; ++e) s0[e] = 0.f;
@@ -414,6 +416,8 @@ __global__ __launch_bounds__(512, 2) void moba_fwd_kernel(const FwdParams<E> p) 
       l_run += pe;
       pb[0][e] = (elem)pe;
     }
+#pragma unroll
+    for (int i = 0; i < kPre; ++i) kpre[i] = k_frag(0, 1, i);
   }
 
   // One pipeline step on key block (tile it, block kb).  sc: its S^T with the running max decided
@@ -421,16 +425,19 @@ __global__ __launch_bounds__(512, 2) void moba_fwd_kernel(const FwdParams<E> p) 
   // kn/vs: LDS byte offsets (compile-time) of the K tile of the next block and the V tile of this block.  Each of the 16 slots is one MFMA
   // plus a share of the vector work; the pins and scheduling barriers keep that order.
   auto step = [&](f32x16& sc, f32x16& sn, int kn, int nkb, int next_key0, auto has_next_c, bool masked, int vs,
-                  int kb) __attribute__((always_inline)) {
+                  int kb, bool pre, int pre_kn, int pre_kb) __attribute__((always_inline)) {
     constexpr bool has_next = decltype(has_next_c)::value;
     // ---- phase 1: S^T of the next block under exponentials 8..15 of this block ----
+    // (its first K fragments were read during phase 2 of the step before: kpre)
     elem8 ka[8];
     elem8 va[8];
     float pf[8];
     float rs = 0.f;
     if constexpr (has_next) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) ka[i] = k_frag(kn, nkb, i);
+      for (int i = 0; i < kPre; ++i) ka[i] = kpre[i];
+#pragma unroll
+      for (int i = kPre; i < 4; ++i) ka[i] = k_frag(kn, nkb, i);
     }
 #pragma unroll
     for (int s8 = 0; s8 < 8; ++s8) {
@@ -469,6 +476,7 @@ __global__ __launch_bounds__(512, 2) void moba_fwd_kernel(const FwdParams<E> p) 
       for (int k = 0; k < 8; ++k) {
         const int j2 = k >> 2, db = k & 3;
         if (k + 4 < 8) va[k + 4] = v_frag(vs, kb, 1, db);
+        if (k >= 8 - kPre && pre) kpre[k - (8 - kPre)] = k_frag(pre_kn, pre_kb, k - (8 - kPre));  // for the next step
         oacc[db] = mfma32(va[k], pb[j2], oacc[db]);
         if constexpr (has_next) {
           if (k == 1) {
@@ -496,6 +504,7 @@ __global__ __launch_bounds__(512, 2) void moba_fwd_kernel(const FwdParams<E> p) 
     for (int k = 0; k < 8; ++k) {
       const int j2 = k >> 2, db = k & 3;
       if (k + 4 < 8) va[k + 4] = v_frag(vs, kb, 1, db);
+      if (k >= 8 - kPre && pre) kpre[k - (8 - kPre)] = k_frag(pre_kn, pre_kb, k - (8 - kPre));  // for the next step
       oacc[db] = mfma32(va[k], pb[j2], oacc[db]);
       if constexpr (has_next) {
         if (k == 1) {
@@ -556,8 +565,8 @@ __global__ __launch_bounds__(512, 2) void moba_fwd_kernel(const FwdParams<E> p) 
         issue_v(key_tile(it + 2), st2);
       }
     }
-    step(s0, s1, kcur, 1, key0 + 32, std::true_type{}, mask_a, vcur, 0);
-    step(s1, s0, knext, 0, key0n, more_c, mask_b, vcur, 1);
+    step(s0, s1, kcur, 1, key0 + 32, std::true_type{}, mask_a, vcur, 0, more, knext, 0);
+    step(s1, s0, knext, 0, key0n, more_c, mask_b, vcur, 1, more, knext, 1);
   };
   using St0 = std::integral_constant<int, 0>;
   using St1 = std::integral_constant<int, 1>;
