@@ -31,7 +31,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of moba_fwd_kernel from rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled by a copy
 # kernel of known size (profiles/moba_fwd_128k_hbm_traffic.txt); measured for the headline workload only
-FWD_KERNEL_TRAFFIC_BYTES = {"cfg4_L131072_h32_c4096_k12": 71.44e9}
+FWD_KERNEL_TRAFFIC_BYTES = {"cfg4_L131072_h32_c4096_k12": 52.76e9}
 
 WORKLOADS = {
     # name: (seq lens or None, heads, kv_heads, chunk, topk, normalise, backward)
@@ -40,9 +40,6 @@ WORKLOADS = {
     "cfg3_varlen8_h32_c2048_k3": (None, 32, 32, 2048, 3, False, True),
     "cfg4_L131072_h32_c4096_k12": ([131072], 32, 8, 4096, 12, True, False),
     "cfg5_L1048576_h32_c4096_k12": ([1048576], 32, 8, 4096, 12, False, False),
-    # not BASELINE configurations: the headline shape with longer and shorter chunks (per-tile overhead)
-    "x16k_L131072_h32_c16384_k4": ([131072], 32, 8, 16384, 4, True, False),
-    "x1k_L131072_h32_c1024_k48": ([131072], 32, 8, 1024, 48, True, False),
 }
 DEFAULT = "cfg4_L131072_h32_c4096_k12"
 
@@ -125,6 +122,46 @@ def bench_decode(dev, skv, heads, kv_heads=8, iters=50):
                          "frac": gbs / HBM_PEAK_GBS}}
 
 
+def quick_measure(name, dev, steps, warmup, backward):
+    """Forward (and forward + backward) time of one of the other workloads, a few steps each: wall clock around
+    the steps, bracketed by synchronisations, like the headline figure."""
+    from moba_amd import moba_efficient as E
+    from moba_amd.plan import make_plan
+
+    q, k, v, cu, max_seqlen, B, topk = make_inputs(name, dev)
+    S, H, D = q.shape
+    cu_t = torch.tensor(cu, dtype=torch.int32, device=dev)
+    flops = make_plan(cu_t, B, topk).flops_per_head * D * H
+
+    def timed(fn):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps * 1e3
+
+    with torch.no_grad():
+        fwd_ms = timed(lambda: E.moba_attn_varlen(q, k, v, cu_t, max_seqlen, B, topk))
+    out = {"tokens": S, "heads": H, "chunk": B, "topk": topk, "sequences": len(cu) - 1, "fwd_flops": flops,
+           "fwd_ms": fwd_ms, "fwd_tflops": flops / (fwd_ms * 1e-3) / 1e12}
+    if backward:
+        g = torch.Generator(device=dev).manual_seed(1)
+        do = torch.randn(q.shape, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+        qg, kg, vg = (x.requires_grad_(True) for x in (q, k, v))
+
+        def both():
+            qg.grad = kg.grad = vg.grad = None
+            E.moba_attn_varlen(qg, kg, vg, cu_t, max_seqlen, B, topk).backward(do)
+
+        ms = timed(both)
+        # the backward's algorithmic work is 2.5 x the forward's (5 products against 2)
+        out.update(fwd_bwd_ms=ms, fwd_bwd_tflops=3.5 * flops / (ms * 1e-3) / 1e12)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -136,6 +173,8 @@ def main():
     ap.add_argument("--decode", action="store_true",
                     help="also time the decode kernel (one token against a cache of the workload's length, "
                          "8 KV heads) next to PyTorch SDPA")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="with the default workload: do not also time the other BASELINE configurations")
     ap.add_argument("--gqa", action="store_true",
                     help="keep the key/value heads unexpanded (grouped-query operator) instead of the reference "
                          "wrapper's repeat_kv; not the headline configuration")
@@ -178,20 +217,22 @@ def main():
 
     # forward + backward (reported beside the forward figure for the workloads that name it)
     fwd_bwd_ms = None
-    if WORKLOADS[args.workload][6] or args.backward:
+    others = args.workload == DEFAULT and not args.gqa and not args.no_other_configs
+    if WORKLOADS[args.workload][6] or args.backward or others:
         g = torch.Generator(device=dev).manual_seed(1)
         do = torch.randn(q.shape, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
         qg, kg, vg = (x.clone().requires_grad_(True) for x in (q, k, v))
         op = E.moba_attn_varlen_gqa if args.gqa else E.moba_attn_varlen
-        for _ in range(max(1, args.warmup)):
+        bsteps = args.steps if (WORKLOADS[args.workload][6] or args.backward) else min(args.steps, 3)
+        for _ in range(max(1, min(args.warmup, bsteps))):
             op(qg, kg, vg, cu_t, max_seqlen, B, topk).backward(do)
         torch.cuda.synchronize()
         t1 = time.perf_counter()
-        for _ in range(args.steps):
+        for _ in range(bsteps):
             qg.grad = kg.grad = vg.grad = None
             op(qg, kg, vg, cu_t, max_seqlen, B, topk).backward(do)
         torch.cuda.synchronize()
-        fwd_bwd_ms = (time.perf_counter() - t1) / args.steps * 1e3
+        fwd_bwd_ms = (time.perf_counter() - t1) / bsteps * 1e3
         del qg, kg, vg, do
 
     kern_ms = stage_ms["fwd_partials"]
@@ -220,13 +261,24 @@ def main():
     }
     if fwd_bwd_ms is not None:
         # algorithmic backward work is 2.5x the forward's
-        result["fwd_bwd"] = {"ms_per_step": fwd_bwd_ms, "tflops": 3.5 * flops / (fwd_bwd_ms * 1e-3) / 1e12}
+        result["fwd_bwd"] = {"ms_per_step": fwd_bwd_ms, "tflops": 3.5 * flops / (fwd_bwd_ms * 1e-3) / 1e12,
+                             "pct_mfma_peak": 100.0 * 3.5 * flops / (fwd_bwd_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS}
     if "chunk_mean" in stage_ms:
         gbs = k.numel() * 2 / (stage_ms["chunk_mean"] * 1e-3) / 1e9
         result["chunk_mean_hbm"] = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                     "frac": gbs / HBM_PEAK_GBS}
     if args.decode:
         result["decode"] = bench_decode(dev, S if len(cu) == 2 else max_seqlen, H)
+    if others:
+        # the other BASELINE configurations, a few steps each (cfg5: forward only, as BASELINE states it)
+        del q, k, v
+        torch.cuda.empty_cache()
+        result["other_configs"] = {}
+        for name, steps, warmup in (("cfg1_L4096_h4_c512_k3", 20, 5), ("cfg2_L32768_h1_c2048_k3", 20, 5),
+                                    ("cfg3_varlen8_h32_c2048_k3", 3, 1), ("cfg5_L1048576_h32_c4096_k12", 2, 1)):
+            result["other_configs"][name] = quick_measure(name, dev, steps, warmup, backward=not name.startswith("cfg5"))
+            torch.cuda.empty_cache()
+        q, k, v, cu, max_seqlen, B, topk = make_inputs(args.workload, dev, args.gqa)   # for the CPU baseline's sample
     if not args.no_cpu_baseline:
         rep = H // k.shape[1]
         nkv = (8 + rep - 1) // rep  # key/value heads behind the first 8 query heads
