@@ -7,7 +7,17 @@
  * `stream` is a hipStream_t.
  * The library allocates nothing, frees nothing, and never synchronises the device:
  * every launch is enqueued on `stream`.  Return value: 0, or a negative code that
- * moba_strerror() explains.  head_dim 128 (D below; narrower heads are padded with zeros by the
+ * moba_strerror() explains.  A HIP error already pending on the calling thread is neither reported
+ * nor cleared; an error raised by an entry point's own launches is reported (-3) and cleared.
+ * State the library keeps, all of it per device and filled on first use: the number of compute units,
+ * which kernels have been allowed their dynamic LDS size, and the address of the array of
+ * moba_chunk_mean_static.  First calls may come from several threads at once (the writes are idempotent,
+ * the address is guarded by a mutex); nothing else is shared between calls.
+ * Inputs are expected to be finite: the attention kernels are compiled without NaN handling, and with an
+ * infinity or a NaN in q, k, v or dout the outputs are unspecified (no fault, no hang).  Scores of any finite
+ * size are handled (the softmax subtracts a row reference before it exponentiates).
+ * Index limits, checked (code -4): S * H * (K + 1) < 2^31 (slot rows are 32-bit: 1M tokens x 64 heads x top-k 12
+ * is beyond it, 1M x 32 x 12 is not), K <= 64, chunks per sequence <= 3413, tile counts < 2^31.  head_dim 128 (D below; narrower heads are padded with zeros by the
  * caller, see softmax_scale); q, k, v and everything derived from them are
  * bf16 (dtype = MOBA_DTYPE_BF16) or fp16 (dtype = MOBA_DTYPE_F16, the dtype of the reference's
  * example, examples/llama.py:26); below, "elem" stands for that type.
@@ -39,9 +49,51 @@ extern "C" {
 
 enum { MOBA_DTYPE_BF16 = 0, MOBA_DTYPE_F16 = 1 };
 
-#define MOBA_ABI_VERSION 104 /* the signatures below; moba_version() returns the number the library was built with */
+#define MOBA_ABI_VERSION 105 /* the signatures below; moba_version() returns the number the library was built with */
 int moba_version(void);
 const char* moba_strerror(int code);
+
+/* Host-side planner: counts, buffer sizes and the int32 index tables, all functions of the sequence lengths
+ * alone.  Replaces calc_chunks, moba/moba_efficient.py:14-64, and the bookkeeping of :298-323 (number of filtered
+ * chunks, effective top-k, the full-attention fallback).  Pure host code: host pointers, no device call.
+ *   cu_seqlens_host [nseq+1] int32: starts at 0, strictly increasing
+ * moba_plan fills `plan` (counts, table offsets and table_ints); moba_plan_fill does the same and writes the tables
+ * into tables_host [plan->table_ints] int32, which the caller copies to the device once per batch layout: table X
+ * then lives at device_base + plan->off_X (off_X = -1: the table does not exist in the full-attention fallback,
+ * pass NULL).  Tables: cu_seqlens, chunk_tok [N+1], fwd_self_tile_prefix [N+1] / fwd_self_tile_chunk (the
+ * self_tile_* arguments of moba_fwd*), self_tile_prefix / self_tile_chunk (those of moba_bwd), seq_fbase [nseq+1],
+ * fchunk_tok [F], chunk_fb [N], chunk_local [N], pair_off [F+1], chunk_fid [N].
+ * moba_plan_sizes gives, for H query and Hkv key/value heads, the size of every scratch buffer of the calls below. */
+typedef struct moba_plan_t {
+  int64_t S;
+  int32_t nseq, chunk, topk;
+  int32_t N, F, K, P, cmax;
+  int32_t fallback;                        /* 1: full causal attention (K = 0, one "chunk" per sequence) */
+  int32_t fwd_tile_rows, bwd_tile_rows;
+  int64_t pairs_per_head;                  /* M = pairs_per_head * H */
+  int64_t fwd_self_tiles, bwd_self_tiles;  /* the self_tiles arguments of moba_fwd* and of moba_bwd */
+  double flops_per_head_per_dim;           /* forward flops = this * H * D */
+  int64_t off_cu_seqlens, off_chunk_tok, off_fwd_self_tile_prefix, off_fwd_self_tile_chunk, off_self_tile_prefix,
+      off_self_tile_chunk, off_seq_fbase, off_fchunk_tok, off_chunk_fb, off_chunk_local, off_pair_off, off_chunk_fid;
+  int64_t table_ints;
+} moba_plan_t;
+typedef struct moba_sizes_t {
+  int64_t kbar_elems;                      /* [F, Hkv, D] elem */
+  int64_t chunk_mean_workspace_bytes;
+  int64_t sel_ints;                        /* [S, H, K] */
+  int64_t cnt_ints;                        /* [P*H + 1] */
+  int64_t seg_off_ints;                    /* [F*H + 1]; tile_off has the same size */
+  int64_t seg_dest_ints;                   /* [M] */
+  int64_t fwd_hist_bound, bwd_hist_bound;  /* sizes of the two tile_seg tables = the hist_bound arguments */
+  int64_t part_rows;                       /* S*H*(K+1): part_o, part_dq [part_rows, D] elem; part_lse [part_rows] fp32 */
+  int64_t redo_ints;
+  int64_t lse_floats;                      /* [S, H] */
+  int64_t delta_floats;                    /* [2, S, H] */
+} moba_sizes_t;
+int moba_plan(const int32_t* cu_seqlens_host, int nseq, int chunk, int topk, moba_plan_t* plan);
+int moba_plan_fill(const int32_t* cu_seqlens_host, int nseq, int chunk, int topk, moba_plan_t* plan,
+                   int32_t* tables_host);
+int moba_plan_sizes(const moba_plan_t* plan, int H, int Hkv, int D, moba_sizes_t* sizes);
 
 /* Key chunk-mean.  Replaces moba/moba_efficient.py:326-340 (index_select of the
  * filtered chunks, .mean(dim=1) on bf16, .float()).

@@ -21,6 +21,9 @@ _lib = None
 _SIGNATURES = {
     "moba_version": (c_int, []),
     "moba_strerror": (c_char_p, [c_int]),
+    "moba_plan": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p]),
+    "moba_plan_fill": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p]),
+    "moba_plan_sizes": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p]),
     "moba_chunk_mean_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "moba_chunk_mean": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_strides,
                                 c_int, c_void_p]),
@@ -45,7 +48,26 @@ _SIGNATURES = {
     "moba_decode": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_int64] * 4 + [c_float, c_int, c_void_p]),
 }
 OPTIONAL = set()
-ABI_VERSION = 104  # MOBA_ABI_VERSION of include/moba_hip.h, the signatures above
+
+
+class PlanStruct(ctypes.Structure):
+    """moba_plan_t of include/moba_hip.h."""
+    _fields_ = ([("S", c_int64)] + [(n, ctypes.c_int32) for n in ("nseq", "chunk", "topk", "N", "F", "K", "P", "cmax", "fallback",
+                                                               "fwd_tile_rows", "bwd_tile_rows")]
+                + [("pairs_per_head", c_int64), ("fwd_self_tiles", c_int64), ("bwd_self_tiles", c_int64),
+                   ("flops_per_head_per_dim", ctypes.c_double)]
+                + [("off_" + n, c_int64) for n in ("cu_seqlens", "chunk_tok", "fwd_self_tile_prefix", "fwd_self_tile_chunk",
+                                                   "self_tile_prefix", "self_tile_chunk", "seq_fbase", "fchunk_tok", "chunk_fb",
+                                                   "chunk_local", "pair_off", "chunk_fid")]
+                + [("table_ints", c_int64)])
+
+
+class SizesStruct(ctypes.Structure):
+    """moba_sizes_t of include/moba_hip.h."""
+    _fields_ = [(n, c_int64) for n in ("kbar_elems", "chunk_mean_workspace_bytes", "sel_ints", "cnt_ints", "seg_off_ints",
+                                       "seg_dest_ints", "fwd_hist_bound", "bwd_hist_bound", "part_rows", "redo_ints",
+                                       "lse_floats", "delta_floats")]
+ABI_VERSION = 105  # MOBA_ABI_VERSION of include/moba_hip.h, the signatures above
 DTYPE_BF16, DTYPE_F16 = 0, 1
 
 

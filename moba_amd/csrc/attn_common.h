@@ -220,12 +220,12 @@ __device__ __forceinline__ V4 lds_read_tr(uint32_t addr) {
 // asynchronous 16-byte copy global -> LDS: lane i of the wave fills lds_wave_base + 16*i.
 // Issued as inline assembly so that completion is tracked by the explicit wait_vmem()
 // before the tile barrier only (the copy must stay in flight across the compute phase).
-// The statement overwrites M0, which nothing else in these kernels uses.
+// The statement overwrites M0 and says so to the compiler.
 __device__ __forceinline__ void async_copy16(const void* gsrc, uint32_t lds_wave_base) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
                :
                : "v"(gsrc), "s"(lds_wave_base)
-               : "memory");
+               : "memory", "m0");
 }
 // same with the global address split into a wave-uniform base and a per-lane byte offset
 __device__ __forceinline__ void async_copy16_sv(const void* uniform_base, uint32_t lane_off, uint32_t lds_wave_base) {
@@ -236,14 +236,14 @@ __device__ __forceinline__ void async_copy16_sv(const void* uniform_base, uint32
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                :
                : "v"(lane_off), "s"(sb), "s"(lds_wave_base)
-               : "memory");
+               : "memory", "m0");
 }
 // same for 4 bytes per lane: lane i fills lds_wave_base + 4*i
 __device__ __forceinline__ void async_copy4(const void* gsrc, uint32_t lds_wave_base) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off"
                :
                : "v"(gsrc), "s"(lds_wave_base)
-               : "memory");
+               : "memory", "m0");
 }
 __device__ __forceinline__ uint32_t lds_addr(const char* p) {
   return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)p;

@@ -727,6 +727,7 @@ static int launch_bwd(const void* dout, const void* q, const void* k, const void
                       const int32_t* sel, const int32_t* chunk_fid, float* delta, void* part_dq, void* dq, void* dk,
                       void* dv, const TileTables& t, int64_t S, int H, int D, int K, float softmax_scale, int64_t grid_q,
                       int64_t grid_kv, int* queues, hipStream_t st) {
+  LaunchCheck launch_check;
   typedef typename E::elem elem;
   BwdParams<E> p;
   p.q = (const elem*)q; p.k = (const elem*)k; p.v = (const elem*)v; p.dout = (const elem*)dout;
@@ -757,7 +758,7 @@ static int launch_bwd(const void* dout, const void* q, const void* k, const void
   hipLaunchKernelGGL(bwd_dq_reduce_kernel<E>, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st,
                      (const elem*)part_dq, sel, (elem*)dq, rows, K + 1);
   hipLaunchKernelGGL(bwd_dkv_kernel<E>, dim3((unsigned)grid_kv), dim3(256), kBwdDkvLds, st, p);
-  return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
+  return launch_check.result();
 }
 
 extern "C" int moba_bwd_tile_rows(void) { return TM; }

@@ -101,6 +101,7 @@ extern "C" size_t moba_chunk_mean_workspace_bytes(int H, int D, int F, int B) {
 
 static int launch_chunk_mean(const void* k, const int32_t* fchunk_tok, void* kbar, double* partial, int H, int D,
                              int F, int B, int nsplit, int64_t kts, int64_t khs, int dtype, hipStream_t st) {
+  LaunchCheck launch_check;
   const int HD8 = H * D / 8;
   const int tps = (B + nsplit - 1) / nsplit;
   dim3 grid(F, nsplit, (HD8 + 255) / 256);
@@ -117,7 +118,7 @@ static int launch_chunk_mean(const void* k, const int32_t* fchunk_tok, void* kba
     hipLaunchKernelGGL(chunk_mean_finish_kernel<Bf16>, fgrid, dim3(256), 0, st, (const double*)partial, (bf16*)kbar,
                        HD8, B, nsplit, F);
   }
-  return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
+  return launch_check.result();
 }
 
 // argument checks shared by the two entry points; kts, khs receive the key token and head strides (elements)

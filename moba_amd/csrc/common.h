@@ -103,6 +103,19 @@ __device__ __forceinline__ T kernarg_now(int offset) {
   return x;
 }
 
+// Result of the launches of one entry point: an error that was already pending on the calling thread when the
+// entry point began is neither reported nor cleared; an error the entry point's own launches raised is reported
+// and cleared.
+struct LaunchCheck {
+  hipError_t before = hipPeekAtLastError();
+  int result() const {
+    const hipError_t after = hipPeekAtLastError();
+    if (after == hipSuccess || after == before) return MOBA_OK;
+    (void)hipGetLastError();
+    return MOBA_ERR_LAUNCH;
+  }
+};
+
 // Dynamic LDS above 64 KiB must be allowed per kernel, and the allowance belongs to the current
 // device: `done` (one array per kernel) remembers the devices it was given on.
 constexpr int kMaxDevices = 64;

@@ -235,6 +235,7 @@ static void launch_decode(const void* q, const void* k, const void* v, void* out
 extern "C" int moba_decode(const void* q, const void* k, const void* v, void* out, float* part_o, float* part_lse,
                            int B, int H, int Hkv, int Skv, int D, int64_t q_stride_b, int64_t q_stride_h,
                            int64_t kv_stride_b, int64_t kv_stride_h, float scale, int dtype, void* stream) {
+  LaunchCheck launch_check;
   if (!q || !k || !v || !out || !part_o || !part_lse) return MOBA_ERR_ARG;
   if (B <= 0 || H <= 0 || Hkv <= 0 || Skv <= 0 || H % Hkv != 0 || B > 65535 || Hkv > 65535) return MOBA_ERR_ARG;
   if (D != kHeadDim || (dtype != MOBA_DTYPE_BF16 && dtype != MOBA_DTYPE_F16)) return MOBA_ERR_UNSUPPORTED;
@@ -259,5 +260,5 @@ extern "C" int moba_decode(const void* q, const void* k, const void* v, void* ou
   if (dtype == MOBA_DTYPE_F16) { MOBA_DECODE_REP(F16) } else { MOBA_DECODE_REP(Bf16) }
 #undef MOBA_DECODE_REP
 #undef MOBA_DECODE
-  return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
+  return launch_check.result();
 }

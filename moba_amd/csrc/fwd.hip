@@ -672,6 +672,7 @@ template <class E>
 static int launch_partials(const void* q, const void* k, const void* v, void* part_o, float* part_lse,
                            const TileTables& t, int D, float softmax_scale, int64_t grid, int* queues, int* redo,
                            hipStream_t st) {
+  LaunchCheck launch_check;
   FwdParams<E> p;
   p.q = (const typename E::elem*)q; p.k = (const typename E::elem*)k; p.v = (const typename E::elem*)v;
   p.part_o = (typename E::elem*)part_o; p.part_lse = part_lse;
@@ -691,7 +692,7 @@ static int launch_partials(const void* q, const void* k, const void* v, void* pa
           return MOBA_ERR_LAUNCH;
         hipLaunchKernelGGL((moba_fwd_kernel<E, kTilesQueued, true>), dim3((unsigned)grid), dim3(512), kFwdLds, st, p);
         hipLaunchKernelGGL((moba_fwd_kernel<E, kTilesListed, false>), dim3((unsigned)grid), dim3(512), kFwdLds, st, p);
-        return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
+        return launch_check.result();
       }
     }
     if (!allow_dynamic_lds((const void*)moba_fwd_kernel<E, kTilesQueued, false>, kFwdLds, allowed[1])) return MOBA_ERR_LAUNCH;
@@ -700,7 +701,7 @@ static int launch_partials(const void* q, const void* k, const void* v, void* pa
     if (!allow_dynamic_lds((const void*)moba_fwd_kernel<E, kTilePerGroup, false>, kFwdLds, allowed[0])) return MOBA_ERR_LAUNCH;
     hipLaunchKernelGGL((moba_fwd_kernel<E, kTilePerGroup, false>), dim3((unsigned)-grid), dim3(512), kFwdLds, st, p);
   }
-  return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
+  return launch_check.result();
 }
 
 // hist_bound: any upper bound on the number of history tiles (floor(M/128) + F*H is one).
@@ -746,6 +747,7 @@ extern "C" int moba_fwd_partials(const void* q, const void* k, const void* v, vo
 
 extern "C" int moba_fwd_merge(const void* part_o, const float* part_lse, const int32_t* sel, void* out, float* lse,
                               int64_t S, int H, int D, int K, int dtype, void* stream) {
+  LaunchCheck launch_check;
   if (!part_o || !part_lse || !out || !lse || (K > 0 && !sel)) return MOBA_ERR_ARG;
   if (D != kHeadDim || (dtype != MOBA_DTYPE_BF16 && dtype != MOBA_DTYPE_F16)) return MOBA_ERR_UNSUPPORTED;
   if (S <= 0 || H <= 0 || K < 0 || ((uintptr_t)part_o & 15) || ((uintptr_t)out & 15)) return MOBA_ERR_ARG;
@@ -757,7 +759,7 @@ extern "C" int moba_fwd_merge(const void* part_o, const float* part_lse, const i
   else
     hipLaunchKernelGGL(moba_merge_kernel<Bf16>, grid, dim3(256), 0, (hipStream_t)stream, (const bf16*)part_o,
                        part_lse, sel, (bf16*)out, lse, rows, K + 1);
-  return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
+  return launch_check.result();
 }
 
 // Whole attention stage: partial attentions of every tile, then the merge.

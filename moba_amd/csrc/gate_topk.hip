@@ -167,6 +167,7 @@ using namespace moba;
 extern "C" int moba_gate_topk(const void* q, const void* kbar, const int32_t* cu_seqlens, const int32_t* seq_fbase,
                               int32_t* sel, float* scores_out, int64_t S, int H, int Hkv, int D, int nseq, int F,
                               int B, int K, const int64_t* strides, int dtype, void* stream) {
+  LaunchCheck launch_check;
   if (!q || !kbar || !cu_seqlens || !seq_fbase || !sel) return MOBA_ERR_ARG;
   if (Hkv <= 0 || H % Hkv != 0) return MOBA_ERR_ARG;
   if (dtype != MOBA_DTYPE_BF16 && dtype != MOBA_DTYPE_F16) return MOBA_ERR_UNSUPPORTED;
@@ -187,11 +188,12 @@ extern "C" int moba_gate_topk(const void* q, const void* kbar, const int32_t* cu
                        cu_seqlens, seq_fbase, sel, scores_out, (int)S, H, Hkv, nseq, F, B, K, qts, qhs)
   MOBA_DISPATCH_K(K, CALL)
 #undef CALL
-  return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
+  return launch_check.result();
 }
 
 extern "C" int moba_topk_from_scores(const float* scores, int32_t* sel, int64_t S, int H, int F, int K,
                                      void* stream) {
+  LaunchCheck launch_check;
   if (!scores || !sel || S <= 0 || H <= 0 || F <= 0 || K <= 0) return MOBA_ERR_ARG;
   const int64_t rows = S * H;
   dim3 grid((unsigned)((rows + 255) / 256));
@@ -200,5 +202,5 @@ extern "C" int moba_topk_from_scores(const float* scores, int32_t* sel, int64_t 
   hipLaunchKernelGGL(topk_from_scores_kernel<KM>, grid, dim3(256), 0, st, scores, sel, rows, F, K)
   MOBA_DISPATCH_K(K, CALL)
 #undef CALL
-  return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
+  return launch_check.result();
 }

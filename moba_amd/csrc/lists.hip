@@ -229,6 +229,7 @@ extern "C" int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, co
                                 int32_t* seg_off, int32_t* tile_off, int32_t* seg_dest, int32_t* tile_seg,
                                 int64_t S, int H, int K, int N, int F, int P, int cmax, int tile_rows,
                                 int64_t hist_bound, void* stream) {
+  LaunchCheck launch_check;
   if (!sel || !chunk_tok || !chunk_fb || !chunk_local || !pair_off || !cnt || !seg_off || !tile_off || !seg_dest ||
       !tile_seg)
     return MOBA_ERR_ARG;
@@ -261,13 +262,14 @@ extern "C" int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, co
   hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(1024), 0, st, tile_off, F * H);
   hipLaunchKernelGGL(lists_tile_seg_kernel, dim3((unsigned)((hist_bound + 255) / 256)), dim3(256), 0, st,
                      (const int*)tile_off, tile_seg, F * H, (int)hist_bound);
-  return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
+  return launch_check.result();
 }
 
 // The tile tables alone, for another number of rows per tile, from the list starts moba_build_lists wrote
 // (the forward and the backward kernels cut the same lists into tiles of different heights).
 extern "C" int moba_tile_tables(const int32_t* seg_off, int32_t* tile_off, int32_t* tile_seg, int H, int F,
                                 int tile_rows, int64_t hist_bound, void* stream) {
+  LaunchCheck launch_check;
   if (!seg_off || !tile_off || !tile_seg) return MOBA_ERR_ARG;
   if (H <= 0 || F <= 0 || tile_rows <= 0 || hist_bound <= 0 || hist_bound >= 0x7fffffffLL) return MOBA_ERR_ARG;
   if ((int64_t)F * H >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
@@ -277,5 +279,5 @@ extern "C" int moba_tile_tables(const int32_t* seg_off, int32_t* tile_off, int32
   hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(1024), 0, st, tile_off, F * H);
   hipLaunchKernelGGL(lists_tile_seg_kernel, dim3((unsigned)((hist_bound + 255) / 256)), dim3(256), 0, st,
                      (const int*)tile_off, tile_seg, F * H, (int)hist_bound);
-  return hipGetLastError() == hipSuccess ? MOBA_OK : MOBA_ERR_LAUNCH;
+  return launch_check.result();
 }

@@ -151,12 +151,14 @@ def build_lists(sel: torch.Tensor, plan: MobaPlan, tile_rows: int = FWD_TILE_ROW
     S, H, K = sel.shape
     dev = sel.device
     M = plan.pairs_per_head * H
-    cnt = torch.empty(plan.P * H + 1, dtype=torch.int32, device=dev)
-    seg_off = torch.empty(plan.F * H + 1, dtype=torch.int32, device=dev)
-    tile_off = torch.empty(plan.F * H + 1, dtype=torch.int32, device=dev)
-    seg_dest = torch.empty(max(M, 1), dtype=torch.int32, device=dev)
     bound = plan.hist_tile_bound(H, tile_rows)
-    tile_seg = torch.empty(bound, dtype=torch.int32, device=dev)
+    # one allocation for the five arrays (each start a multiple of 4 ints)
+    sizes = [plan.P * H + 1, plan.F * H + 1, plan.F * H + 1, max(M, 1), bound]
+    starts = [0]
+    for n in sizes:
+        starts.append(starts[-1] + (n + 3) // 4 * 4)
+    buf = torch.empty(starts[-1], dtype=torch.int32, device=dev)
+    cnt, seg_off, tile_off, seg_dest, tile_seg = (buf[a:a + n] for a, n in zip(starts, sizes))
     t = plan.tables
     _lib.check(lib.moba_build_lists(_ptr(sel), _ptr(t["chunk_tok"]), _ptr(t["chunk_fb"]), _ptr(t["chunk_local"]),
                                     _ptr(t["pair_off"]), _ptr(cnt), _ptr(seg_off), _ptr(tile_off), _ptr(seg_dest),
@@ -181,11 +183,16 @@ class StageTimer:
     """Optional per-stage device timing: events are recorded on the launch stream around
     each stage, so reading them never perturbs the launches themselves."""
 
-    def __init__(self):
+    def __init__(self, only=None):
+        """only: names of the stages to time (a pair of event records costs the host some tens of
+        microseconds, which shows in small problems); None = all."""
         self.events = {}
+        self.only = None if only is None else set(only)
 
     def span(self, name, device):
         timer = self
+        if self.only is not None and name not in self.only:
+            return _NoSpan()
 
         class _Span:
             def __enter__(self_inner):
@@ -230,14 +237,18 @@ def _forward(q, k, v, plan: MobaPlan, timer: Optional[StageTimer] = None, scale:
             sel = gate_topk(q, kbar, plan)
         with span("build_lists"):
             seg_off, tile_off, seg_dest, tile_seg = build_lists(sel, plan)
-    part_o = torch.empty((S * H * (K + 1), D), dtype=q.dtype, device=dev)
-    part_lse = torch.empty((S * H * (K + 1),), dtype=torch.float32, device=dev)
     out = torch.empty((S, H, D), dtype=q.dtype, device=dev)
     lse = torch.empty((S, H), dtype=torch.float32, device=dev)
+    # One allocation for the scratch of the attention stage: the per-slot partial outputs, their log-sum-exps,
     # the forward kernel's tile counters, then the list of tiles its fixed-reference softmax hands to the kernel
-    # that tracks the running maximum (count first; the call zeroes the counters and the count)
+    # that tracks the running maximum (count first; the call zeroes the counters and the count).
     bound = plan.hist_tile_bound(H, FWD_TILE_ROWS)
-    scratch = torch.empty(8 + 1 + bound + plan.fwd_self_tiles * H, dtype=torch.int32, device=dev)
+    rows = S * H * (K + 1)
+    n_ints = 8 + 1 + bound + plan.fwd_self_tiles * H
+    ws = torch.empty(rows * D * q.element_size() + rows * 4 + n_ints * 4, dtype=torch.uint8, device=dev)
+    part_o = ws[:rows * D * q.element_size()].view(q.dtype).view(rows, D)
+    part_lse = ws[rows * D * q.element_size():][:rows * 4].view(torch.float32)
+    scratch = ws[rows * D * q.element_size() + rows * 4:].view(torch.int32)
     queues, redo = scratch[:8], (scratch[8:] if FIXED_REFERENCE else None)
     with span("fwd_partials"):
         _lib.check(lib.moba_fwd_partials(_ptr(q), _ptr(k), _ptr(v), _ptr(part_o), _ptr(part_lse), _ptr(seg_off),

@@ -93,3 +93,59 @@ def test_plan_accepts_inference_tensors():
         assert make_plan(cu, 32, 3).cu == [0, 120, 260]
         assert make_plan(cu, 32, 3, host_lengths=[0, 120, 260]).cu == [0, 120, 260]
     assert make_plan(cu, 32, 3).cu == [0, 120, 260]      # and outside the mode as well
+
+
+@pytest.mark.parametrize("seed", range(30))
+def test_c_planner_equals_python_planner(seed):
+    """moba_plan / moba_plan_fill / moba_plan_sizes (host functions of the C ABI, for hosts that are not Python)
+    against the numpy planner: same counts, same tables, same buffer sizes."""
+    import ctypes
+    from moba_amd import _lib
+    lib = _lib.load()
+    rng = np.random.default_rng(1000 + seed)
+    cu = rand_cu(rng, int(rng.integers(1, 7)), 1, 900)
+    B = int(rng.integers(1, 300))
+    topk = int(rng.integers(1, 7))
+    if seed == 0:
+        cu, B, topk = [0, 131072], 4096, 12
+    plan = make_plan(cu, B, topk)
+    cu_arr = (ctypes.c_int32 * len(cu))(*cu)
+    ps, ps2 = _lib.PlanStruct(), _lib.PlanStruct()
+    assert lib.moba_plan(cu_arr, len(cu) - 1, B, topk, ctypes.byref(ps)) == 0
+    tab = (ctypes.c_int32 * max(1, ps.table_ints))()
+    assert lib.moba_plan_fill(cu_arr, len(cu) - 1, B, topk, ctypes.byref(ps2), tab) == 0
+    assert bytes(ps) == bytes(ps2)
+    tab = np.frombuffer(tab, dtype=np.int32)
+    assert (ps.S, ps.nseq, ps.N, ps.F, ps.K, ps.P, ps.cmax, bool(ps.fallback)) == \
+        (plan.S, plan.nseq, plan.N, plan.F, plan.K, plan.P, plan.cmax, plan.fallback)
+    assert (ps.pairs_per_head, ps.fwd_self_tiles, ps.bwd_self_tiles) == (plan.pairs_per_head, plan.fwd_self_tiles, plan.self_tiles)
+    assert (ps.fwd_tile_rows, ps.bwd_tile_rows) == (FWD_TILE_ROWS, TILE_ROWS)
+    assert ps.flops_per_head_per_dim == plan.flops_per_head
+    seen = 0
+    for name, arr in plan.host.items():
+        off = getattr(ps, "off_" + name)
+        assert off >= 0 and np.array_equal(tab[off:off + arr.size], arr.astype(np.int32)), name
+        seen += arr.size
+    assert seen == ps.table_ints
+    if plan.fallback:
+        assert ps.off_fchunk_tok == ps.off_pair_off == ps.off_chunk_fid == -1
+    H, Hkv = 6, 3
+    sz = _lib.SizesStruct()
+    assert lib.moba_plan_sizes(ctypes.byref(ps), H, Hkv, 128, ctypes.byref(sz)) == 0
+    assert sz.fwd_hist_bound == plan.hist_tile_bound(H, FWD_TILE_ROWS) and sz.bwd_hist_bound == plan.hist_tile_bound(H, TILE_ROWS)
+    assert sz.sel_ints == plan.S * H * plan.K and sz.cnt_ints == plan.P * H + 1 and sz.seg_off_ints == plan.F * H + 1
+    assert sz.seg_dest_ints == max(1, plan.pairs_per_head * H) and sz.part_rows == plan.S * H * (plan.K + 1)
+    assert sz.redo_ints == 1 + sz.fwd_hist_bound + plan.fwd_self_tiles * H and sz.kbar_elems == plan.F * Hkv * 128
+    assert sz.chunk_mean_workspace_bytes == (lib.moba_chunk_mean_workspace_bytes(Hkv, 128, plan.F, B) if plan.F else 0)
+
+
+def test_c_planner_rejects_bad_input():
+    import ctypes
+    from moba_amd import _lib
+    lib = _lib.load()
+    ps = _lib.PlanStruct()
+    for cu in ([0, 5, 5, 9], [1, 5], [0, 4, 3]):
+        arr = (ctypes.c_int32 * len(cu))(*cu)
+        assert lib.moba_plan(arr, len(cu) - 1, 4, 3, ctypes.byref(ps)) == -1
+    arr = (ctypes.c_int32 * 2)(0, 8)
+    assert lib.moba_plan(arr, 1, 0, 3, ctypes.byref(ps)) == -1 and lib.moba_plan(arr, 1, 4, 0, ctypes.byref(ps)) == -1
