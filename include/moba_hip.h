@@ -29,10 +29,14 @@
  * history chunks per (token, head), M = number of selected (token, head, chunk)
  * triples, P = number of (filtered chunk, later chunk of the same sequence) pairs.
  *
- * `strides` (a host pointer, read during the call) describes q, k and v where an entry point
- * takes it: {q token stride, q head stride, k/v token stride, k/v head stride} in elements; the
- * D elements of one (token, head) are contiguous, k and v share their strides, every stride is a
- * positive multiple of 8 and the k/v token stride is at most 2^23.  NULL means packed
+ * `strides` (a host pointer to seven int64, read during the call) describes q, k and v where an entry
+ * point takes it: {q token stride, q head stride, k/v token stride, k/v head stride, rows per batch
+ * entry, q batch stride, k/v batch stride} in elements; the D elements of one (token, head) are
+ * contiguous, k and v share their strides, every stride is a positive multiple of 8 and the k/v token
+ * stride is at most 2^23.  With rows per batch entry R > 0, packed token t lies in batch entry t / R at
+ * position t % R (every sequence must then lie inside one batch entry): this is how a
+ * [batch, heads, seqlen, D] tensor of the transformers layout is read without the transposing copy of
+ * moba/wrapper.py:7-15; R = 0 (and batch strides 0): one affine range of tokens.  NULL means packed
  * [S,H,D] / [S,Hkv,D].  This is what lets a slice of a fused qkv projection or a
  * [heads, tokens, D] cache be read in place, as flash-attn reads them for the reference
  * (moba/moba_efficient.py:89-128 passes such views on unchanged).  Outputs are always packed.
@@ -49,7 +53,7 @@ extern "C" {
 
 enum { MOBA_DTYPE_BF16 = 0, MOBA_DTYPE_F16 = 1 };
 
-#define MOBA_ABI_VERSION 105 /* the signatures below; moba_version() returns the number the library was built with */
+#define MOBA_ABI_VERSION 106 /* the signatures below; moba_version() returns the number the library was built with */
 int moba_version(void);
 const char* moba_strerror(int code);
 

@@ -67,7 +67,7 @@ class SizesStruct(ctypes.Structure):
     _fields_ = [(n, c_int64) for n in ("kbar_elems", "chunk_mean_workspace_bytes", "sel_ints", "cnt_ints", "seg_off_ints",
                                        "seg_dest_ints", "fwd_hist_bound", "bwd_hist_bound", "part_rows", "redo_ints",
                                        "lse_floats", "delta_floats")]
-ABI_VERSION = 105  # MOBA_ABI_VERSION of include/moba_hip.h, the signatures above
+ABI_VERSION = 106  # MOBA_ABI_VERSION of include/moba_hip.h, the signatures above
 DTYPE_BF16, DTYPE_F16 = 0, 1
 
 

@@ -33,13 +33,32 @@ struct TileTables {
   // byte strides of q[token][head][:] and of k, v[token][kv head][:] (k and v share theirs); the
   // 128 elements of a (token, head) are contiguous
   int64_t q_tok_b, q_head_b, kv_tok_b, kv_head_b;
+  // batched layouts ([batch, heads, tokens, dim] tensors seen as packed tokens): token t lies in batch entry
+  // t / batch_rows at position t % batch_rows; batch_rows = 0 for one affine range of tokens
+  int batch_rows;
+  int64_t q_batch_b, kv_batch_b;
 };
 
-// strides: {q token, q head, k/v token, k/v head} in elements, or null for packed [S, H, 128] /
+// byte offset of the row of token `tok` (without the head term) in q and in k, v
+__device__ __forceinline__ int64_t q_tok_bytes(const TileTables& t, int tok) {
+  if (t.batch_rows == 0) return (int64_t)tok * t.q_tok_b;
+  const int b = tok / t.batch_rows;
+  return (int64_t)b * t.q_batch_b + (int64_t)(tok - b * t.batch_rows) * t.q_tok_b;
+}
+__device__ __forceinline__ int64_t kv_tok_bytes(const TileTables& t, int tok) {
+  if (t.batch_rows == 0) return (int64_t)tok * t.kv_tok_b;
+  const int b = tok / t.batch_rows;
+  return (int64_t)b * t.kv_batch_b + (int64_t)(tok - b * t.batch_rows) * t.kv_tok_b;
+}
+
+// strides: {q token, q head, k/v token, k/v head, rows per batch entry, q batch, k/v batch} in elements
+// (seven entries; the last three are 0 for one affine range of tokens), or null for packed [S, H, 128] /
 // [S, Hkv, 128] tensors.  Returns false for strides the kernels cannot address: not multiples of
 // 8 elements (16-byte accesses), not positive, or a key/value token stride whose 64-row tile
 // offsets leave 31 bits.
+constexpr int kStrideEntries = 7;
 inline bool set_layout(TileTables& t, const int64_t* strides) {
+  t.batch_rows = 0; t.q_batch_b = 0; t.kv_batch_b = 0;
   if (!strides) {
     t.q_tok_b = (int64_t)t.H * kHeadDim * 2; t.q_head_b = kHeadDim * 2;
     t.kv_tok_b = (int64_t)t.Hkv * kHeadDim * 2; t.kv_head_b = kHeadDim * 2;
@@ -50,6 +69,11 @@ inline bool set_layout(TileTables& t, const int64_t* strides) {
   if (strides[2] > (1 << 23)) return false;
   t.q_tok_b = strides[0] * 2; t.q_head_b = strides[1] * 2;
   t.kv_tok_b = strides[2] * 2; t.kv_head_b = strides[3] * 2;
+  if (strides[4] != 0) {
+    if (strides[4] < 0 || strides[4] > 0x7fffffffLL || strides[5] <= 0 || strides[6] <= 0 || (strides[5] & 7) || (strides[6] & 7))
+      return false;
+    t.batch_rows = (int)strides[4]; t.q_batch_b = strides[5] * 2; t.kv_batch_b = strides[6] * 2;
+  }
   return true;
 }
 

@@ -121,7 +121,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams<E> p) {
   elem8 bq[8], bdo[8];
   {
     const int64_t off = ((int64_t)t.tok * H + h) * kHeadDim + 8 * hh;
-    const elem* qsrc = reinterpret_cast<const elem*>((const char*)p.q + t.tok * p.t.q_tok_b + h * p.t.q_head_b) + 8 * hh;
+    const elem* qsrc = reinterpret_cast<const elem*>((const char*)p.q + q_tok_bytes(p.t, t.tok) + h * p.t.q_head_b) + 8 * hh;
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
       bq[ks] = *reinterpret_cast<const elem8*>(qsrc + 16 * ks);
@@ -142,13 +142,14 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams<E> p) {
     const int key = 4 * (4 * i + wave_u) + ld_kin;
     ld_off[i] = (uint32_t)(key * row_bytes + sw_col16(key, ld_pc) * 16);
   }
-  const char* k_head = (const char*)p.k + (int64_t)kv_tok0 * row_bytes + hkv * p.t.kv_head_b;
-  const char* v_head = (const char*)p.v + (int64_t)kv_tok0 * row_bytes + hkv * p.t.kv_head_b;
+  const int64_t kv_off = kv_tok_bytes(p.t, kv_tok0) + hkv * p.t.kv_head_b;
+  const char* k_head = (const char*)p.k + kv_off;
+  const char* v_head = (const char*)p.v + kv_off;
   auto issue_tile = [&](int kt, int buf) __attribute__((always_inline)) {
     const uint32_t kdst = lds_base + buf * kTileBytes;
     const uint32_t vdst = lds_base + (2 + buf) * kTileBytes;
     const int key0 = kt * TN;
-    const bool full = (key0 + TN <= nkeys) && (kv_tok0 + key0 + TN <= p.t.S);
+    const bool full = key0 + TN <= nkeys;  // (the keys of a tile all belong to one chunk, hence to one sequence)
     if (full) {  // uniform tile base in SGPRs + constant per-lane offsets: no address arithmetic
       const char* kb_ = k_head + (int64_t)key0 * row_bytes;
       const char* vb_ = v_head + (int64_t)key0 * row_bytes;
@@ -163,10 +164,10 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams<E> p) {
         const int slab = 4 * i + wave_u;
         const int key = 4 * slab + ld_kin;
         const int c16 = sw_col16(key, ld_pc);
-        const int64_t tk = min((int64_t)kv_tok0 + key0 + key, (int64_t)p.t.S - 1);
-        const int64_t off = tk * row_bytes + hkv * p.t.kv_head_b + c16 * 16;
-        async_copy16((const char*)p.k + off, kdst + slab * 1024);
-        async_copy16((const char*)p.v + off, vdst + slab * 1024);
+        // (keys past the end of the range: the last key again -- their rows are cleared after they land)
+        const int64_t off = (int64_t)min(key0 + key, nkeys - 1) * row_bytes + c16 * 16;
+        async_copy16(k_head + off, kdst + slab * 1024);
+        async_copy16(v_head + off, vdst + slab * 1024);
       }
     }
   };
@@ -434,7 +435,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
   // ---- K^T and V^T operands of this lane's key: [16*ks + 8*hh .. +7] ----
   elem8 bk[8], bv[8];
   {
-    const int64_t off = (c0 + min(mykey, len - 1)) * p.t.kv_tok_b + hkv * p.t.kv_head_b + 16 * hh;  // bytes
+    const int64_t off = kv_tok_bytes(p.t, c0) + min(mykey, len - 1) * p.t.kv_tok_b + hkv * p.t.kv_head_b + 16 * hh;  // bytes
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
       bk[ks] = *reinterpret_cast<const elem8*>((const char*)p.k + off + 32 * ks);
@@ -479,7 +480,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
     const int row = 4 * slab + ld_rin;
     const int c16 = sw_col16(row, ld_pc);
     if ((g & 1) == 0)
-      async_copy16((const char*)p.q + (toks[i] * p.t.q_tok_b + h * p.t.q_head_b + c16 * 16), qdst + slab * 1024);
+      async_copy16((const char*)p.q + (q_tok_bytes(p.t, toks[i]) + h * p.t.q_head_b + c16 * 16), qdst + slab * 1024);
     else
       async_copy16((const char*)p.dout + (((int64_t)toks[i] * H + h) * kHeadDim + c16 * 8) * 2,
                    qdst + TQ * kHeadDim * 2 + slab * 1024);

@@ -19,7 +19,7 @@ template <class E>
 __global__ __launch_bounds__(256) void chunk_mean_partial_kernel(
     const typename E::elem* __restrict__ k, const int* __restrict__ fchunk_tok, double* __restrict__ partial,
     int HD8 /* H*D/8 */, int D8 /* D/8 */, int B, int nsplit, int tok_per_split, int64_t row_stride,
-    int64_t head_stride) {
+    int64_t head_stride, int batch_rows, int64_t batch_stride) {
   MOBA_ELEM_TYPES(E)
   const int col = blockIdx.z * 256 + threadIdx.x;
   if (col >= HD8) return;
@@ -28,7 +28,11 @@ __global__ __launch_bounds__(256) void chunk_mean_partial_kernel(
   const int t0 = split * tok_per_split;
   const int t1 = min(B, t0 + tok_per_split);
   const int head = col / D8;
-  const elem* src = k + ((int64_t)fchunk_tok[f] + t0) * row_stride + head * head_stride + (col - head * D8) * 8;
+  // (a chunk lies inside one sequence, hence inside one batch entry of a batched layout)
+  const int tok0 = fchunk_tok[f];
+  const int be = batch_rows ? tok0 / batch_rows : 0;
+  const elem* src = k + be * batch_stride + ((int64_t)(tok0 - be * batch_rows) + t0) * row_stride + head * head_stride +
+                    (col - head * D8) * 8;
   double acc[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.0;
@@ -100,7 +104,8 @@ extern "C" size_t moba_chunk_mean_workspace_bytes(int H, int D, int F, int B) {
 }
 
 static int launch_chunk_mean(const void* k, const int32_t* fchunk_tok, void* kbar, double* partial, int H, int D,
-                             int F, int B, int nsplit, int64_t kts, int64_t khs, int dtype, hipStream_t st) {
+                             int F, int B, int nsplit, int64_t kts, int64_t khs, int batch_rows, int64_t kbs, int dtype,
+                             hipStream_t st) {
   LaunchCheck launch_check;
   const int HD8 = H * D / 8;
   const int tps = (B + nsplit - 1) / nsplit;
@@ -109,29 +114,34 @@ static int launch_chunk_mean(const void* k, const int32_t* fchunk_tok, void* kba
   const dim3 fgrid((unsigned)((n + 255) / 256));
   if (dtype == MOBA_DTYPE_F16) {
     hipLaunchKernelGGL(chunk_mean_partial_kernel<F16>, grid, dim3(256), 0, st, (const f16*)k, fchunk_tok, partial,
-                       HD8, D / 8, B, nsplit, tps, kts, khs);
+                       HD8, D / 8, B, nsplit, tps, kts, khs, batch_rows, kbs);
     hipLaunchKernelGGL(chunk_mean_finish_kernel<F16>, fgrid, dim3(256), 0, st, (const double*)partial, (f16*)kbar,
                        HD8, B, nsplit, F);
   } else {
     hipLaunchKernelGGL(chunk_mean_partial_kernel<Bf16>, grid, dim3(256), 0, st, (const bf16*)k, fchunk_tok, partial,
-                       HD8, D / 8, B, nsplit, tps, kts, khs);
+                       HD8, D / 8, B, nsplit, tps, kts, khs, batch_rows, kbs);
     hipLaunchKernelGGL(chunk_mean_finish_kernel<Bf16>, fgrid, dim3(256), 0, st, (const double*)partial, (bf16*)kbar,
                        HD8, B, nsplit, F);
   }
   return launch_check.result();
 }
 
-// argument checks shared by the two entry points; kts, khs receive the key token and head strides (elements)
+// argument checks shared by the two entry points; kts, khs, kbr, kbs receive the key token and head strides, the
+// rows per batch entry and the batch stride (elements)
 static int check_chunk_mean_args(const void* k, const int32_t* fchunk_tok, void* kbar, int64_t S, int H, int D, int F,
-                                 int B, const int64_t* strides, int dtype, int64_t& kts, int64_t& khs) {
+                                 int B, const int64_t* strides, int dtype, int64_t& kts, int64_t& khs, int& kbr,
+                                 int64_t& kbs) {
   if (dtype != MOBA_DTYPE_BF16 && dtype != MOBA_DTYPE_F16) return MOBA_ERR_UNSUPPORTED;
   if (!k || !fchunk_tok || !kbar || S <= 0 || H <= 0 || D <= 0 || F < 0 || B <= 0) return MOBA_ERR_ARG;
   if ((H * D) % 8 != 0 || ((uintptr_t)k & 15) || ((uintptr_t)kbar & 15)) return MOBA_ERR_ARG;
   if (D % 8 != 0) return MOBA_ERR_ARG;
-  // strides (elements): {., ., k token, k head}; null = packed [S, H, D]
+  // strides (elements): {., ., k token, k head, rows per batch entry, ., k batch}; null = packed [S, H, D]
   kts = strides ? strides[2] : (int64_t)H * D;
   khs = strides ? strides[3] : D;
+  kbr = strides ? (int)strides[4] : 0;
+  kbs = strides ? strides[6] : 0;
   if (kts <= 0 || khs <= 0 || (kts & 7) || (khs & 7)) return MOBA_ERR_ARG;
+  if (kbr < 0 || (kbr > 0 && (kbs <= 0 || (kbs & 7)))) return MOBA_ERR_ARG;
   return MOBA_OK;
 }
 
@@ -139,12 +149,13 @@ extern "C" int moba_chunk_mean(const void* k, const int32_t* fchunk_tok, void* k
                                int64_t S, int H, int D, int F, int B, const int64_t* strides, int dtype,
                                void* stream) {
   if (F == 0) return MOBA_OK;
-  int64_t kts = 0, khs = 0;
-  const int rc = check_chunk_mean_args(k, fchunk_tok, kbar, S, H, D, F, B, strides, dtype, kts, khs);
+  int64_t kts = 0, khs = 0, kbs = 0;
+  int kbr = 0;
+  const int rc = check_chunk_mean_args(k, fchunk_tok, kbar, S, H, D, F, B, strides, dtype, kts, khs, kbr, kbs);
   if (rc != MOBA_OK) return rc;
   if (!workspace || ((uintptr_t)workspace & 7)) return MOBA_ERR_ARG;
   return launch_chunk_mean(k, fchunk_tok, kbar, (double*)workspace, H, D, F, B, pick_nsplit(H * D / 8, F, B), kts, khs,
-                           dtype, (hipStream_t)stream);
+                           kbr, kbs, dtype, (hipStream_t)stream);
 }
 
 // ---- the same stage for callers that cannot allocate: the partial sums live in a fixed array of the library ----
@@ -174,8 +185,9 @@ extern "C" size_t moba_chunk_mean_static_capacity(void) { return kStaticPartialB
 extern "C" int moba_chunk_mean_static(const void* k, const int32_t* fchunk_tok, void* kbar, int64_t S, int H, int D,
                                       int F, int B, const int64_t* strides, int dtype, void* stream) {
   if (F == 0) return MOBA_OK;
-  int64_t kts = 0, khs = 0;
-  const int rc = check_chunk_mean_args(k, fchunk_tok, kbar, S, H, D, F, B, strides, dtype, kts, khs);
+  int64_t kts = 0, khs = 0, kbs = 0;
+  int kbr = 0;
+  const int rc = check_chunk_mean_args(k, fchunk_tok, kbar, S, H, D, F, B, strides, dtype, kts, khs, kbr, kbs);
   if (rc != MOBA_OK) return rc;
   // The sums are exact in fp64, so the mean does not depend on the number of token splits: take the
   // widest split (up to the one moba_chunk_mean would use) whose partial sums fit the array.
@@ -186,5 +198,5 @@ extern "C" int moba_chunk_mean_static(const void* k, const int32_t* fchunk_tok, 
   while (nsplit > 1 && per_split * nsplit > kStaticPartialBytes) nsplit /= 2;
   double* partial = static_partials();
   if (!partial) return MOBA_ERR_LAUNCH;
-  return launch_chunk_mean(k, fchunk_tok, kbar, partial, H, D, F, B, nsplit, kts, khs, dtype, (hipStream_t)stream);
+  return launch_chunk_mean(k, fchunk_tok, kbar, partial, H, D, F, B, nsplit, kts, khs, kbr, kbs, dtype, (hipStream_t)stream);
 }

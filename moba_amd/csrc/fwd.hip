@@ -125,9 +125,9 @@ __global__ __launch_bounds__(512, 2) void moba_fwd_kernel(const FwdParams<E> p) 
   }
   const char* k_head = nullptr;  // key 0 of the current tile's key range, this tile's key/value head
   const char* v_head = nullptr;
-  auto issue = [&](const char* head, const char* tensor, int kt, uint32_t dst) __attribute__((always_inline)) {
+  auto issue = [&](const char* head, int kt, uint32_t dst) __attribute__((always_inline)) {
     const int key0 = kt * TN;
-    const bool full = (key0 + TN <= nkeys) && (kv_tok0 + key0 + TN <= p.t.S);
+    const bool full = key0 + TN <= nkeys;  // (the keys of a tile all belong to one chunk, hence to one sequence)
     if (full) {  // uniform tile base in SGPRs + constant per-lane offsets: no address arithmetic
       const char* base = head + (int64_t)key0 * row_bytes;
 #pragma unroll
@@ -141,13 +141,13 @@ __global__ __launch_bounds__(512, 2) void moba_fwd_kernel(const FwdParams<E> p) 
       for (int i = 0; i < 2; ++i) {
         const int slab = 8 * i + wave_u;
         const int key = 4 * slab + kin;
-        const int64_t tk = min((int64_t)kv_tok0 + key0 + key, (int64_t)p.t.S - 1);
-        async_copy16(tensor + tk * row_bytes + hkv * p.t.kv_head_b + sw_col16(key, ld_pc) * 16, dst + slab * 1024);
+        // (keys past the end of the range: the last key again -- their scores are masked, their V rows cleared)
+        async_copy16(head + (int64_t)min(key0 + key, nkeys - 1) * row_bytes + sw_col16(key, ld_pc) * 16, dst + slab * 1024);
       }
     }
   };
-  auto issue_k = [&](int kt, int stage) __attribute__((always_inline)) { issue(k_head, (const char*)p.k, kt, lds_base + stage * kTileBytes); };
-  auto issue_v = [&](int kt, int stage) __attribute__((always_inline)) { issue(v_head, (const char*)p.v, kt, lds_base + kFwdVBase + stage * kTileBytes); };
+  auto issue_k = [&](int kt, int stage) __attribute__((always_inline)) { issue(k_head, kt, lds_base + stage * kTileBytes); };
+  auto issue_v = [&](int kt, int stage) __attribute__((always_inline)) { issue(v_head, kt, lds_base + kFwdVBase + stage * kTileBytes); };
   // rows of V past the end of the key range must not reach the MFMA (0 * NaN): clear them
   auto scrub_v = [&](int kt, int stage) __attribute__((always_inline)) {
     const int key0 = kt * TN;
@@ -321,8 +321,9 @@ __global__ __launch_bounds__(512, 2) void moba_fwd_kernel(const FwdParams<E> p) 
       // and V tiles (global -> LDS)
       h = t.h; nkeys = t.nkeys; kv_tok0 = t.kv_tok0;
       hkv = h / pn.t.rep;  // key/value head of this query head
-      k_head = (const char*)pn.k + (int64_t)kv_tok0 * row_bytes + hkv * pn.t.kv_head_b;
-      v_head = (const char*)pn.v + (int64_t)kv_tok0 * row_bytes + hkv * pn.t.kv_head_b;
+      const int64_t kv_off = kv_tok_bytes(pn.t, kv_tok0) + hkv * pn.t.kv_head_b;
+      k_head = (const char*)pn.k + kv_off;
+      v_head = (const char*)pn.v + kv_off;
       nkt = (nkeys + TN - 1) / TN;
       rot = t.rot % nkt;
       issue_k(key_tile(0), 0);
@@ -339,7 +340,7 @@ __global__ __launch_bounds__(512, 2) void moba_fwd_kernel(const FwdParams<E> p) 
       limit = t.limit;
       min_limit = __builtin_amdgcn_readfirstlane(t.wave_min_limit);
       row_valid = er < t.row_count;
-      const elem* src = reinterpret_cast<const elem*>((const char*)pn.q + t.tok * pn.t.q_tok_b + h * pn.t.q_head_b) + 8 * (tx >> 5 & 1);
+      const elem* src = reinterpret_cast<const elem*>((const char*)pn.q + q_tok_bytes(pn.t, t.tok) + h * pn.t.q_head_b) + 8 * (tx >> 5 & 1);
 #pragma unroll
       for (int ks = 0; ks < 8; ++ks) bq[ks] = *reinterpret_cast<const elem8*>(src + 16 * ks);
     }

@@ -55,7 +55,8 @@ template <class E, int KMAX>
 __global__ __launch_bounds__(256) void gate_topk_kernel(
     const typename E::elem* __restrict__ q, const typename E::elem* __restrict__ kbar, const int* __restrict__ cu_seqlens,
     const int* __restrict__ seq_fbase, int* __restrict__ sel, float* __restrict__ scores_out,
-    int S, int H, int Hkv, int nseq, int F, int B, int K, int64_t q_tok_stride, int64_t q_head_stride) {
+    int S, int H, int Hkv, int nseq, int F, int B, int K, int64_t q_tok_stride, int64_t q_head_stride,
+    int batch_rows, int64_t q_batch_stride) {
   MOBA_ELEM_TYPES(E)
   __shared__ float sc[4][64][33];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -91,7 +92,8 @@ __global__ __launch_bounds__(256) void gate_topk_kernel(
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) {
       const int tok = min(tok0 + 32 * qb + n, S - 1);
-      const elem* src = q + (tok * q_tok_stride + hc * q_head_stride) + 8 * hh;
+      const int be = batch_rows ? tok / batch_rows : 0;  // batch entry of the token in a batched layout
+      const elem* src = q + (be * q_batch_stride + (tok - be * batch_rows) * q_tok_stride + hc * q_head_stride) + 8 * hh;
 #pragma unroll
       for (int ks = 0; ks < 8; ++ks) bq[qb][ks] = *reinterpret_cast<const elem8*>(src + 16 * ks);
     }
@@ -174,18 +176,21 @@ extern "C" int moba_gate_topk(const void* q, const void* kbar, const int32_t* cu
   if (S <= 0 || S > 0x7fffffff - 64 || H <= 0 || nseq <= 0 || F <= 0 || B <= 0 || K <= 0) return MOBA_ERR_ARG;
   if (D != kHeadDim) return MOBA_ERR_UNSUPPORTED;
   if (((uintptr_t)q & 15) || ((uintptr_t)kbar & 15)) return MOBA_ERR_ARG;
-  // strides (elements): {q token, q head, ...}; null = packed [S, H, 128]
+  // strides (elements): {q token, q head, ., ., rows per batch entry, q batch, .}; null = packed [S, H, 128]
   const int64_t qts = strides ? strides[0] : (int64_t)H * kHeadDim, qhs = strides ? strides[1] : kHeadDim;
+  const int qbr = strides ? (int)strides[4] : 0;
+  const int64_t qbs = strides ? strides[5] : 0;
   if (qts <= 0 || qhs <= 0 || (qts & 7) || (qhs & 7)) return MOBA_ERR_ARG;
+  if (qbr < 0 || (qbr > 0 && (qbs <= 0 || (qbs & 7)))) return MOBA_ERR_ARG;
   dim3 grid((unsigned)((S + 63) / 64), (unsigned)((H + 3) / 4));
   hipStream_t st = (hipStream_t)stream;
 #define CALL(KM)                                                                                               \
   if (dtype == MOBA_DTYPE_F16)                                                                                 \
     hipLaunchKernelGGL((gate_topk_kernel<F16, KM>), grid, dim3(256), 0, st, (const f16*)q, (const f16*)kbar,   \
-                       cu_seqlens, seq_fbase, sel, scores_out, (int)S, H, Hkv, nseq, F, B, K, qts, qhs);            \
+                       cu_seqlens, seq_fbase, sel, scores_out, (int)S, H, Hkv, nseq, F, B, K, qts, qhs, qbr, qbs);  \
   else                                                                                                         \
     hipLaunchKernelGGL((gate_topk_kernel<Bf16, KM>), grid, dim3(256), 0, st, (const bf16*)q, (const bf16*)kbar, \
-                       cu_seqlens, seq_fbase, sel, scores_out, (int)S, H, Hkv, nseq, F, B, K, qts, qhs)
+                       cu_seqlens, seq_fbase, sel, scores_out, (int)S, H, Hkv, nseq, F, B, K, qts, qhs, qbr, qbs)
   MOBA_DISPATCH_K(K, CALL)
 #undef CALL
   return launch_check.result();

@@ -49,11 +49,30 @@ def _aligned(t: torch.Tensor) -> torch.Tensor:
     return t if t.data_ptr() % 16 == 0 else t.clone()
 
 
+def _dims(t: torch.Tensor):
+    """(tokens, heads, head_dim) as the kernels see a [tokens, heads, head_dim] tensor or a batched
+    [batch, heads, tokens, head_dim] one (the transformers layout: batch * tokens packed tokens)."""
+    if t.dim() == 4:
+        b, h, l, d = t.shape
+        return b * l, h, d
+    return tuple(t.shape)
+
+
 def _row_strides(t: torch.Tensor):
-    """(token stride, head stride) in elements of a [tokens, heads, head_dim] tensor; the stride of a
-    dimension of size 1 means nothing and is replaced by the packed one."""
+    """(token stride, head stride) in elements; the stride of a dimension of size 1 means nothing and is
+    replaced by the packed one."""
+    if t.dim() == 4:
+        b, H, S, D = t.shape
+        return (t.stride(2) if S > 1 else D), (t.stride(1) if H > 1 else S * D)
     S, H, D = t.shape
     return (t.stride(0) if S > 1 else H * D), (t.stride(1) if H > 1 else D)
+
+
+def _batch_stride(t: torch.Tensor):
+    """(rows per batch entry, batch stride in elements) of a batched tensor; (0, 0) otherwise."""
+    if t.dim() != 4 or t.shape[0] == 1:
+        return 0, 0
+    return t.shape[2], t.stride(0)
 
 
 def _addressable(t: torch.Tensor) -> bool:
@@ -62,8 +81,9 @@ def _addressable(t: torch.Tensor) -> bool:
     [heads, tokens, head_dim] cache seen as [tokens, heads, head_dim], ...), as flash-attn does for
     the reference (moba/moba_efficient.py:89-128 hands such views straight to it)."""
     ts, hs = _row_strides(t)
-    return (t.stride(2) == 1 and ts > 0 and hs > 0 and ts % 8 == 0 and hs % 8 == 0 and ts <= 1 << 23
-            and t.data_ptr() % 16 == 0)
+    rows, bs = _batch_stride(t)
+    return (t.stride(-1) == 1 and ts > 0 and hs > 0 and ts % 8 == 0 and hs % 8 == 0 and ts <= 1 << 23
+            and (rows == 0 or (bs > 0 and bs % 8 == 0)) and t.data_ptr() % 16 == 0)
 
 
 def _in_place(q, k, v):
@@ -77,10 +97,15 @@ def _in_place(q, k, v):
 
 
 def _strides(q: Optional[torch.Tensor], k: Optional[torch.Tensor]):
-    """The strides argument of the C ABI: {q token, q head, k/v token, k/v head} in elements."""
+    """The strides argument of the C ABI: {q token, q head, k/v token, k/v head, rows per batch entry,
+    q batch, k/v batch} in elements (the last three 0 unless q, k are batched 4-D tensors)."""
     qs = _row_strides(q) if q is not None else (HEAD_DIM, HEAD_DIM)
     ks = _row_strides(k) if k is not None else (HEAD_DIM, HEAD_DIM)
-    return (ctypes.c_int64 * 4)(qs[0], qs[1], ks[0], ks[1])
+    qr, qb = _batch_stride(q) if q is not None else (0, 0)
+    kr, kb = _batch_stride(k) if k is not None else (0, 0)
+    rows = qr or kr
+    # (a tensor given alone stands for both: the entry point reads only its own entries)
+    return (ctypes.c_int64 * 7)(qs[0], qs[1], ks[0], ks[1], rows, qb or kb if rows else 0, kb or qb if rows else 0)
 
 
 def _check_qkv(q, k, v, gqa=False):
@@ -103,7 +128,7 @@ def _check_qkv(q, k, v, gqa=False):
 def chunk_mean(k: torch.Tensor, plan: MobaPlan) -> torch.Tensor:
     """kbar [F, H, D] in k's dtype: mean of K over every filtered chunk (exact sum, rounded once)."""
     lib = _lib.load()
-    S, H, D = k.shape
+    S, H, D = _dims(k)
     if not _addressable(k):
         k = _aligned(k)
     kbar = torch.empty((plan.F, H, D), dtype=k.dtype, device=k.device)
@@ -119,7 +144,7 @@ def gate_topk(q: torch.Tensor, kbar: torch.Tensor, plan: MobaPlan, return_scores
     """sel [S, H, K] int32: selected filtered-chunk ids per (token, head), -1 padded.
     kbar may have fewer heads than q (grouped-query attention)."""
     lib = _lib.load()
-    S, H, D = q.shape
+    S, H, D = _dims(q)
     Hkv = kbar.shape[1]
     if not _addressable(q):
         q = _aligned(q)
@@ -222,8 +247,10 @@ class _NoSpan:
 
 
 def _forward(q, k, v, plan: MobaPlan, timer: Optional[StageTimer] = None, scale: float = 0.0):
+    """q, k, v: [tokens, heads, 128], or batched [batch, heads, tokens, 128] (read in place, see _dims)."""
     lib = _lib.load()
-    S, H, D = q.shape
+    S, H, D = _dims(q)
+    Hkv = _dims(k)[1]
     dev = q.device
     K = plan.K
     t = plan.tables
@@ -254,7 +281,7 @@ def _forward(q, k, v, plan: MobaPlan, timer: Optional[StageTimer] = None, scale:
         _lib.check(lib.moba_fwd_partials(_ptr(q), _ptr(k), _ptr(v), _ptr(part_o), _ptr(part_lse), _ptr(seg_off),
                                          _ptr(tile_off), _ptr(seg_dest), _ptr(t.get("fchunk_tok")),
                                          _ptr(t["chunk_tok"]), _ptr(t["fwd_self_tile_prefix"]), _ptr(tile_seg),
-                                         _ptr(t["fwd_self_tile_chunk"]), S, H, k.shape[1], D, K, plan.F, plan.N,
+                                         _ptr(t["fwd_self_tile_chunk"]), S, H, Hkv, D, K, plan.F, plan.N,
                                          plan.chunk_size, bound, plan.fwd_self_tiles, _strides(q, k),
                                          _ptr(queues), _ptr(redo), scale, _dtype_code(q), _stream(dev)),
                    "moba_fwd_partials")
@@ -266,15 +293,16 @@ def _forward(q, k, v, plan: MobaPlan, timer: Optional[StageTimer] = None, scale:
 
 def _backward(dout, q, k, v, out, lse, sel, seg_off, seg_dest, plan: MobaPlan, scale: float = 0.0):
     lib = _lib.load()
-    S, H, D = q.shape
+    S, H, D = _dims(q)
+    Hkv = _dims(k)[1]
     dev = q.device
     K = plan.K
     t = plan.tables
     # the backward kernels cut the gather lists into tiles of their own height
     tile_off, tile_seg = (None, None) if plan.fallback else tile_tables(seg_off, plan, H, TILE_ROWS)
-    dq = torch.empty(q.shape, dtype=q.dtype, device=dev)  # packed, whatever the strides of q, k, v
-    dk = torch.empty(k.shape, dtype=k.dtype, device=dev)
-    dv = torch.empty(v.shape, dtype=v.dtype, device=dev)
+    dq = torch.empty((S, H, D), dtype=q.dtype, device=dev)  # packed, whatever the strides of q, k, v
+    dk = torch.empty((S, Hkv, D), dtype=k.dtype, device=dev)
+    dv = torch.empty((S, Hkv, D), dtype=v.dtype, device=dev)
     delta = torch.empty((2, S, H), dtype=torch.float32, device=dev)
     part_dq = torch.empty((S * H * (K + 1), D), dtype=q.dtype, device=dev)
     queues = torch.empty(16, dtype=torch.int32, device=dev)  # tile counters of the two backward kernels (zeroed there)
@@ -282,7 +310,7 @@ def _backward(dout, q, k, v, out, lse, sel, seg_off, seg_dest, plan: MobaPlan, s
                             _ptr(tile_off), _ptr(seg_dest), _ptr(t.get("fchunk_tok")), _ptr(t["chunk_tok"]),
                             _ptr(t["self_tile_prefix"]), _ptr(tile_seg), _ptr(t["self_tile_chunk"]),
                             _ptr(t.get("chunk_fid")), _ptr(delta), _ptr(part_dq), _ptr(dq), _ptr(dk), _ptr(dv),
-                            S, H, k.shape[1], D, K, plan.F, plan.N, plan.chunk_size, plan.hist_tile_bound(H),
+                            S, H, Hkv, D, K, plan.F, plan.N, plan.chunk_size, plan.hist_tile_bound(H),
                             plan.self_tiles, _strides(q, k), _ptr(queues), scale, _dtype_code(q), _stream(dev)),
                "moba_bwd")
     return dq, dk, dv
@@ -306,6 +334,9 @@ class _MobaAttention(torch.autograd.Function):
         q, k, v, out, lse = ctx.saved_tensors
         sel, seg_off, seg_dest = ctx.aux
         dq, dk, dv = _backward(_aligned(dout.to(q.dtype)), q, k, v, out, lse, sel, seg_off, seg_dest, ctx.plan, ctx.scale)
+        if q.dim() == 4:   # gradients in the layout of the batched inputs: views of the packed results
+            b, _, l, d = q.shape
+            dq, dk, dv = (g.view(b, l, -1, d).transpose(1, 2) for g in (dq, dk, dv))
         return dq, dk, dv, None, None, None
 
 
@@ -344,8 +375,33 @@ def moba_attn_varlen_gqa(q, k, v, cu_seqlens, max_seqlen, moba_chunk_size, moba_
     return moba_attn_varlen_with_lse(q, k, v, cu_seqlens, max_seqlen, moba_chunk_size, moba_topk, gqa=True)[0]
 
 
+def moba_attn_batched(query, key, value, moba_chunk_size, moba_topk):
+    """The operator on the transformers layout: query [batch, heads, seqlen, head_dim], key and value
+    [batch, kv_heads, seqlen, head_dim], every batch entry one sequence.  The tensors are read where they lie
+    (no transposing copies, which ``hf_to_fa`` costs for batch > 1, moba/wrapper.py:56-58; no key/value head
+    expansion); returns [batch * seqlen, heads, head_dim] like the packed operator.  Layouts the kernels cannot
+    address, and head_dim below 128, go through packed copies."""
+    from .wrapper import _cu_seqlens_for, hf_to_fa
+    b, h, l, d = query.shape
+    if key.shape != value.shape or key.dim() != 4 or key.shape[0] != b or key.shape[2] != l or key.shape[3] != d:
+        raise ValueError("query must be [batch, heads, seqlen, head_dim] and key, value [batch, kv_heads, seqlen, head_dim]")
+    cu_seqlens = _cu_seqlens_for(b, l, query.device)
+    make_plan(cu_seqlens, moba_chunk_size, moba_topk, host_lengths=range(0, (b + 1) * l, l))
+    in_place = (d == HEAD_DIM and _addressable(query) and _addressable(key) and _addressable(value)
+                and _row_strides(key) == _row_strides(value) and _batch_stride(key) == _batch_stride(value))
+    if not in_place:
+        return moba_attn_varlen_gqa(hf_to_fa(query), hf_to_fa(key), hf_to_fa(value), cu_seqlens, l, moba_chunk_size,
+                                    moba_topk)
+    _check_qkv(query.select(0, 0).transpose(0, 1), key.select(0, 0).transpose(0, 1), value.select(0, 0).transpose(0, 1),
+               gqa=True)
+    plan = make_plan(cu_seqlens, moba_chunk_size, moba_topk, device=query.device)
+    return _MobaAttention.apply(query, key, value, plan)[0]
+
+
 # lets moba_layer skip the key/value head expansion when it drives this operator
 moba_attn_varlen.grouped_query_impl = moba_attn_varlen_gqa
+# ... and the transposing copies of a batch of more than one sequence
+moba_attn_varlen.batched_impl = moba_attn_batched
 # ... and tells it that make_plan(host_lengths=...) spares the device-to-host read of cu_seqlens
 moba_attn_varlen.takes_host_lengths = True
 moba_attn_varlen_gqa.takes_host_lengths = True

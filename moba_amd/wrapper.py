@@ -77,6 +77,18 @@ def moba_layer(
     batch, q_heads, q_len, head_dim = query.shape
     _, kv_heads, kv_len, _ = key.shape
     if q_len == kv_len:
+        chunk_size = moba_config.moba_chunk_size
+        num_layers = getattr(getattr(module, "config", None), "num_hidden_layers", None)
+        if moba_config.is_full_attention_layer(getattr(module, "layer_idx", None), num_layers):
+            # one chunk per sequence: no history chunks, and every implementation of the operator then
+            # computes plain causal attention (moba/moba_efficient.py:313-321, moba/moba_naive.py:58-81)
+            chunk_size = max(chunk_size, kv_len)
+        batched = getattr(moba_impl, "batched_impl", None) if batch > 1 else None
+        if batched is not None:
+            # an implementation that reads [batch, heads, seqlen, head_dim] in place (the HIP operator): no
+            # transposing copies of q, k, v (hf_to_fa's reshape copies when batch > 1, moba/wrapper.py:56-58)
+            # and no key/value head expansion
+            return batched(query, key, value, chunk_size, moba_config.moba_topk), None
         q = hf_to_fa(query)
         k = hf_to_fa(key)
         v = hf_to_fa(value)
@@ -91,12 +103,6 @@ def moba_layer(
                 k = torch.repeat_interleave(k, rep, dim=1)
                 v = torch.repeat_interleave(v, rep, dim=1)
         cu_seqlens = _cu_seqlens_for(batch, kv_len, query.device)
-        chunk_size = moba_config.moba_chunk_size
-        num_layers = getattr(getattr(module, "config", None), "num_hidden_layers", None)
-        if moba_config.is_full_attention_layer(getattr(module, "layer_idx", None), num_layers):
-            # one chunk per sequence: no history chunks, and every implementation of the operator then
-            # computes plain causal attention (moba/moba_efficient.py:313-321, moba/moba_naive.py:58-81)
-            chunk_size = max(chunk_size, kv_len)
         if getattr(moba_impl, "takes_host_lengths", False):
             # the lengths are known here on the host: spare the operator its device-to-host read
             from .plan import make_plan

@@ -455,3 +455,49 @@ def test_more_than_64_history_chunks_is_refused():
         moba_attn_varlen(q.cuda(), k.cuda(), v.cuda(), cu_t, mx, 32, 80)
     out = moba_attn_varlen(q.cuda(), k.cuda(), v.cuda(), cu_t, mx, 32, 65)   # k = 64 is the last one served
     assert torch.isfinite(out.float()).all()
+
+
+@pytest.mark.parametrize("b,hq,hkv,s,B,topk,dtype", [
+    (3, 4, 2, 1500, 128, 3, torch.bfloat16),
+    (2, 8, 8, 2048, 256, 4, torch.float16),
+    (4, 4, 1, 700, 100, 2, torch.bfloat16),
+    (2, 2, 2, 1024, 2048, 3, torch.bfloat16),      # one chunk per sequence: full causal attention
+])
+def test_batched_layout_in_place(b, hq, hkv, s, B, topk, dtype):
+    """[batch, heads, seqlen, head_dim] tensors (the transformers layout) are read where they lie -- no transposing
+    copies for batch > 1 -- and give bit for bit the output and the gradients of the packed operator on the copies
+    hf_to_fa makes (moba/wrapper.py:7-15, :56-58); the packed operator itself is checked against the oracle."""
+    from moba_amd import moba_attn_varlen, moba_attn_varlen_gqa
+    from moba_amd import moba_efficient as E
+    from moba_amd.wrapper import hf_to_fa
+    g = torch.Generator().manual_seed(31)
+    query = torch.randn((b, hq, s, 128), generator=g).to(dtype).cuda().requires_grad_(True)
+    key = torch.randn((b, hkv, s, 128), generator=g).to(dtype).cuda().requires_grad_(True)
+    value = torch.randn((b, hkv, s, 128), generator=g).to(dtype).cuda().requires_grad_(True)
+    do = torch.randn((b * s, hq, 128), generator=g).to(dtype).cuda()
+    assert E._addressable(query) and E._addressable(key) and E._strides(query, key)[4] == s
+    out = E.moba_attn_batched(query, key, value, B, topk)
+    out.backward(do)
+    qp, kp, vp = (hf_to_fa(x.detach()).contiguous().requires_grad_(True) for x in (query, key, value))
+    cu = torch.arange(0, (b + 1) * s, s, dtype=torch.int32, device="cuda")
+    want = moba_attn_varlen_gqa(qp, kp, vp, cu, s, B, topk)
+    want.backward(do)
+    assert out.shape == (b * s, hq, 128) and torch.equal(out, want)
+    for got, ref in ((query.grad, qp.grad), (key.grad, kp.grad), (value.grad, vp.grad)):
+        assert got.shape[0] == b and torch.equal(hf_to_fa(got), ref)
+    # and the oracle, on the packed copies with expanded key/value heads
+    rep = hq // hkv
+    cu_l = cu.tolist()
+    from moba_amd.plan import make_plan
+    plan = make_plan(cu, B, topk)
+    sel = None if plan.fallback else E.gate_topk(qp.detach(), E.chunk_mean(kp.detach(), plan), plan).cpu()
+    ref = O.moba_attn_varlen_oracle(qp.detach().cpu(), torch.repeat_interleave(kp.detach().cpu(), rep, dim=1),
+                                    torch.repeat_interleave(vp.detach().cpu(), rep, dim=1), cu_l, s, B, topk, sel=sel)
+    err = (out.detach().cpu().float() - ref).abs()
+    assert err.max() < MAX_ABS and err.mean() < MEAN_ABS, (err.max().item(), err.mean().item())
+    # a layout the kernels cannot address (rows 8 bytes off a 16-byte line) takes the copying path, same result
+    buf = torch.zeros(query.numel() + 4, dtype=dtype, device="cuda")
+    buf[4:].copy_(query.detach().reshape(-1))
+    odd = buf[4:].view(query.shape)
+    assert not E._addressable(odd)
+    assert torch.equal(E.moba_attn_batched(odd, key.detach(), value.detach(), B, topk), want)

@@ -124,13 +124,13 @@ def test_full_attention_layers_through_the_hip_operator():
     model = _model(torch.bfloat16)
     ids = torch.randint(0, 128, (2, 1024), device="cuda")
     import moba_amd.moba_efficient as E
-    chunk_sizes, real = [], E.moba_attn_varlen_with_lse
+    chunk_sizes, real = [], E.moba_attn_varlen.batched_impl
 
-    def spying(q, k, v, cu_seqlens, max_seqlen, moba_chunk_size, moba_topk, **kw):
+    def spying(query, key, value, moba_chunk_size, moba_topk):   # (a batch of two: the adapter's batched path)
         chunk_sizes.append(moba_chunk_size)
-        return real(q, k, v, cu_seqlens, max_seqlen, moba_chunk_size, moba_topk, **kw)
+        return real(query, key, value, moba_chunk_size, moba_topk)
 
-    E.moba_attn_varlen_with_lse = spying
+    E.moba_attn_varlen.batched_impl = spying
     try:
         with torch.no_grad():
             model.config._attn_implementation = "eager"
@@ -149,7 +149,7 @@ def test_full_attention_layers_through_the_hip_operator():
             model.config._attn_implementation = "moba"
             none_full = model(ids).logits.float()
     finally:
-        E.moba_attn_varlen_with_lse = real
+        E.moba_attn_varlen.batched_impl = real
         register_moba(MoBAConfig(moba_chunk_size=128, moba_topk=3))
     err = (both_full - eager).abs()
     assert err.max() < 6e-2 and err.mean() < 4e-3, (err.max().item(), err.mean().item())
