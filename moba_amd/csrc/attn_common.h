@@ -115,15 +115,38 @@ __device__ __forceinline__ int logical_tile_id() {
 constexpr int kTileUnused = -1, kTilePastEnd = -2;
 __device__ __forceinline__ int decode_tile_code(const TileTables& p, int logical) {
   if (logical < 0) return kTileUnused;
-  if (logical < p.hist_bound) return p.tile_seg[logical];
+  if (logical < p.hist_bound) return table_load(p.tile_seg + logical);
   const int st = logical - p.hist_bound;
   if (st >= p.self_total) return kTilePastEnd;
-  return p.self_tile_chunk[st / p.H];  // self_tile_prefix[c]*H <= st < self_tile_prefix[c+1]*H
+  return table_load(p.self_tile_chunk + st / p.H);  // self_tile_prefix[c]*H <= st < self_tile_prefix[c+1]*H
 }
 // Step 1, wave-uniform: head, key range, number of rows, from the small per-segment / per-chunk tables.
+// In two halves, so that a kernel can have the table entries on their way while it does something else:
+// tile_head_entries starts the four lookups, decode_tile_head turns their results into the description.
 // Returns false (and row_count = 0) for a code that is not a tile.
 // (tm: rows per tile of the tables in p)
-__device__ __forceinline__ bool decode_tile_head(const TileTables& p, int logical, int code, Tile& t, int tm = TM) {
+struct TileHeadEntries {
+  int a, b, c, d;  // history tile: tile_off[seg], seg_off[seg], seg_off[seg+1], fchunk_tok[f];
+                   // self tile: self_tile_prefix[c], self_tile_prefix[c+1], chunk_tok[c], chunk_tok[c+1]
+};
+__device__ __forceinline__ TileHeadEntries tile_head_entries(const TileTables& p, int logical, int code) {
+  TileHeadEntries e = {0, 0, 0, 0};
+  if (code < 0) return e;
+  if (logical < p.hist_bound) {
+    e.a = table_load(p.tile_off + code);
+    e.b = table_load(p.seg_off + code);
+    e.c = table_load(p.seg_off + code + 1);
+    e.d = table_load(p.fchunk_tok + code / p.H);
+  } else {
+    e.a = table_load(p.self_tile_prefix + code);
+    e.b = table_load(p.self_tile_prefix + code + 1);
+    e.c = table_load(p.chunk_tok + code);
+    e.d = table_load(p.chunk_tok + code + 1);
+  }
+  return e;
+}
+__device__ __forceinline__ bool decode_tile_head(const TileTables& p, int logical, int code, const TileHeadEntries& e,
+                                                 Tile& t, int tm = TM) {
   const int H = p.H;
   t.id = logical;
   t.row_count = 0;
@@ -131,30 +154,32 @@ __device__ __forceinline__ bool decode_tile_head(const TileTables& p, int logica
   if (code < 0) return false;
   if (logical < p.hist_bound) {
     const int seg = code;
-    const int tile = logical - p.tile_off[seg];
+    const int tile = logical - e.a;
     const int f = seg / H;
     t.h = seg - f * H;
-    t.base = p.seg_off[seg] + tile * tm;
-    t.row_count = min(tm, p.seg_off[seg + 1] - t.base);
-    t.kv_tok0 = p.fchunk_tok[f];
+    t.base = e.b + tile * tm;
+    t.row_count = min(tm, e.c - t.base);
+    t.kv_tok0 = e.d;
     t.nkeys = p.B;
     t.rot = tile;
     return true;
   }
   const int st = logical - p.hist_bound;
-  const int c = code;
-  const int rem = st - p.self_tile_prefix[c] * H;
-  const int nt = p.self_tile_prefix[c + 1] - p.self_tile_prefix[c];
+  const int rem = st - e.a * H;
+  const int nt = e.b - e.a;
   t.h = rem / nt;
   const int tin = nt - 1 - (rem - t.h * nt);  // longest tiles first
-  const int c0 = p.chunk_tok[c];
-  const int len = p.chunk_tok[c + 1] - c0;
+  const int c0 = e.c;
+  const int len = e.d - c0;
   t.base = -1 - tin * tm;                   // self tile: -(first row of the tile inside its chunk) - 1
   t.row_count = min(tm, len - tin * tm);
   t.kv_tok0 = c0;
   t.nkeys = min(len, tin * tm + tm);
   t.rot = 0;
   return true;
+}
+__device__ __forceinline__ bool decode_tile_head(const TileTables& p, int logical, int code, Tile& t, int tm = TM) {
+  return decode_tile_head(p, logical, code, tile_head_entries(p, logical, code), t, tm);
 }
 __device__ __forceinline__ bool decode_tile_head(const TileTables& p, int logical, Tile& t, int tm = TM) {
   return decode_tile_head(p, logical, decode_tile_code(p, logical), t, tm);

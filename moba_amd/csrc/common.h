@@ -98,9 +98,30 @@ __device__ __forceinline__ T kernarg_now(int offset) {
   typedef __attribute__((address_space(4))) const char* kernarg_ptr;
   kernarg_ptr kp = (kernarg_ptr)__builtin_amdgcn_kernarg_segment_ptr();
   asm volatile("" : "+s"(kp));  // not the pointer the compiler knows: the loads stay where they are written
-  T x;
-  __builtin_memcpy(&x, kp + offset, sizeof(T));
-  return x;
+  // read through a pointer of the piece's own type: with the alignment known the loads are scalar loads
+  // (a byte-wise copy makes them vector loads, which queue behind every vector load and copy in flight)
+#if defined(__HIP_DEVICE_COMPILE__)
+  return *reinterpret_cast<__attribute__((address_space(4))) const T*>(kp + offset);
+#else
+  return T();  // (the host pass only parses device code)
+#endif
+}
+
+// Load from a table that no kernel writes while this one runs, at an address that is the same in every lane:
+// read through the constant address space, so that the compiler may use a scalar load (its own counter, not
+// queued behind the vector loads and copies in flight).
+template <class T>
+__device__ __forceinline__ T table_load(const T* p) {
+  const uint64_t a = (uint64_t)(uintptr_t)p;  // made uniform explicitly: a scalar load whatever the compiler can prove
+  // (the builtin returns a signed int: through uint32_t, or the low half would be sign-extended over the high one)
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)a);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+  const uint64_t ua = ((uint64_t)hi << 32) | lo;
+#if defined(__HIP_DEVICE_COMPILE__)
+  return *reinterpret_cast<__attribute__((address_space(4))) const T*>(ua);
+#else
+  return T();  // (the host pass only parses device code)
+#endif
 }
 
 // Result of the launches of one entry point: an error that was already pending on the calling thread when the

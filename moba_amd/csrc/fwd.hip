@@ -98,6 +98,8 @@ __global__ __launch_bounds__(512, 2) void moba_fwd_kernel(const FwdParams<E> p) 
   // and used at the next; the entries travel global -> LDS, so nothing of this occupies vector registers.
   const int r = wave * 32 + n;
   Tile t, t1;              // the tile being computed; the next one (its row entries on their way to LDS)
+  int id1 = -1, code1 = kTileUnused;   // id and first lookup of the next tile
+  TileHeadEntries head1 = {0, 0, 0, 0};  // its small-table entries
   int id2 = -1, code2 = kTileUnused;   // id and first lookup of the tile after next
   int id3 = -1;                        // id of the tile after that, as drawn
   int queue = blockIdx.x & 7, empty_queues = 0;
@@ -242,14 +244,12 @@ __global__ __launch_bounds__(512, 2) void moba_fwd_kernel(const FwdParams<E> p) 
   if constexpr (kFixedRef) {
     if (tid == 0) *reinterpret_cast<int*>(smem + kFwdRedoWord) = 0;  // first read many barriers from here
   }
-  while (true) {
-  // ================= tile switch =================
-  wait_vmem();  // nothing of this wave is in flight any more: the next tile's row entries are in LDS
-  if (have_partial) {
-    // ---- the finished tile's partial: normalise, write ----
-    // The accumulators hold O^T (a lane owns 4-element pieces of one row); the rows go through this
-    // wave's 8 KiB of LDS (free since the barrier that ended the tile) so that they leave as whole
-    // 256-byte rows, four per store instruction, instead of 8-byte pieces of 32 rows.
+  // The finished tile's partial: normalise, write.  The accumulators hold O^T (a lane owns 4-element pieces of
+  // one row); the rows go through 4 KiB of LDS per wave, half a row at a time, so that they leave as 128-byte
+  // pieces of rows, eight rows per store instruction, instead of 8-byte pieces of 32 rows.  The 4 KiB lie in the
+  // third K and V stages, which take their next copies only behind the barrier of the next tile's first key
+  // tile: the first two stages are already receiving the next tile's keys and values while this runs.
+  auto write_partial = [&]() __attribute__((always_inline)) {
     const FwdParams<E> pn = kernarg_now<FwdParams<E>>(0);
     int ln = lane;  // taken afresh: none of the addresses below is computed ahead of the tile loop
     asm volatile("" : "+v"(ln));
@@ -261,43 +261,79 @@ __global__ __launch_bounds__(512, 2) void moba_fwd_kernel(const FwdParams<E> p) 
       const bool bad = valid_done && __builtin_bit_cast(uint32_t, l_tot) >= __builtin_bit_cast(uint32_t, kFixedRefMaxSum);
       if (__any(bad) && ln == 0) *reinterpret_cast<volatile int*>(smem + kFwdRedoWord) = 1;
     }
-    char* stage = smem + wave_u * 8192;
-    char* wrow = stage + en * 256 + 8 * ehh;
-#pragma unroll
-    for (int db = 0; db < 4; ++db)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        u32x2 w;
-        w[0] = pack2<E>(oacc[db][4 * g + 0] * inv, oacc[db][4 * g + 1] * inv);
-        w[1] = pack2<E>(oacc[db][4 * g + 2] * inv, oacc[db][4 * g + 3] * inv);
-        // elements 32*db + 8*g + 4*hh .. +3 of row n: 16-byte column 4*db + g, swizzled by the row
-        *reinterpret_cast<u32x2*>(wrow + (((4 * db + g) ^ (en & 15)) << 4)) = w;
-      }
+    char* stage = smem + (wave_u < 4 ? 2 * kTileBytes + wave_u * 4096 : kFwdVBase + 2 * kTileBytes + (wave_u - 4) * 4096);
+    char* wrow = stage + en * 128 + 8 * ehh;
+    const int wsw = (en >> 1) & 7;  // rows 128 bytes apart: the 16-byte column is swizzled by the row pair
     if (valid_done && ehh == 0) pn.part_lse[dest_done] = m_run + fast_log2(l_tot);
-    const int c16 = ln & 15;
+    const int c16 = ln & 7;
+    int dest[4];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int row = 4 * i + (ln >> 4);
-      const int dest = __shfl(dest_done, row, 64);
-      const u32x4 x = *reinterpret_cast<const u32x4*>(stage + row * 256 + ((c16 ^ (row & 15)) << 4));
-      if (row < rows_done) *reinterpret_cast<u32x4*>(pn.part_o + (int64_t)dest * kHeadDim + c16 * 8) = x;
+    for (int i = 0; i < 4; ++i) dest[i] = __shfl(dest_done, 8 * i + (ln >> 3), 64);
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+#pragma unroll
+      for (int d2 = 0; d2 < 2; ++d2)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int db = 2 * half + d2;
+          u32x2 w;
+          w[0] = pack2<E>(oacc[db][4 * g + 0] * inv, oacc[db][4 * g + 1] * inv);
+          w[1] = pack2<E>(oacc[db][4 * g + 2] * inv, oacc[db][4 * g + 3] * inv);
+          // elements 32*db + 8*g + 4*hh .. +3 of row n: 16-byte column 4*d2 + g of this half
+          *reinterpret_cast<u32x2*>(wrow + (((4 * d2 + g) ^ wsw) << 4)) = w;
+        }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int row = 8 * i + (ln >> 3);
+        const u32x4 x = *reinterpret_cast<const u32x4*>(stage + row * 128 + ((c16 ^ ((row >> 1) & 7)) << 4));
+        if (row < rows_done) *reinterpret_cast<u32x4*>(pn.part_o + (int64_t)dest[i] * kHeadDim + 64 * half + c16 * 8) = x;
+      }
     }
-#pragma unroll
-    for (int db = 0; db < 4; ++db)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) oacc[db][e] = 0.f;
-    if constexpr (kMode == kTilePerGroup) return;
-    m_run = -INFINITY;
-    l_run = 0.f;
-    __syncthreads();  // the K stages take the next tile's copies only after every wave has read its rows back
+  };
+  // a tile of the fixed-reference kernel whose rows left the safe range (marked in LDS by the waves that wrote
+  // its partial; call behind a barrier that follows those writes) enters the list of tiles to compute again
+  auto list_for_redo = [&]() __attribute__((always_inline)) {
     if constexpr (kFixedRef) {
-      // one thread enters the tile in the list if any wave marked it (the word is next written by a later
-      // tile's epilogue, several barriers from here)
       if (tid == 0 && *reinterpret_cast<volatile int*>(smem + kFwdRedoWord) != 0) {
+        const FwdParams<E> pn = kernarg_now<FwdParams<E>>(0);
         *reinterpret_cast<volatile int*>(smem + kFwdRedoWord) = 0;
         const int at = __hip_atomic_fetch_add(pn.redo, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         pn.redo[1 + at] = id_done;
       }
+    }
+  };
+  // Queued tiles: the Q rows of the next tile are requested while the current tile still computes -- between
+  // the two steps of its last key tile, the first point at which the registers of the Q^T operand are free
+  // (the last step forms no S^T) -- so that they travel under the last matrix instructions and the partial's
+  // stores.  The next tile's row entries have been in LDS since this tile's first key tile; its rows are decoded
+  // here.  On every pass, from row 0 when no tile follows: the operand carries no value around the loop.
+  auto prefetch_q = [&]() __attribute__((always_inline)) {
+    if constexpr (kQueued) {
+      const FwdParams<E> pn = kernarg_now<FwdParams<E>>(0);
+      int tx = threadIdx.x;  // taken afresh
+      asm volatile("" : "+v"(tx));
+      const int er = (tx >> 6) * 32 + (tx & 31);
+      wait_vmem();  // (the entries' copy; nothing else of this wave is in flight here)
+      int q_tok = 0, q_head = 0;
+      if (t1.row_count > 0) {
+        const int entry = *reinterpret_cast<const int*>(smem + kFwdEntries + 4 * tx);
+        decode_tile_rows(pn.t, tx >> 6, er, entry, t1);
+        q_tok = t1.tok;
+        q_head = t1.h;
+      }
+      const elem* src = reinterpret_cast<const elem*>((const char*)pn.q + q_tok_bytes(pn.t, q_tok) + q_head * pn.t.q_head_b) + 8 * (tx >> 5 & 1);
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) bq[ks] = *reinterpret_cast<const elem8*>(src + 16 * ks);
+    }
+  };
+  while (true) {
+  // ================= tile switch =================
+  // The next tile's first copies and loads are issued before the finished tile's partial is written: they
+  // travel while the partial is normalised and stored.
+  if constexpr (kMode == kTilePerGroup) {
+    if (have_partial) {
+      write_partial();
+      return;
     }
   }
   int drawn = 0;  // wave 0, lane 0: the value of the queue's counter
@@ -309,13 +345,17 @@ __global__ __launch_bounds__(512, 2) void moba_fwd_kernel(const FwdParams<E> p) 
     if constexpr (kQueued) {
       t = t1;  // the next tile becomes the current one: its rows' gather-list entries are in LDS by now
     } else if constexpr (kMode == kTilesListed) {
-      if (list_pos >= pn.redo[0]) return;  // (uniform; the count is final: the kernel that wrote it has ended)
-      const int listed = pn.redo[1 + list_pos];
-      list_pos += gridDim.x;
-      if (!decode_tile_head(pn.t, listed, t, kFwdTileRows)) return;  // (cannot happen: listed ids are tiles)
+      t.row_count = 0;
+      t.nkeys = -1;  // unless there is another tile in the list
+      if (list_pos < pn.redo[0]) {  // (uniform; the count is final: the kernel that wrote it has ended)
+        const int listed = pn.redo[1 + list_pos];
+        list_pos += gridDim.x;
+        if (!decode_tile_head(pn.t, listed, t, kFwdTileRows)) t.nkeys = -1;  // (cannot happen: listed ids are tiles)
+      }
     } else {
       if (!decode_tile_head(pn.t, logical_tile_id(), t, kFwdTileRows)) return;
     }
+    int q_tok = 0, q_head = 0;  // token and head of this lane's query row
     if (t.row_count > 0) {
       // the wave-uniform half of the description is enough to start the first copies: the first two K
       // and V tiles (global -> LDS)
@@ -333,26 +373,52 @@ __global__ __launch_bounds__(512, 2) void moba_fwd_kernel(const FwdParams<E> p) 
         issue_v(key_tile(1), 1);
       }
 
-      // the per-row half, then the Q rows.  Q^T operand: lane (n, hh) holds q[tok][16*ks + 8*hh .. +7]
-      const int entry = kQueued ? *reinterpret_cast<const int*>(smem + kFwdEntries + 4 * tx)
-                                : decode_tile_row_entry(pn.t, er, t);
-      decode_tile_rows(pn.t, tx >> 6, er, entry, t);
+      // the per-row half (queued: decoded when the Q rows were requested, see prefetch_q), then the Q rows
+      if constexpr (!kQueued) decode_tile_rows(pn.t, tx >> 6, er, decode_tile_row_entry(pn.t, er, t), t);
       limit = t.limit;
       min_limit = __builtin_amdgcn_readfirstlane(t.wave_min_limit);
       row_valid = er < t.row_count;
-      const elem* src = reinterpret_cast<const elem*>((const char*)pn.q + q_tok_bytes(pn.t, t.tok) + h * pn.t.q_head_b) + 8 * (tx >> 5 & 1);
+      q_tok = t.tok;
+      q_head = h;
+    }
+    if constexpr (!kQueued) {
+      // Q^T operand: lane (n, hh) holds q[tok][16*ks + 8*hh .. +7]
+      // (loaded on every pass, from row 0 when there is no tile, so that the operand carries no value from one
+      // pass of the loop to the next)
+      const elem* src = reinterpret_cast<const elem*>((const char*)pn.q + q_tok_bytes(pn.t, q_tok) + q_head * pn.t.q_head_b) + 8 * (tx >> 5 & 1);
 #pragma unroll
       for (int ks = 0; ks < 8; ++ks) bq[ks] = *reinterpret_cast<const elem8*>(src + 16 * ks);
     }
     if constexpr (kQueued) {
-      // look-ahead: small-table lookups of the tile after, big-table lookup of the one after that, a new id
-      if (!decode_tile_head(pn.t, id2, code2, t1, kFwdTileRows)) t1.nkeys = (code2 == kTilePastEnd) ? -1 : 0;
+      // look-ahead: small-table lookups of the tile after (their results are taken up behind the partial's
+      // stores), big-table lookup of the one after that, a new id
+      id1 = id2;
+      code1 = code2;
+      head1 = tile_head_entries(pn.t, id1, code1);
       id2 = id3;
       code2 = decode_tile_code(pn.t, id2);
       if (tx == 0) drawn = __hip_atomic_fetch_add(pn.queues + queue, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
   }
-  if (t.nkeys < 0) break;  // (uniform) no tiles left
+  if (have_partial) write_partial();
+  if constexpr (kQueued) {
+    const TileTables tt = kernarg_now<TileTables>(offsetof(FwdParams<E>, t));
+    if (!decode_tile_head(tt, id1, code1, head1, t1, kFwdTileRows)) t1.nkeys = (code1 == kTilePastEnd) ? -1 : 0;
+  }
+  // (on every pass, so that the accumulators carry no value from one pass of the loop to the next)
+#pragma unroll
+  for (int db = 0; db < 4; ++db)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) oacc[db][e] = 0.f;
+  m_run = -INFINITY;
+  l_run = 0.f;
+  if (t.nkeys < 0) {  // (uniform) no tiles left
+    if constexpr (kFixedRef) {
+      __syncthreads();
+      list_for_redo();
+    }
+    break;
+  }
   // every copy of this wave has landed, and wave 0 has its draw
   wait_vmem();
   if constexpr (kQueued) {
@@ -363,6 +429,7 @@ __global__ __launch_bounds__(512, 2) void moba_fwd_kernel(const FwdParams<E> p) 
     if (nkt > 1) scrub_v(key_tile(1), 1);
   }
   __syncthreads();
+  list_for_redo();  // (the finished tile's id is still in id_done)
   if constexpr (kQueued) {
     // the id drawn: queue `queue` counts the ids (8i + queue) * kQueueRun + j; past the last tile the
     // workgroup moves to the next queue, and after eight empty queues in a row there is nothing left
@@ -388,7 +455,10 @@ __global__ __launch_bounds__(512, 2) void moba_fwd_kernel(const FwdParams<E> p) 
     }
   }
   have_partial = t.row_count > 0;
-  if (!have_partial) continue;
+  if (!have_partial) {
+    prefetch_q();
+    continue;
+  }
   dest_done = t.dest;
   id_done = t.id;
   valid_done = row_valid;
@@ -567,6 +637,7 @@ __global__ __launch_bounds__(512, 2) void moba_fwd_kernel(const FwdParams<E> p) 
       }
     }
     step(s0, s1, kcur, 1, key0 + 32, std::true_type{}, mask_a, vcur, 0, more, knext, 0);
+    if constexpr (!more) prefetch_q();
     step(s1, s0, knext, 0, key0n, more_c, mask_b, vcur, 1, more, knext, 1);
   };
   using St0 = std::integral_constant<int, 0>;
