@@ -205,21 +205,41 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams<E> p) {
     for (int e = 0; e < 16; ++e) dqacc[db][e] = 0.f;
   const float sl2 = p.scale_log2;
 
+  // Per-lane LDS byte addresses of the fragments inside K stage 0 (numbers, not pointers into smem: a read's
+  // address is then one register plus an immediate for stage, key block and V, with no base left to add):
+  // row fragments (key 32*kb + n, 16-byte column 2*s8 + hh) and transposed quads (keys 32*kb + 16*j2 + 4*hh +
+  // i0 and + 8, 8 bytes at d = 32*db + 16*(g16&1) + 4*i1).
   const int g16 = lane >> 4, i0 = (lane & 15) >> 2, i1 = lane & 3;
-  const int row_off = n * 256;
-  const int row_sw = ((n & 3) << 2) ^ ((n >> 2) & 3);
-  const int tr_c16 = 2 * (g16 & 1) + (i1 >> 1);
-  const int tr_sub = (i1 & 1) * 8;
+  uint32_t foff[8], toffA[4], toffB[4];
+  {
+    const int row_sw = ((n & 3) << 2) ^ ((n >> 2) & 3);
+#pragma unroll
+    for (int s8 = 0; s8 < 8; ++s8) {
+      foff[s8] = lds_base + n * 256 + (((2 * s8 + hh) ^ row_sw) << 4);
+      asm volatile("" : "+v"(foff[s8]));  // finished addresses, kept as they are
+    }
+    const int tr_c16 = 2 * (g16 & 1) + (i1 >> 1);
+    const int tr_sub = (i1 & 1) * 8;
+#pragma unroll
+    for (int db = 0; db < 4; ++db) {
+      const int c16 = 4 * db + tr_c16;
+      toffA[db] = lds_base + (4 * hh + i0) * 256 + ((c16 ^ (i0 << 2) ^ hh) << 4) + tr_sub;
+      toffB[db] = lds_base + (4 * hh + i0 + 8) * 256 + ((c16 ^ (i0 << 2) ^ (hh + 2)) << 4) + tr_sub;
+      asm volatile("" : "+v"(toffA[db]));
+      asm volatile("" : "+v"(toffB[db]));
+    }
+  }
 
-  for (int it = 0; it < nkt; ++it) {
+  // one key tile; buf_c: its LDS stage, a constant in the two copies of the loop body
+  auto key_tile_body = [&](int it, auto buf_c) __attribute__((always_inline)) {
+    constexpr int buf = decltype(buf_c)::value;
     const int kt = key_tile(it);
-    const int buf = it & 1;
     const bool has_next = it + 1 < nkt;
     if (has_next) issue_tile(key_tile(it + 1), buf ^ 1);
 
     if (kt * TN <= t.wave_max_limit) {
-      const char* ks = smem + buf * kTileBytes;
-      const char* vs = smem + (2 + buf) * kTileBytes;
+      constexpr uint32_t ks = buf * kTileBytes;         // K stage, relative to stage 0
+      constexpr uint32_t vs = (2 + buf) * kTileBytes;   // V stage
       const bool masked = kt * TN + TN - 1 > t.wave_min_limit;
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb) {
@@ -228,9 +248,8 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams<E> p) {
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int s8 = 0; s8 < 8; ++s8) {
-          const int o = kb * 8192 + row_off + (((2 * s8 + hh) ^ row_sw) << 4);
-          ka[s8] = *reinterpret_cast<const elem8*>(ks + o);
-          va[s8] = *reinterpret_cast<const elem8*>(vs + o);
+          ka[s8] = *lds_ptr<const elem8>(foff[s8] + (ks + kb * 8192));
+          va[s8] = *lds_ptr<const elem8>(foff[s8] + (vs + kb * 8192));
         }
         f32x16 sacc, dpacc;
 #pragma unroll
@@ -253,11 +272,8 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams<E> p) {
         elem4 tr[8][2];
         auto issue_tr = [&](int idx) __attribute__((always_inline)) {
           const int j2 = idx >> 2, db = idx & 3;
-          const int keyA = 16 * (2 * kb + j2) + 4 * hh + i0;
-          const int keyB = keyA + 8;
-          const int c16 = 4 * db + tr_c16;
-          tr[idx][0] = lds_read_tr<elem4>(ks + keyA * 256 + ((c16 ^ (i0 << 2) ^ hh) << 4) + tr_sub);
-          tr[idx][1] = lds_read_tr<elem4>(ks + keyB * 256 + ((c16 ^ (i0 << 2) ^ (hh + 2)) << 4) + tr_sub);
+          tr[idx][0] = lds_read_tr<elem4>(toffA[db] + (ks + 16 * (2 * kb + j2) * 256));
+          tr[idx][1] = lds_read_tr<elem4>(toffB[db] + (ks + 16 * (2 * kb + j2) * 256));
         };
 #pragma unroll
         for (int idx = 0; idx < 4; ++idx) issue_tr(idx);
@@ -293,6 +309,14 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams<E> p) {
       scrub_tile(key_tile(it + 1), buf ^ 1);
     }
     __syncthreads();
+  };
+  {
+    int it = 0;
+    for (; it + 1 < nkt; it += 2) {
+      key_tile_body(it, std::integral_constant<int, 0>{});
+      key_tile_body(it + 1, std::integral_constant<int, 1>{});
+    }
+    if (it < nkt) key_tile_body(it, std::integral_constant<int, 0>{});
   }
 
   // The accumulators hold dQ^T (a lane owns 4-element pieces of one row).  The partial is rounded to the
