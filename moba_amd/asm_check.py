@@ -122,10 +122,27 @@ def device_assembly(hipcc: str, flags: list[str], source: str) -> str:
     return r.stdout
 
 
+def dkv_kernel_symbols(asm: str) -> list[str]:
+    """Names (up to the template arguments) of every instantiation of bwd_dkv_kernel in the assembly."""
+    out = []
+    for l in asm.split("\n"):
+        m = _LABEL.match(l)
+        if m and "bwd_dkv_kernel" in m.group(1) and not m.group(1).startswith(".L"):
+            name = m.group(1)
+            cut = name.find("EEEv")
+            name = name[name.index("bwd_dkv_kernel"):cut if cut > 0 else len(name)]
+            if name not in out:
+                out.append(name)
+    return out
+
+
 def check_dkv_kernel(asm: str) -> str:
     """Raises if a hand-issued MFMA result of bwd_dkv_kernel is touched too early; returns a one-line report."""
     lines = []
-    for sym in ("bwd_dkv_kernelINS_4Bf16", "bwd_dkv_kernelINS_3F16"):
+    symbols = dkv_kernel_symbols(asm)
+    if not symbols:
+        raise RuntimeError("no bwd_dkv_kernel in the assembly (the check looks at nothing)")
+    for sym in symbols:
         dist, count, where = min_result_distance(asm, sym)
         if count == 0:
             raise RuntimeError(f"{sym}: no MFMA with a vector-register destination found (the check looks at nothing)")

@@ -398,7 +398,9 @@ __global__ __launch_bounds__(256) void bwd_dq_reduce_kernel(const typename E::el
 }
 
 // ------------------------------------------------------------------------------------ dK, dV
-template <class E>
+// kBatched: q is a batched layout (rows of different batch entries are not an affine function of the token);
+// the common case has no division and no branch in the address of a gathered Q row.
+template <class E, bool kBatched>
 __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
   MOBA_ELEM_TYPES(E)
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -504,7 +506,8 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
     const int row = 4 * slab + ld_rin;
     const int c16 = sw_col16(row, ld_pc);
     if ((g & 1) == 0)
-      async_copy16((const char*)p.q + (q_tok_bytes(p.t, toks[i]) + h * p.t.q_head_b + c16 * 16), qdst + slab * 1024);
+      async_copy16((const char*)p.q + ((kBatched ? q_tok_bytes(p.t, toks[i]) : (int64_t)toks[i] * p.t.q_tok_b) + h * p.t.q_head_b + c16 * 16),
+                   qdst + slab * 1024);
     else
       async_copy16((const char*)p.dout + (((int64_t)toks[i] * H + h) * kHeadDim + c16 * 8) * 2,
                    qdst + TQ * kHeadDim * 2 + slab * 1024);
@@ -708,12 +711,13 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
     if (has_next) wait_vmem();
     __syncthreads();
     // the copies of stage qi+2 go out one at a time inside the next phase A
-    const bool issue_next = qi + 2 < ntile;
-    if (issue_next) prepare_stage(qi + 2);
+    // (past the last stage the copies go on, into buffers that nobody reads, with the rows of the last
+    // lookup: the stage loop then has no branch around any of them)
+    prepare_stage(qi + 2);
     fetch_rows(qi + 3);
 
     phase_b(qs, 0, pb, dsb, qs_next, 0, qs, 1);
-    auto dma = [&](int g) __attribute__((always_inline)) { if (issue_next) issue_part(g, buf2); };
+    auto dma = [&](int g) __attribute__((always_inline)) { issue_part(g, buf2); };
     if (masked) phase_a(sA, dA, sB, dB, std::true_type{}, 1, rows_here, is_self, qpos0, pb, dsb, dma);
     else        phase_a(sA, dA, sB, dB, std::false_type{}, 1, rows_here, is_self, qpos0, pb, dsb, dma);
     phase_b(qs, 1, pb, dsb, qs_next, 1, qs_next, 0);
@@ -722,6 +726,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
   // The last phase A left an S and a dO V^T that nobody reads: their registers may be reused at once on the way
   // out of the loop, and the compiler puts no wait states behind the hand-issued MFMAs that wrote them.
   asm volatile("s_nop 15");
+  wait_vmem();  // (the copies past the last stage: nothing may be on its way into LDS when the workgroup ends)
   }  // query heads
 
   if (key_valid) {
@@ -771,9 +776,11 @@ static int launch_bwd(const void* dout, const void* q, const void* k, const void
   p.hk_shift = 31 + lg;
   p.hk_magic = (uint32_t)((1ull << p.hk_shift) / hk + 1);
 
-  static bool allowed_dq[kMaxDevices], allowed_dkv[kMaxDevices];  // one pair per element type
+  static bool allowed_dq[kMaxDevices], allowed_dkv[2][kMaxDevices];  // one set per element type
+  const bool batched = t.batch_rows != 0;
   if (!allow_dynamic_lds((const void*)bwd_dq_kernel<E>, kBwdDqLds, allowed_dq) ||
-      !allow_dynamic_lds((const void*)bwd_dkv_kernel<E>, kBwdDkvLds, allowed_dkv))
+      !(batched ? allow_dynamic_lds((const void*)bwd_dkv_kernel<E, true>, kBwdDkvLds, allowed_dkv[1])
+                : allow_dynamic_lds((const void*)bwd_dkv_kernel<E, false>, kBwdDkvLds, allowed_dkv[0])))
     return MOBA_ERR_LAUNCH;
   const int64_t rows = S * H;
   hipLaunchKernelGGL(bwd_delta_kernel<E>, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st, (const elem*)dout,
@@ -782,7 +789,8 @@ static int launch_bwd(const void* dout, const void* q, const void* k, const void
   hipLaunchKernelGGL(bwd_dq_kernel<E>, dim3((unsigned)grid_q), dim3(256), kBwdDqLds, st, p);
   hipLaunchKernelGGL(bwd_dq_reduce_kernel<E>, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st,
                      (const elem*)part_dq, sel, (elem*)dq, rows, K + 1);
-  hipLaunchKernelGGL(bwd_dkv_kernel<E>, dim3((unsigned)grid_kv), dim3(256), kBwdDkvLds, st, p);
+  if (batched) hipLaunchKernelGGL((bwd_dkv_kernel<E, true>), dim3((unsigned)grid_kv), dim3(256), kBwdDkvLds, st, p);
+  else hipLaunchKernelGGL((bwd_dkv_kernel<E, false>), dim3((unsigned)grid_kv), dim3(256), kBwdDkvLds, st, p);
   return launch_check.result();
 }
 
@@ -810,7 +818,7 @@ extern "C" int moba_bwd(const void* dout, const void* q, const void* k, const vo
   if ((int64_t)S * H * (K + 1) >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
   const int64_t total_q = (K > 0 ? hist_bound : 0) + self_tiles * H;
   // the dK/dV kernel: one workgroup per CU, resident, drawing its tiles from the queues
-  const int cus = compute_units();
+  const int cus = resident_compute_units();
   if (cus <= 0) return MOBA_ERR_LAUNCH;
   const int64_t grid_kv = ((int64_t)cus + 7) / 8 * 8;
   const int64_t grid_q = 2 * grid_kv;  // the dQ kernel fits two workgroups on a CU

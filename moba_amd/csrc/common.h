@@ -1,5 +1,6 @@
 // Shared device helpers for the gfx950 MoBA kernels.
 #pragma once
+#include <cstdlib>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -159,6 +160,21 @@ inline int compute_units() {
   if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 0;
   if (dev < kMaxDevices) count[dev] = n;
   return n;
+}
+
+// Diagnostic: the environment variable MOBA_RESIDENT_CUS (read once) makes the kernels whose workgroups stay
+// resident and draw tiles from queues occupy only that many compute units' worth of workgroups.  With part of
+// the chip idle the rest runs at a higher clock: this is how the power-limited clock under full load is told
+// apart from the kernels' own efficiency.  Results do not depend on it.
+inline int resident_compute_units() {
+  static int limit = -1;
+  if (limit < 0) {
+    const char* e = getenv("MOBA_RESIDENT_CUS");
+    limit = e ? atoi(e) : 0;
+    if (limit < 0) limit = 0;
+  }
+  const int cus = compute_units();
+  return (limit > 0 && limit < cus) ? limit : cus;
 }
 
 // largest i in [0, n) with a[i] <= x, for ascending a with a[0] <= x

@@ -796,7 +796,7 @@ extern "C" int moba_fwd_partials(const void* q, const void* k, const void* v, vo
   if (total >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
   // one workgroup of eight waves per CU (what the kernel's registers allow), all resident at once and drawing
   // tiles from the queues; a multiple of 8 so that every XCD starts on its own queue with as many
-  const int cus = compute_units();
+  const int cus = resident_compute_units();
   if (cus <= 0) return MOBA_ERR_LAUNCH;
   int64_t grid = ((int64_t)cus + 7) / 8 * 8;
   // with fewer than a few tiles per resident workgroup the queues do not pay: one workgroup per id then
