@@ -584,9 +584,15 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
         if (u == 0) mfma32_into_vgprs(s_next, qa[s8], bk[s8], s8 == 0);
         else        mfma32_into_vgprs(dp_next, oa[s8], bv[s8], s8 == 0);
         const int e = k + u, g = e >> 2, rr = e & 3;
-        pe[e] = fast_exp2(s_cur[e] * sl2 - l4[g][rr]);
+        // (the inputs are taken up here: without the pins the scale-and-subtract of all sixteen elements runs
+        // ahead of the first MFMA of the phase, with the matrix pipe idle meanwhile)
+        float sx = s_cur[e];
+        MOBA_PIN(sx);
+        pe[e] = fast_exp2(sx * sl2 - l4[g][rr]);
         if (e > 0) {
-          ds[e - 1] = pe[e - 1] * (dp_cur[e - 1] - d4[(e - 1) >> 2][(e - 1) & 3]);
+          float dx = dp_cur[e - 1];
+          MOBA_PIN(dx);
+          ds[e - 1] = pe[e - 1] * (dx - d4[(e - 1) >> 2][(e - 1) & 3]);
           MOBA_PIN(ds[e - 1]);
         }
         if constexpr (decltype(masked_c)::value) {
