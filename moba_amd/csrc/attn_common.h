@@ -66,7 +66,7 @@ inline bool set_layout(TileTables& t, const int64_t* strides) {
   }
   for (int i = 0; i < 4; ++i)
     if (strides[i] <= 0 || (strides[i] & 7)) return false;
-  if (strides[2] > (1 << 23)) return false;
+  if (strides[2] > (1 << 23) || strides[0] >= (1LL << 30)) return false;  // (byte strides of a token fit 32 bits)
   t.q_tok_b = strides[0] * 2; t.q_head_b = strides[1] * 2;
   t.kv_tok_b = strides[2] * 2; t.kv_head_b = strides[3] * 2;
   if (strides[4] != 0) {

@@ -485,6 +485,12 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
     for (int i = 0; i < 4; ++i) raw[i] = src[min(base + 4 * (4 * i + wave_u) + ld_rin, list_rows - 1)];
     raw[4] = src[min(base + lane, list_rows - 1)];
   };
+  uint64_t q_lane_base = 0, do_lane_base = 0;  // this lane's 16 bytes in token 0's row of q and dO, head h
+  auto set_lane_bases = [&]() __attribute__((always_inline)) {
+    const int c16 = ld_pc ^ (ld_rin << 2) ^ (wave_u & 3);  // sw_col16(4*slab + ld_rin, ld_pc) for slab = 4*i + wave
+    q_lane_base = (uint64_t)p.q + (uint64_t)((int64_t)h * p.t.q_head_b + c16 * 16);
+    do_lane_base = (uint64_t)p.dout + (uint64_t)(h * (kHeadDim * 2) + c16 * 16);
+  };
   int toks[5];  // tokens of the rows of the stage whose copies are being issued
   auto prepare_stage = [&](int qi) __attribute__((always_inline)) {
     if (qi < nself) {
@@ -499,18 +505,23 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
   // part g of the 8 row copies of a stage (slab g/2 of Q for even g, of dO for odd g); the last part also
   // brings the softmax statistics.  A copy instruction occupies the wave for tens of cycles while the
   // address unit takes its 64 lanes, so the parts are issued one at a time between MFMAs, not in a burst.
+  // The 16 bytes a lane copies lie at the same place in every row it copies (the swizzled column of row
+  // 4*slab + lane/16 depends on the slab only through slab % 4, which is the wave): with that place added to
+  // the head's base once per head, the address of a copy is one multiply-add of the row's token (tokens and
+  // token strides fit 32 bits).
   auto issue_part = [&](int g, int buf) __attribute__((always_inline)) {
     const uint32_t qdst = lds_base + buf * kQStage;
     const int i = g >> 1;
     const int slab = 4 * i + wave_u;
-    const int row = 4 * slab + ld_rin;
-    const int c16 = sw_col16(row, ld_pc);
-    if ((g & 1) == 0)
-      async_copy16((const char*)p.q + ((kBatched ? q_tok_bytes(p.t, toks[i]) : (int64_t)toks[i] * p.t.q_tok_b) + h * p.t.q_head_b + c16 * 16),
-                   qdst + slab * 1024);
-    else
-      async_copy16((const char*)p.dout + (((int64_t)toks[i] * H + h) * kHeadDim + c16 * 8) * 2,
+    if ((g & 1) == 0) {
+      if constexpr (kBatched)
+        async_copy16((const char*)q_lane_base + q_tok_bytes(p.t, toks[i]), qdst + slab * 1024);
+      else
+        async_copy16((const char*)(q_lane_base + (uint64_t)(uint32_t)toks[i] * (uint32_t)p.t.q_tok_b), qdst + slab * 1024);
+    } else {
+      async_copy16((const char*)(do_lane_base + (uint64_t)(uint32_t)toks[i] * (uint32_t)(H * kHeadDim * 2)),
                    qdst + TQ * kHeadDim * 2 + slab * 1024);
+    }
     if (g == 7 && wave_u < 2) {
       const float* src = (wave_u == 0 ? p.lse2 : p.delta) + ((int64_t)toks[4] * H + h);
       async_copy4(src, qdst + 2 * TQ * kHeadDim * 2 + wave_u * (TQ * 4));
@@ -671,6 +682,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
 
   for (int hq = hkv * rep; hq < (hkv + 1) * rep; ++hq) {
   select_head(hq);
+  set_lane_bases();
   __syncthreads();  // every wave is done with the LDS stages of the previous head
 #pragma unroll
   for (int i = 0; i < 5; ++i) raw[i] = 0;
