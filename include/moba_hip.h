@@ -12,7 +12,9 @@
  * State the library keeps, all of it per device and filled on first use: the number of compute units,
  * which kernels have been allowed their dynamic LDS size, and the address of the array of
  * moba_chunk_mean_static.  First calls may come from several threads at once (the writes are idempotent,
- * the address is guarded by a mutex); nothing else is shared between calls.
+ * the address is guarded by a mutex); nothing else is shared between calls.  One environment variable is read,
+ * once: MOBA_RESIDENT_CUS=<n> (a diagnostic) makes the kernels whose workgroups stay resident occupy only n
+ * compute units' worth of workgroups; results do not depend on it.
  * Inputs are expected to be finite: the attention kernels are compiled without NaN handling, and with an
  * infinity or a NaN in q, k, v or dout the outputs are unspecified (no fault, no hang).  Scores of any finite
  * size are handled (the softmax subtracts a row reference before it exponentiates).
