@@ -586,7 +586,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
     __builtin_amdgcn_sched_barrier(0);
     // The product of element e is formed in the slot of element e+1: an exponential followed at once by
     // an instruction that uses it costs an idle issue cycle.
-    float pe[16], ds[16];
+    float pe[16], ds[16], sx[16], dx[16];
 #pragma unroll
     for (int k = 0; k < 16; k += 2) {
       const int s8 = k >> 1;
@@ -595,15 +595,22 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
         if (u == 0) mfma32_into_vgprs(s_next, qa[s8], bk[s8], s8 == 0);
         else        mfma32_into_vgprs(dp_next, oa[s8], bv[s8], s8 == 0);
         const int e = k + u, g = e >> 2, rr = e & 3;
-        // (the inputs are taken up here: without the pins the scale-and-subtract of all sixteen elements runs
-        // ahead of the first MFMA of the phase, with the matrix pipe idle meanwhile)
-        float sx = s_cur[e];
-        MOBA_PIN(sx);
-        pe[e] = fast_exp2(sx * sl2 - l4[g][rr]);
+        // (the inputs of an element are taken up one slot before the element's own: without the pins the
+        // scale-and-subtract of all sixteen elements runs ahead of the first MFMA of the phase, with the matrix
+        // pipe idle meanwhile; a pin right in front of its use costs a wait state)
+        if (e == 0) {
+          sx[0] = s_cur[0];
+          MOBA_PIN(sx[0]);
+        }
+        if (e + 1 < 16) {
+          sx[e + 1] = s_cur[e + 1];
+          MOBA_PIN(sx[e + 1]);
+        }
+        dx[e] = dp_cur[e];
+        MOBA_PIN(dx[e]);
+        pe[e] = fast_exp2(sx[e] * sl2 - l4[g][rr]);
         if (e > 0) {
-          float dx = dp_cur[e - 1];
-          MOBA_PIN(dx);
-          ds[e - 1] = pe[e - 1] * (dx - d4[(e - 1) >> 2][(e - 1) & 3]);
+          ds[e - 1] = pe[e - 1] * (dx[e - 1] - d4[(e - 1) >> 2][(e - 1) & 3]);
           MOBA_PIN(ds[e - 1]);
         }
         if constexpr (decltype(masked_c)::value) {
@@ -623,7 +630,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
       dma(k >> 1);  // one global -> LDS copy (or nothing) per pair of MFMAs
       __builtin_amdgcn_sched_barrier(0);
     }
-    ds[15] = pe[15] * (dp_cur[15] - d4[3][3]);
+    ds[15] = pe[15] * (dx[15] - d4[3][3]);
     dsb[1][6] = (elem)ds[14];
     dsb[1][7] = (elem)ds[15];
     __builtin_amdgcn_sched_barrier(0);
