@@ -55,7 +55,7 @@ extern "C" {
 
 enum { MOBA_DTYPE_BF16 = 0, MOBA_DTYPE_F16 = 1 };
 
-#define MOBA_ABI_VERSION 106 /* the signatures below; moba_version() returns the number the library was built with */
+#define MOBA_ABI_VERSION 107 /* the signatures below; moba_version() returns the number the library was built with */
 int moba_version(void);
 const char* moba_strerror(int code);
 
@@ -214,14 +214,19 @@ int moba_fwd(const void* q, const void* k, const void* v, void* part_o, float* p
  *   delta [2,S,H] fp32 scratch (rowsum(dO*O), then the LSE in the log2 domain); part_dq [S*H*(K+1), D] elem scratch (the per-slot dQ, rounded as the per-chunk dQ that flash-attn returns to the reference is)
  *   dq, dk, dv: out; dk and dv of a key/value head sum over its query heads
  *   queues [16] int32 scratch: tile counters of the dQ and dK/dV kernels (as in moba_fwd_partials)
+ *   dkv_scratch: moba_bwd_dkv_scratch_bytes(S, Hkv, self_tiles) bytes, 16-byte aligned, or null.  With few key tiles
+ *              (fewer than two per compute unit, S >= 16384) the dK/dV kernel cuts each into up to 4 parts that run
+ *              side by side and leave fp32 sums there, added up in a fixed order (deterministic all the same);
+ *              without the scratch, or when the query returns 0, every tile is one piece.
  *   softmax_scale: as in the forward call */
+size_t moba_bwd_dkv_scratch_bytes(int64_t S, int Hkv, int64_t self_tiles);
 int moba_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out, const float* lse,
              const int32_t* sel, const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest,
              const int32_t* fchunk_tok, const int32_t* chunk_tok, const int32_t* self_tile_prefix,
              const int32_t* tile_seg, const int32_t* self_tile_chunk, const int32_t* chunk_fid, float* delta,
              void* part_dq, void* dq, void* dk, void* dv, int64_t S, int H, int Hkv, int D, int K, int F, int N, int B,
-             int64_t hist_bound, int64_t self_tiles, const int64_t* strides, int32_t* queues, float softmax_scale,
-             int dtype, void* stream);
+             int64_t hist_bound, int64_t self_tiles, const int64_t* strides, int32_t* queues, void* dkv_scratch,
+             int64_t dkv_scratch_bytes, float softmax_scale, int dtype, void* stream);
 
 /* Decode: one query token per sequence against the key/value cache.  Replaces the
  * flash_attn_func call of the adapter's decode branch, moba/wrapper.py:76-82 (full attention

@@ -54,7 +54,30 @@ struct BwdParams {
   uint32_t hk_magic;  // n / (H*K1) == (n * hk_magic) >> hk_shift for every n < 2^31
   uint32_t hk_shift;
   int* queues;        // [16] tile counters, one per XCD, of the dQ kernel and of the dK/dV kernel; zero at the start
+  // Small problems: every key tile of the dK/dV kernel is cut into dkv_split parts (its rows' stages in equal
+  // shares) that run as tiles of their own and leave fp32 sums in part_dkv [tiles * dkv_split][2][128][128],
+  // which bwd_dkv_reduce_kernel adds up in a fixed order.  dkv_split = 1: whole tiles, dk and dv written directly.
+  float* part_dkv;
+  int dkv_split;
 };
+
+// which 128-key tile of which key/value head: the forward's self-tile enumeration over Hkv heads
+struct KvTile {
+  int c, hkv, key0, c0, len;  // chunk, key/value head, first key inside the chunk, first token and length of the chunk
+};
+template <class E>
+__device__ __forceinline__ KvTile decode_kv_tile(const BwdParams<E>& p, int st) {
+  const int Hkv = p.t.Hkv;
+  KvTile t;
+  t.c = p.t.self_tile_chunk[st / Hkv];
+  const int rem = st - p.t.self_tile_prefix[t.c] * Hkv;
+  const int nt = p.t.self_tile_prefix[t.c + 1] - p.t.self_tile_prefix[t.c];
+  t.hkv = rem / nt;
+  t.key0 = (rem - t.hkv * nt) * TM;
+  t.c0 = p.t.chunk_tok[t.c];
+  t.len = p.t.chunk_tok[t.c + 1] - t.c0;
+  return t;
+}
 
 template <class E>
 __global__ __launch_bounds__(256) void bwd_delta_kernel(const typename E::elem* __restrict__ dout,
@@ -422,22 +445,18 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
   __syncthreads();
   const int drawn = __builtin_amdgcn_readfirstlane(*reinterpret_cast<const int*>(smem + kDkvIdSlot));
   const int64_t id = ((int64_t)(drawn / kXcdBlock) * 8 + queue) * kXcdBlock + (drawn % kXcdBlock);
-  if (id >= p.t.self_total / rep) {
+  const int split = p.dkv_split;
+  if (id >= (int64_t)(p.t.self_total / rep) * split) {
     queue = (queue + 1) & 7;
     if (++empty_queues == 8) break;
     continue;
   }
   empty_queues = 0;
-  // ---- which 128-key tile of which key/value head: the forward's self-tile enumeration over Hkv heads ----
-  const int st = (int)id;
-  const int c = p.t.self_tile_chunk[st / Hkv];
-  const int rem = st - p.t.self_tile_prefix[c] * Hkv;
-  const int nt = p.t.self_tile_prefix[c + 1] - p.t.self_tile_prefix[c];
-  const int hkv = rem / nt;
-  const int tin = rem - hkv * nt;
-  const int c0 = p.t.chunk_tok[c];
-  const int len = p.t.chunk_tok[c + 1] - c0;
-  const int key0 = tin * TM;
+  // ---- which part of which 128-key tile (consecutive ids: the parts of one tile) ----
+  const int unit = (int)id;
+  const int part = unit % split;
+  const KvTile kt = decode_kv_tile(p, unit / split);
+  const int c = kt.c, hkv = kt.hkv, c0 = kt.c0, len = kt.len, key0 = kt.key0;
   const int mykey = key0 + wave * 32 + n;        // position inside the chunk
   const bool key_valid = mykey < len;
 
@@ -689,17 +708,20 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
 
   for (int hq = hkv * rep; hq < (hkv + 1) * rep; ++hq) {
   select_head(hq);
+  // this part's share of the head's stages
+  const int q_first = (int)((int64_t)ntile * part / split), q_end = (int)((int64_t)ntile * (part + 1) / split);
+  if (q_end == q_first) continue;  // (uniform)
   set_lane_bases();
   __syncthreads();  // every wave is done with the LDS stages of the previous head
 #pragma unroll
   for (int i = 0; i < 5; ++i) raw[i] = 0;
-  fetch_rows(0);
-  issue_stage(0, 0);
-  fetch_rows(1);
+  fetch_rows(q_first);
+  issue_stage(q_first, 0);
+  fetch_rows(q_first + 1);
   wait_vmem();
   __syncthreads();
-  if (ntile > 1) issue_stage(1, 1);
-  fetch_rows(2);
+  if (q_end - q_first > 1) issue_stage(q_first + 1, 1);
+  fetch_rows(q_first + 2);
 
   // S of block 0 (a phase A whose softmax half works on zeros and is discarded)
   f32x16 sA, dA, sB, dB;
@@ -715,11 +737,11 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
     load_frags(smem, 1);
   }
   int buf = 0;
-  for (int qi = 0; qi < ntile; ++qi) {
+  for (int qi = q_first; qi < q_end; ++qi) {
     const char* qs = smem + buf * kQStage;
     const int buf1 = buf == 2 ? 0 : buf + 1;
     const int buf2 = buf1 == 2 ? 0 : buf1 + 1;
-    const bool has_next = qi + 1 < ntile;
+    const bool has_next = qi + 1 < q_end;
     const bool is_self = qi < nself;
     // number of real rows in this stage, and for self stages the chunk position of row 0
     const int rows_here = is_self ? min(TQ, self_rows - qi * TQ) : min(TQ, list_rows - (qi - nself) * TQ);
@@ -754,7 +776,19 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
   wait_vmem();  // (the copies past the last stage: nothing may be on its way into LDS when the workgroup ends)
   }  // query heads
 
-  if (key_valid) {
+  if (split > 1) {
+    // this part's sums, unscaled, in fp32: [dk, dv][key of the tile][128]
+    float* dst = p.part_dkv + (int64_t)unit * (2 * TM * kHeadDim) + (wave * 32 + n) * kHeadDim + 4 * hh;
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        *reinterpret_cast<f32x4*>(dst + 32 * db + 8 * g) =
+            f32x4{dkacc[db][4 * g + 0], dkacc[db][4 * g + 1], dkacc[db][4 * g + 2], dkacc[db][4 * g + 3]};
+        *reinterpret_cast<f32x4*>(dst + TM * kHeadDim + 32 * db + 8 * g) =
+            f32x4{dvacc[db][4 * g + 0], dvacc[db][4 * g + 1], dvacc[db][4 * g + 2], dvacc[db][4 * g + 3]};
+      }
+  } else if (key_valid) {
     const int64_t off = ((int64_t)(c0 + mykey) * Hkv + hkv) * kHeadDim;
 #pragma unroll
     for (int db = 0; db < 4; ++db)
@@ -773,6 +807,34 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
 #undef MOBA_PIN
 }
 
+// dk, dv of the 128-key tiles from the fp32 sums of their parts, added in the order of the parts.
+// Sixteen workgroups per tile; a thread owns four consecutive elements of one key (coalesced 16-byte loads).
+template <class E>
+__global__ __launch_bounds__(256) void bwd_dkv_reduce_kernel(const BwdParams<E> p) {
+  MOBA_ELEM_TYPES(E)
+  const int tile = blockIdx.x >> 4;
+  const KvTile kt = decode_kv_tile(p, tile);
+  const int in_tile = (blockIdx.x & 15) * 256 + threadIdx.x;  // 128 keys x 32 groups of four elements
+  const int key = in_tile >> 5, d = (in_tile & 31) * 4;
+  if (kt.key0 + key >= kt.len) return;
+  const int split = p.dkv_split;
+  const float* src = p.part_dkv + (int64_t)tile * split * (2 * TM * kHeadDim) + key * kHeadDim + d;
+  f32x4 sk = {0.f, 0.f, 0.f, 0.f}, sv = sk;
+  for (int r = 0; r < split; ++r) {
+    const float* s = src + (int64_t)r * (2 * TM * kHeadDim);
+    sk += *reinterpret_cast<const f32x4*>(s);
+    sv += *reinterpret_cast<const f32x4*>(s + TM * kHeadDim);
+  }
+  const int64_t off = ((int64_t)(kt.c0 + kt.key0 + key) * p.t.Hkv + kt.hkv) * kHeadDim + d;
+  u32x2 wk, wv;
+  wk[0] = pack2<E>(sk[0] * p.scale, sk[1] * p.scale);
+  wk[1] = pack2<E>(sk[2] * p.scale, sk[3] * p.scale);
+  wv[0] = pack2<E>(sv[0], sv[1]);
+  wv[1] = pack2<E>(sv[2], sv[3]);
+  *reinterpret_cast<u32x2*>(p.dk + off) = wk;
+  *reinterpret_cast<u32x2*>(p.dv + off) = wv;
+}
+
 }  // namespace moba
 
 using namespace moba;
@@ -781,7 +843,7 @@ template <class E>
 static int launch_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out, const float* lse,
                       const int32_t* sel, const int32_t* chunk_fid, float* delta, void* part_dq, void* dq, void* dk,
                       void* dv, const TileTables& t, int64_t S, int H, int D, int K, float softmax_scale, int64_t grid_q,
-                      int64_t grid_kv, int* queues, hipStream_t st) {
+                      int64_t grid_kv, int* queues, float* part_dkv, int dkv_split, hipStream_t st) {
   LaunchCheck launch_check;
   typedef typename E::elem elem;
   BwdParams<E> p;
@@ -789,6 +851,8 @@ static int launch_bwd(const void* dout, const void* q, const void* k, const void
   p.lse = lse; p.delta = delta; p.lse2 = delta + S * H; p.part_dq = (elem*)part_dq; p.dk = (elem*)dk; p.dv = (elem*)dv;
   p.chunk_fid = chunk_fid;
   p.queues = queues;
+  p.part_dkv = part_dkv;
+  p.dkv_split = dkv_split;
   p.t = t;
   p.scale = softmax_scale > 0.f ? softmax_scale : (float)(1.0 / sqrt((double)D));
   p.scale_log2 = softmax_scale > 0.f ? (float)(1.4426950408889634 * (double)softmax_scale)
@@ -816,10 +880,30 @@ static int launch_bwd(const void* dout, const void* q, const void* k, const void
                      (const elem*)part_dq, sel, (elem*)dq, rows, K + 1);
   if (batched) hipLaunchKernelGGL((bwd_dkv_kernel<E, true>), dim3((unsigned)grid_kv), dim3(256), kBwdDkvLds, st, p);
   else hipLaunchKernelGGL((bwd_dkv_kernel<E, false>), dim3((unsigned)grid_kv), dim3(256), kBwdDkvLds, st, p);
+  if (dkv_split > 1)
+    hipLaunchKernelGGL(bwd_dkv_reduce_kernel<E>, dim3((unsigned)(t.self_total / t.rep) * 16), dim3(256), 0, st, p);
   return launch_check.result();
 }
 
 extern "C" int moba_bwd_tile_rows(void) { return TM; }
+
+// Parts per key tile of the dK/dV kernel.  With fewer tiles than two per compute unit the tiles of the first
+// chunks of a sequence, whose gather lists are the longest, set the kernel's time while most of the chip is
+// idle: they are cut into parts then (at most 4: every part leaves 128 KiB of fp32 sums to be added up).
+// Problems below 16384 tokens are too short for the parts' extra traffic to pay.
+static int dkv_split_for(int64_t S, int64_t tiles) {
+  const int cus = resident_compute_units();
+  if (cus <= 0 || tiles <= 0 || tiles >= 2 * (int64_t)cus || S < 16384) return 1;
+  const int64_t r = (3 * (int64_t)cus + tiles - 1) / tiles;
+  return (int)(r < 1 ? 1 : (r > 4 ? 4 : r));
+}
+
+extern "C" size_t moba_bwd_dkv_scratch_bytes(int64_t S, int Hkv, int64_t self_tiles) {
+  if (S <= 0 || Hkv <= 0 || self_tiles <= 0) return 0;
+  const int64_t tiles = self_tiles * Hkv;
+  const int split = dkv_split_for(S, tiles);
+  return split > 1 ? (size_t)tiles * split * (2 * TM * kHeadDim) * sizeof(float) : 0;
+}
 
 extern "C" int moba_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out,
                         const float* lse, const int32_t* sel, const int32_t* seg_off, const int32_t* tile_off,
@@ -828,7 +912,7 @@ extern "C" int moba_bwd(const void* dout, const void* q, const void* k, const vo
                         const int32_t* chunk_fid, float* delta, void* part_dq,
                         void* dq, void* dk, void* dv, int64_t S, int H, int Hkv, int D, int K, int F, int N, int B,
                         int64_t hist_bound, int64_t self_tiles, const int64_t* strides, int32_t* queues,
-                        float softmax_scale, int dtype, void* stream) {
+                        void* dkv_scratch, int64_t dkv_scratch_bytes, float softmax_scale, int dtype, void* stream) {
   if (!dout || !q || !k || !v || !out || !lse || !chunk_tok || !self_tile_prefix || !self_tile_chunk || !delta ||
       !part_dq || !dq || !dk || !dv || !queues)
     return MOBA_ERR_ARG;
@@ -857,10 +941,17 @@ extern "C" int moba_bwd(const void* dout, const void* q, const void* k, const vo
   t.hist_bound = (K > 0) ? (int)hist_bound : 0;
   t.self_total = (int)(self_tiles * H);
   if (!set_layout(t, strides)) return MOBA_ERR_ARG;
+  // the key tiles are cut into parts only if the caller brought the scratch for their sums
+  const int64_t kv_tiles = self_tiles * Hkv;
+  int dkv_split = dkv_split_for(S, kv_tiles);
+  if (dkv_split > 1 && (!dkv_scratch || ((uintptr_t)dkv_scratch & 15) ||
+                        dkv_scratch_bytes < (int64_t)(kv_tiles * dkv_split * (2 * TM * kHeadDim) * sizeof(float))))
+    dkv_split = 1;
+  if (kv_tiles * dkv_split >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
   hipStream_t st = (hipStream_t)stream;
   return dtype == MOBA_DTYPE_F16
              ? launch_bwd<F16>(dout, q, k, v, out, lse, sel, chunk_fid, delta, part_dq, dq, dk, dv, t, S, H, D, K,
-                               softmax_scale, grid_q, grid_kv, queues, st)
+                               softmax_scale, grid_q, grid_kv, queues, (float*)dkv_scratch, dkv_split, st)
              : launch_bwd<Bf16>(dout, q, k, v, out, lse, sel, chunk_fid, delta, part_dq, dq, dk, dv, t, S, H, D, K,
-                                softmax_scale, grid_q, grid_kv, queues, st);
+                                softmax_scale, grid_q, grid_kv, queues, (float*)dkv_scratch, dkv_split, st);
 }

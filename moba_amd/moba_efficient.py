@@ -306,12 +306,16 @@ def _backward(dout, q, k, v, out, lse, sel, seg_off, seg_dest, plan: MobaPlan, s
     delta = torch.empty((2, S, H), dtype=torch.float32, device=dev)
     part_dq = torch.empty((S * H * (K + 1), D), dtype=q.dtype, device=dev)
     queues = torch.empty(16, dtype=torch.int32, device=dev)  # tile counters of the two backward kernels (zeroed there)
+    # small problems: the fp32 sums of the parts the dK/dV kernel cuts its key tiles into (0 bytes otherwise)
+    kv_bytes = int(lib.moba_bwd_dkv_scratch_bytes(S, Hkv, plan.self_tiles))
+    kv_scratch = torch.empty(kv_bytes, dtype=torch.uint8, device=dev) if kv_bytes else None
     _lib.check(lib.moba_bwd(_ptr(dout), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(sel), _ptr(seg_off),
                             _ptr(tile_off), _ptr(seg_dest), _ptr(t.get("fchunk_tok")), _ptr(t["chunk_tok"]),
                             _ptr(t["self_tile_prefix"]), _ptr(tile_seg), _ptr(t["self_tile_chunk"]),
                             _ptr(t.get("chunk_fid")), _ptr(delta), _ptr(part_dq), _ptr(dq), _ptr(dk), _ptr(dv),
                             S, H, Hkv, D, K, plan.F, plan.N, plan.chunk_size, plan.hist_tile_bound(H),
-                            plan.self_tiles, _strides(q, k), _ptr(queues), scale, _dtype_code(q), _stream(dev)),
+                            plan.self_tiles, _strides(q, k), _ptr(queues), _ptr(kv_scratch), kv_bytes, scale,
+                            _dtype_code(q), _stream(dev)),
                "moba_bwd")
     return dq, dk, dv
 

@@ -304,6 +304,55 @@ def test_backward_is_deterministic():
         assert torch.equal(a, b)
 
 
+def test_key_tiles_cut_into_parts():
+    """With few key tiles (here 16384 tokens x 1 key/value head = 128 tiles on 256 compute units) the dK/dV kernel
+    cuts every tile into parts that leave fp32 sums for a reduction kernel: grouped-query heads, three sequences
+    with partial last chunks.  The result is deterministic, equals the uncut kernel's up to the rounding of the
+    different summation order, and both lie within the tolerance of the oracle."""
+    from moba_amd import _lib, moba_attn_varlen_gqa
+    from moba_amd import moba_efficient as E
+    from moba_amd.plan import make_plan
+    heads, kv_heads, B, topk = 2, 1, 1024, 3
+    q, _, _, do, cu, mx = make_case(3, 16384, heads, seed=21)
+    _, k, v, _, _, _ = make_case(3, 16384, kv_heads, seed=22)
+    cu_t = torch.tensor(cu, dtype=torch.int32, device="cuda")
+    lib = _lib.load()
+    plan = make_plan(cu_t, B, topk)
+    assert lib.moba_bwd_dkv_scratch_bytes(16384, kv_heads, plan.self_tiles) > 0
+
+    def run():
+        qg, kg, vg = (x.cuda().requires_grad_(True) for x in (q, k, v))
+        out = moba_attn_varlen_gqa(qg, kg, vg, cu_t, mx, B, topk)
+        out.backward(do.cuda())
+        return out.detach(), qg.grad, kg.grad, vg.grad
+
+    cut, again = run(), run()
+    for a, b in zip(cut, again):
+        assert torch.equal(a, b)
+    real = lib.moba_bwd_dkv_scratch_bytes
+    try:
+        lib.moba_bwd_dkv_scratch_bytes = lambda *a: 0   # no scratch: every key tile in one piece
+        whole = run()
+    finally:
+        lib.moba_bwd_dkv_scratch_bytes = real
+    assert torch.equal(cut[0], whole[0]) and torch.equal(cut[1], whole[1])
+    for name, a, b in (("dk", cut[2], whole[2]), ("dv", cut[3], whole[3])):
+        e = (a.float() - b.float()).abs()
+        assert e.max() <= 2.0 ** -7 * b.float().abs().max() and (e > 0).float().mean() < 0.05, (name, e.max().item())
+    # ... and the oracle, on expanded key/value heads with the kernel's own selection
+    sel = E.gate_topk(q.cuda(), E.chunk_mean(k.cuda(), plan), plan).cpu()
+    qc = q.clone().requires_grad_(True)
+    kc, vc = (x.clone().requires_grad_(True) for x in (k, v))
+    rep = heads // kv_heads
+    ref = O.moba_attn_varlen_oracle(qc, torch.repeat_interleave(kc, rep, dim=1), torch.repeat_interleave(vc, rep, dim=1),
+                                    cu, mx, B, topk, sel=sel)
+    ref.backward(do.float())
+    for name, got_g, want_g in (("dk", cut[2], kc.grad), ("dv", cut[3], vc.grad)):
+        e = (got_g.cpu().float() - want_g.float()).abs()
+        scale = want_g.abs().max().clamp_min(1.0)
+        assert e.max() < MAX_ABS * scale and e.mean() < MEAN_ABS * rep, (name, e.max().item(), e.mean().item())
+
+
 def test_float16_large_gradients_stay_finite():
     """dQ = scale * dS K is summed from per-chunk partials kept in the element type.  The partials are
     scaled before they are rounded, so they leave the fp16 range only where dQ itself would: here
