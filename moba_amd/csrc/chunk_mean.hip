@@ -61,6 +61,20 @@ __global__ __launch_bounds__(256) void chunk_mean_partial_kernel(
   for (int e = 0; e < 8; ++e) dst[e] = acc[e];
 }
 
+// fp64 -> fp32 rounded to odd (an inexact result gets the neighbour whose last bit is set): rounding that fp32
+// value to bf16 or fp16 to nearest-even then gives what rounding the fp64 value once would, where two
+// nearest-even roundings in a row can land on the wrong side of a tie.
+__device__ __forceinline__ float round_to_odd_f32(double x) {
+  float f = (float)x;  // nearest-even
+  if ((double)f != x) {
+    uint32_t u = __builtin_bit_cast(uint32_t, f);
+    if (fabs((double)f) > fabs(x)) u -= 1;  // the neighbour toward zero (never crosses zero: |f| > |x| >= 0)
+    u |= 1;
+    f = __builtin_bit_cast(float, u);
+  }
+  return f;
+}
+
 template <class E>
 __global__ __launch_bounds__(256) void chunk_mean_finish_kernel(
     const double* __restrict__ partial, typename E::elem* __restrict__ kbar, int HD8, int B, int nsplit, int F) {
@@ -80,7 +94,7 @@ __global__ __launch_bounds__(256) void chunk_mean_finish_kernel(
   elem8 o;
   const double inv = (double)B;
 #pragma unroll
-  for (int e = 0; e < 8; ++e) o[e] = (elem)(float)(acc[e] / inv);
+  for (int e = 0; e < 8; ++e) o[e] = (elem)round_to_odd_f32(acc[e] / inv);
   *reinterpret_cast<elem8*>(kbar + idx * 8) = o;
 }
 

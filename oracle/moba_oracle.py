@@ -94,8 +94,10 @@ def chunk_mean(k: torch.Tensor, cu_seqlens: Sequence[int], chunk_size: int) -> t
     The reference takes ``.mean(dim=1)`` of a bf16 view and then ``.float()``
     (moba/moba_efficient.py:335-340): accumulate wide, round once to bf16.
     The oracle accumulates in fp64 (exact for any realistic bf16 data, hence
-    independent of summation order), divides by B in fp64, rounds to fp32 and
-    then to the input dtype (round-to-nearest-even both times).
+    independent of summation order), divides by B in fp64 and rounds that
+    quotient once, to nearest-even, to the input dtype (through an fp32 value
+    rounded to odd, so that the second rounding cannot land on the wrong side
+    of a tie: ``round_once``).
     Returns [F, H, D] in k.dtype.
     """
     meta = calc_chunks(cu_seqlens, chunk_size)
@@ -107,8 +109,22 @@ def chunk_mean(k: torch.Tensor, cu_seqlens: Sequence[int], chunk_size: int) -> t
         blk = k[s0:s0 + chunk_size].to(torch.float64)
         assert blk.shape[0] == chunk_size
         mean64 = blk.sum(dim=0) / float(chunk_size)
-        out[i] = mean64.to(torch.float32).to(k.dtype)
+        out[i] = round_once(mean64, k.dtype)
     return out
+
+
+def round_once(x64: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """fp64 -> bf16/fp16 with a single round-to-nearest-even.  torch converts through fp32, and two nearest-even
+    roundings in a row can differ from one (a value just above a tie of the narrow type that fp32 rounds onto
+    the tie); rounding the intermediate fp32 to odd instead makes the second rounding see on which side of every
+    tie the fp64 value lies."""
+    f = x64.to(torch.float32)
+    inexact = f.to(torch.float64) != x64
+    away = f.to(torch.float64).abs() > x64.abs()
+    u = f.view(torch.int32)
+    u = torch.where(inexact & away, u - 1, u)      # the fp32 neighbour toward zero (bit patterns grow with |value|)
+    u = torch.where(inexact, u | 1, u)
+    return u.view(torch.float32).to(dtype)
 
 
 # --------------------------------------------------------------------------

@@ -35,6 +35,23 @@ def test_chunk_mean_bit_exact(batch, seqlen, heads, B):
     assert torch.equal(got.view(torch.int16), want.view(torch.int16))
 
 
+def test_chunk_mean_rounds_once():
+    """Means just above, just below and on a tie of the element type (see the oracle's test of the same name):
+    the kernel rounds the fp64 mean once."""
+    from moba_amd import moba_efficient as E
+    for dtype, step, tiny in ((torch.bfloat16, 2.0 ** -7, 2.0 ** -38), (torch.float16, 2.0 ** -10, 2.0 ** -24)):
+        k = torch.zeros((8, 1, 128), dtype=dtype)
+        k[0, 0, :] = 4.0
+        k[1, 0, 0] = 2 * step; k[2, 0, 0] = tiny
+        k[1, 0, 1] = 2 * step; k[2, 0, 1] = -tiny
+        k[1, 0, 2] = 2 * step
+        k[1, 0, 3] = 6 * step
+        plan = _plan([0, 8], 4, 2)
+        got = E.chunk_mean(k.cuda(), plan).cpu()
+        assert torch.equal(got, O.chunk_mean(k, [0, 8], 4))
+        assert got[0, 0, 0].item() == 1 + step and got[0, 0, 1].item() == 1.0 and got[0, 0, 3].item() == 1 + 2 * step
+
+
 def test_chunk_mean_exact_integers():
     from moba_amd import moba_efficient as E
     g = torch.Generator().manual_seed(2)

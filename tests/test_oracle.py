@@ -76,6 +76,38 @@ def test_chunk_mean_vs_torch_mean():
     assert (diff == 0).float().mean() > 0.995
 
 
+def test_chunk_mean_rounds_once():
+    """A mean just above the tie between two neighbours of the narrow type: 4 + 2^-6 + 2^-38 over 4 tokens is
+    1 + 2^-8 + 2^-40.  One rounding gives the upper neighbour; rounding to fp32 first lands on the tie itself
+    (1 + 2^-8), which nearest-even then sends down.  Known answers, bf16 and fp16 (tie of 1 and 1 + 2^-10 is
+    1 + 2^-11: 4 + 2^-9 + 2^-24, the smallest fp16), plus the mirror image just below a tie and an exact tie."""
+    for dtype, step, tiny in ((torch.bfloat16, 2.0 ** -7, 2.0 ** -38), (torch.float16, 2.0 ** -10, 2.0 ** -24)):
+        k = torch.zeros((8, 1, 8), dtype=dtype)
+        k[0, 0, :] = 4.0
+        k[1, 0, 0] = 2 * step; k[2, 0, 0] = tiny            # just above the tie  -> 1 + step
+        k[1, 0, 1] = 2 * step; k[2, 0, 1] = -tiny         # just below the tie  -> 1
+        k[1, 0, 2] = 2 * step                                      # the tie itself      -> 1 (even)
+        k[1, 0, 3] = 6 * step                                      # tie of 1+step, 1+2step -> 1 + 2 step (even)
+        kb = O.chunk_mean(k, [0, 8], 4).double()
+        assert kb.shape == (1, 1, 8)
+        assert kb[0, 0, 0] == 1 + step and kb[0, 0, 1] == 1.0 and kb[0, 0, 2] == 1.0 and kb[0, 0, 3] == 1 + 2 * step
+        assert (kb[0, 0, 4:] == 1.0).all()
+    # the helper against exact rational arithmetic on random fp64 values near and far from ties
+    from fractions import Fraction
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(2000, generator=g, dtype=torch.float64)
+    x[:500] = (1 + torch.randint(0, 256, (500,), generator=g).double() * 2.0 ** -8) * (1 + (torch.rand(500, generator=g, dtype=torch.float64) - 0.5) * 2.0 ** -30)
+    got = O.round_once(x, torch.bfloat16).double()
+    for xi, gi in zip(x.tolist(), got.tolist()):
+        f = Fraction(xi)
+        e = math.floor(math.log2(abs(xi)))
+        ulp = Fraction(2) ** (e - 7)
+        lo = (f / ulp).__floor__() * ulp
+        hi = lo + ulp
+        want = lo if (f - lo < hi - f or (f - lo == hi - f and (lo / ulp) % 2 == 0)) else hi
+        assert Fraction(gi) == want, (xi, gi, float(want))
+
+
 # ---------------------------------------------------------------- gate
 def test_gate_scores_bruteforce():
     q, k, v, _, cu, _ = make_case(3, 192, 2, head_dim=16, seed=3)
