@@ -4,6 +4,7 @@ reproducing the reference's own test matrix and data recipe
 goes through the C ABI."""
 
 import itertools
+import os
 
 import numpy as np
 import pytest
@@ -318,7 +319,9 @@ def test_key_tiles_cut_into_parts():
     cu_t = torch.tensor(cu, dtype=torch.int32, device="cuda")
     lib = _lib.load()
     plan = make_plan(cu_t, B, topk)
-    assert lib.moba_bwd_dkv_scratch_bytes(16384, kv_heads, plan.self_tiles) > 0
+    if lib.moba_bwd_dkv_scratch_bytes(16384, kv_heads, plan.self_tiles) == 0:
+        assert "MOBA_RESIDENT_CUS" in os.environ     # (only the diagnostic that shrinks the chip turns the parts off)
+        pytest.skip("the key tiles are not cut with MOBA_RESIDENT_CUS set")
 
     def run():
         qg, kg, vg = (x.cuda().requires_grad_(True) for x in (q, k, v))
