@@ -55,7 +55,7 @@ extern "C" {
 
 enum { MOBA_DTYPE_BF16 = 0, MOBA_DTYPE_F16 = 1 };
 
-#define MOBA_ABI_VERSION 107 /* the signatures below; moba_version() returns the number the library was built with */
+#define MOBA_ABI_VERSION 108 /* the signatures below; moba_version() returns the number the library was built with */
 int moba_version(void);
 const char* moba_strerror(int code);
 
@@ -167,7 +167,13 @@ int moba_tile_tables(const int32_t* seg_off, int32_t* tile_off, int32_t* tile_se
 /* Attention.  Replaces MixedAttention.forward, moba/moba_efficient.py:69-183 (two
  * flash-attn varlen forwards and the LSE merge), and with K = 0 and one chunk per
  * sequence the full-causal case of moba/moba_efficient.py:318-321.
- *   part_o [S*H*(K+1), D] elem and part_lse [S*H*(K+1)] fp32: per-slot partial results
+ *   part_o [key_split*S*H*(K+1), D] elem and part_lse [key_split*S*H*(K+1)] fp32: per-slot partial results
+ *   key_split: 1, or for small problems the power of two (up to 8) that moba_fwd_key_split() names: the kernel
+ *              then cuts the keys of every history tile into that many parts, each a tile of its own, so that a
+ *              problem of a few hundred tiles still spreads evenly over the compute units; the merge takes the
+ *              parts as further slots (part g of a slot row lies S*H*(K+1) rows behind part g-1).  Refused
+ *              (MOBA_ERR_ARG) for problems large enough for the resident-workgroup kernel or when B is not a
+ *              multiple of 64*key_split.  The same value goes to moba_fwd_partials and moba_fwd_merge.
  *   self_tile_prefix [N+1] int32: prefix sum of ceil(chunk_len / moba_fwd_tile_rows())
  *   self_tile_chunk [self_tile_prefix[N]] int32: the chunk of each of those tiles
  *   tile_off, tile_seg: from moba_build_lists or moba_tile_tables with tile_rows = moba_fwd_tile_rows()
@@ -193,16 +199,18 @@ int moba_fwd_partials(const void* q, const void* k, const void* v, void* part_o,
                       const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest,
                       const int32_t* fchunk_tok, const int32_t* chunk_tok, const int32_t* self_tile_prefix,
                       const int32_t* tile_seg, const int32_t* self_tile_chunk, int64_t S, int H, int Hkv, int D, int K,
-                      int F, int N, int B, int64_t hist_bound, int64_t self_tiles, const int64_t* strides,
-                      int32_t* queues, int32_t* redo, float softmax_scale, int dtype, void* stream);
+                      int F, int N, int B, int64_t hist_bound, int64_t self_tiles, int key_split,
+                      const int64_t* strides, int32_t* queues, int32_t* redo, float softmax_scale, int dtype,
+                      void* stream);
 int moba_fwd_merge(const void* part_o, const float* part_lse, const int32_t* sel, void* out, float* lse, int64_t S,
-                   int H, int D, int K, int dtype, void* stream);
+                   int H, int D, int K, int key_split, int dtype, void* stream);
+int moba_fwd_key_split(int64_t S, int H, int K, int B, int64_t hist_bound, int64_t self_tiles);
 int moba_fwd(const void* q, const void* k, const void* v, void* part_o, float* part_lse, const int32_t* sel,
              const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest, const int32_t* fchunk_tok,
              const int32_t* chunk_tok, const int32_t* self_tile_prefix, const int32_t* tile_seg,
              const int32_t* self_tile_chunk, void* out, float* lse, int64_t S, int H, int Hkv, int D, int K, int F,
-             int N, int B, int64_t hist_bound, int64_t self_tiles, const int64_t* strides, int32_t* queues,
-             int32_t* redo, float softmax_scale, int dtype, void* stream);
+             int N, int B, int64_t hist_bound, int64_t self_tiles, int key_split, const int64_t* strides,
+             int32_t* queues, int32_t* redo, float softmax_scale, int dtype, void* stream);
 
 /* Backward.  Replaces MixedAttention.backward, moba/moba_efficient.py:185-267, and the
  * autograd scatter of its gathered gradients.  Deterministic (no floating-point atomics).

@@ -37,6 +37,11 @@ struct TileTables {
   // t / batch_rows at position t % batch_rows; batch_rows = 0 for one affine range of tokens
   int batch_rows;
   int64_t q_batch_b, kv_batch_b;
+  // forward, one workgroup per tile id only: every history tile is cut into 1 << key_split_log2 parts along its
+  // keys, each a tile of its own whose partial goes to slot row `dest + part * part_stride` (0, 0 elsewhere)
+  int key_split_log2, part_stride;
+  int xcd_block_log2;  // ... ids reach the XCDs in runs of 1 << xcd_block_log2
+  int self_first;      // ... the self tiles take the first ids (they are the longer ones once the history tiles are cut)
 };
 
 // byte offset of the row of token `tok` (without the head term) in q and in k, v
@@ -59,6 +64,7 @@ __device__ __forceinline__ int64_t kv_tok_bytes(const TileTables& t, int tok) {
 constexpr int kStrideEntries = 7;
 inline bool set_layout(TileTables& t, const int64_t* strides) {
   t.batch_rows = 0; t.q_batch_b = 0; t.kv_batch_b = 0;
+  t.key_split_log2 = 0; t.part_stride = 0; t.xcd_block_log2 = 6; t.self_first = 0;
   if (!strides) {
     t.q_tok_b = (int64_t)t.H * kHeadDim * 2; t.q_head_b = kHeadDim * 2;
     t.kv_tok_b = (int64_t)t.Hkv * kHeadDim * 2; t.kv_head_b = kHeadDim * 2;
@@ -100,11 +106,12 @@ static __global__ void zero_queues_kernel(int* queues, int* also) {
   if (also && threadIdx.x == 0) *also = 0;
 }
 
-// Workgroup ids are dealt round-robin to the 8 XCDs; give each XCD runs of kXcdBlock
-// consecutive logical tiles so that tiles sharing a K/V chunk share an L2.
-__device__ __forceinline__ int logical_tile_id() {
+// Workgroup ids are dealt round-robin to the 8 XCDs; give each XCD runs of 1 << block_log2 (at most kXcdBlock)
+// consecutive logical tiles so that tiles sharing a K/V chunk share an L2.  (A grid of few tiles takes shorter
+// runs: whole runs of 64 would leave some XCDs with twice the tiles of others, or with none.)
+__device__ __forceinline__ int logical_tile_id(int block_log2) {
   const int x = blockIdx.x & 7, y = blockIdx.x >> 3;
-  return ((y / kXcdBlock) * 8 + x) * kXcdBlock + (y % kXcdBlock);
+  return ((((y >> block_log2) << 3) + x) << block_log2) + (y & ((1 << block_log2) - 1));
 }
 
 // Tile decoding in steps, so that a kernel can start the key/value copies (which need only the

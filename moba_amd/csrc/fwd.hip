@@ -241,6 +241,7 @@ __global__ __launch_bounds__(512, 2) void moba_fwd_kernel(const FwdParams<E> p) 
   int dest_done = 0, rows_done = 0, id_done = 0;
   bool valid_done = false;
   int list_pos = blockIdx.x;  // kTilesListed: position in the list of the next tile
+  int key_part = 0;           // kTilePerGroup: which part of a history tile's keys this workgroup takes
   if constexpr (kFixedRef) {
     if (tid == 0) *reinterpret_cast<int*>(smem + kFwdRedoWord) = 0;  // first read many barriers from here
   }
@@ -353,7 +354,24 @@ __global__ __launch_bounds__(512, 2) void moba_fwd_kernel(const FwdParams<E> p) 
         if (!decode_tile_head(pn.t, listed, t, kFwdTileRows)) t.nkeys = -1;  // (cannot happen: listed ids are tiles)
       }
     } else {
-      if (!decode_tile_head(pn.t, logical_tile_id(), t, kFwdTileRows)) return;
+      // the parts of the history tiles (hist_bound << ks ids, the part in the low bits) and the self tiles,
+      // whichever kind takes longer first: workgroups start in the order of their ids
+      int logical = logical_tile_id(pn.t.xcd_block_log2);
+      const int ks = pn.t.key_split_log2;
+      const int parts_end = pn.t.hist_bound << ks;
+      int hist_part = pn.t.self_first ? logical - pn.t.self_total : (logical < parts_end ? logical : -1);
+      if (hist_part >= parts_end) return;
+      if (hist_part >= 0) {
+        key_part = hist_part & ((1 << ks) - 1);
+        logical = hist_part >> ks;
+      } else {
+        logical = pn.t.hist_bound + (pn.t.self_first ? logical : logical - parts_end);
+      }
+      if (!decode_tile_head(pn.t, logical, t, kFwdTileRows)) return;
+      if (t.base >= 0) {  // this part's share of the chunk's keys
+        t.nkeys >>= ks;
+        t.kv_tok0 += key_part * t.nkeys;
+      }
     }
     int q_tok = 0, q_head = 0;  // token and head of this lane's query row
     if (t.row_count > 0) {
@@ -374,7 +392,10 @@ __global__ __launch_bounds__(512, 2) void moba_fwd_kernel(const FwdParams<E> p) 
       }
 
       // the per-row half (queued: decoded when the Q rows were requested, see prefetch_q), then the Q rows
-      if constexpr (!kQueued) decode_tile_rows(pn.t, tx >> 6, er, decode_tile_row_entry(pn.t, er, t), t);
+      if constexpr (!kQueued) {
+        decode_tile_rows(pn.t, tx >> 6, er, decode_tile_row_entry(pn.t, er, t), t);
+        if constexpr (kMode == kTilePerGroup) t.dest += key_part * pn.t.part_stride;  // (part 0 for a self tile)
+      }
       limit = t.limit;
       min_limit = __builtin_amdgcn_readfirstlane(t.wave_min_limit);
       row_valid = er < t.row_count;
@@ -674,7 +695,7 @@ template <class E>
 __global__ __launch_bounds__(256) void moba_merge_kernel(const typename E::elem* __restrict__ part_o,
                                                          const float* __restrict__ part_lse,
                                                          const int* __restrict__ sel, typename E::elem* __restrict__ out,
-                                                         float* __restrict__ lse, int64_t rows, int K1) {
+                                                         float* __restrict__ lse, int64_t rows, int K1, int parts) {
   MOBA_ELEM_TYPES(E)
   const int64_t row_raw = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
   const bool row_ok = row_raw < rows;
@@ -684,26 +705,32 @@ __global__ __launch_bounds__(256) void moba_merge_kernel(const typename E::elem*
   const float* pl = part_lse + row * K1;
   const int* ps = sel + row * K;
   const elem* po = part_o + row * K1 * kHeadDim + c8 * 8;
+  const elem* const po0 = po;  // the self slot: always written
   // Lane c8 of the row's group fetches the LSE and the presence of slot j0 + c8, so the slot
   // statistics cost one round trip per 16 slots; weights travel by lane shuffles.  Absent slots
-  // are redirected to slot 0 with weight 0, so the partial-output loads are unconditional and
+  // are redirected to the self slot with weight 0, so the partial-output loads are unconditional and
   // eight of them are in flight together.  Slots are accumulated in ascending order.
+  // With `parts` > 1 the history slots hold `parts` partials each (the forward cut the chunks' keys): those of
+  // part g lie rows * K1 slot rows behind those of part g - 1; the self slot has part 0 only.
+  const int64_t part_rows = rows * K1;
   float mx = -INFINITY;
-  for (int j0 = 0; j0 < K1; j0 += 16) {
-    const int j = j0 + c8;
-    const bool ok = j < K1 && (j == 0 || ps[j - 1] >= 0);
-    const float l = ok ? pl[j] : -INFINITY;
-    mx = fmaxf(mx, l);
-  }
+  for (int part = 0; part < parts; ++part)
+    for (int j0 = 0; j0 < K1; j0 += 16) {
+      const int j = j0 + c8;
+      const bool ok = j < K1 && (j == 0 ? part == 0 : ps[j - 1] >= 0);
+      const float l = ok ? pl[part * part_rows + j] : -INFINITY;
+      mx = fmaxf(mx, l);
+    }
 #pragma unroll
   for (int o = 8; o >= 1; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 16));
   float acc[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.f;
   float wsum = 0.f;
+  for (int part = 0; part < parts; ++part, pl += part_rows, po += part_rows * kHeadDim)
   for (int j0 = 0; j0 < K1; j0 += 16) {
     const int j = j0 + c8;
-    const bool ok = j < K1 && (j == 0 || ps[j - 1] >= 0);
+    const bool ok = j < K1 && (j == 0 ? part == 0 : ps[j - 1] >= 0);
     const float wl = ok ? fast_exp2(pl[j] - mx) : 0.f;
     const int nslot = min(16, K1 - j0);
     for (int u0 = 0; u0 < nslot; u0 += 8) {
@@ -712,9 +739,9 @@ __global__ __launch_bounds__(256) void moba_merge_kernel(const typename E::elem*
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
         w[u] = __shfl(wl, u0 + u, 16);           // 0 for slots past K1 too (their lanes computed ok = false)
-        const int jj = w[u] > 0.f ? j0 + u0 + u : 0;
+        const elem* src = w[u] > 0.f ? po + (int64_t)(j0 + u0 + u) * kHeadDim : po0;
         if (u0 + u < nslot)                      // uniform: no loads for slots that do not exist
-          x[u] = __builtin_nontemporal_load(reinterpret_cast<const elem8*>(po + (int64_t)jj * kHeadDim));
+          x[u] = __builtin_nontemporal_load(reinterpret_cast<const elem8*>(src));
       }
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
@@ -739,6 +766,38 @@ __global__ __launch_bounds__(256) void moba_merge_kernel(const typename E::elem*
 using namespace moba;
 
 extern "C" int moba_fwd_tile_rows(void) { return kFwdTileRows; }
+
+constexpr int kMaxKeySplit = 8;
+// workgroups of the forward kernel: resident ones drawing from the queues (> 0), or one per tile id (< 0, see
+// moba_fwd_partials)
+static int fwd_xcd_block_log2(int64_t total) {  // runs of at most an eighth of an XCD's share of the ids
+  int b = 0;
+  while (b < 6 && (128LL << b) <= total) ++b;
+  return b;
+}
+static int64_t fwd_grid(int64_t total, int cus) {
+  int64_t grid = ((int64_t)cus + 7) / 8 * 8;
+  if (total < 8 * grid) {
+    const int64_t run = 8LL << fwd_xcd_block_log2(total);
+    grid = -((total + run - 1) / run * run);
+  }
+  return grid;
+}
+// Into how many parts moba_fwd_partials should cut the keys of every history tile: 1 unless the problem is so
+// small that whole tiles leave compute units idle at the end (a tile of 256 rows x 2048 keys takes 65 us, and
+// workgroups start in the order of their ids, not where the work is); then the largest power of two that
+// keeps 512 keys per part (a part costs 4 us of its own) and the number of tiles within three per unit.
+extern "C" int moba_fwd_key_split(int64_t S, int H, int K, int B, int64_t hist_bound, int64_t self_tiles) {
+  if (S <= 0 || H <= 0 || K <= 0 || B <= 0 || hist_bound <= 0 || self_tiles <= 0) return 1;
+  const int cus = resident_compute_units();
+  if (cus <= 0) return 1;
+  const int64_t own = self_tiles * H;
+  int split = 1;
+  while (split < kMaxKeySplit && B % (TN * 2 * split) == 0 && B / (2 * split) >= 512 &&
+         hist_bound * 2 * split + own <= 3 * (int64_t)cus && S * H * (K + 1) * 2 * split < 0x7fffffffLL)
+    split *= 2;
+  return split;
+}
 
 template <class E>
 static int launch_partials(const void* q, const void* k, const void* v, void* part_o, float* part_lse,
@@ -782,8 +841,9 @@ extern "C" int moba_fwd_partials(const void* q, const void* k, const void* v, vo
                                  const int32_t* fchunk_tok, const int32_t* chunk_tok,
                                  const int32_t* self_tile_prefix, const int32_t* tile_seg,
                                  const int32_t* self_tile_chunk, int64_t S, int H, int Hkv, int D, int K, int F,
-                                 int N, int B, int64_t hist_bound, int64_t self_tiles, const int64_t* strides,
-                                 int32_t* queues, int32_t* redo, float softmax_scale, int dtype, void* stream) {
+                                 int N, int B, int64_t hist_bound, int64_t self_tiles, int key_split,
+                                 const int64_t* strides, int32_t* queues, int32_t* redo, float softmax_scale,
+                                 int dtype, void* stream) {
   if (!q || !k || !v || !part_o || !part_lse || !chunk_tok || !self_tile_prefix || !self_tile_chunk || !queues)
     return MOBA_ERR_ARG;
   if (Hkv <= 0 || H % Hkv != 0) return MOBA_ERR_ARG;
@@ -791,17 +851,22 @@ extern "C" int moba_fwd_partials(const void* q, const void* k, const void* v, vo
   if (D != kHeadDim || (dtype != MOBA_DTYPE_BF16 && dtype != MOBA_DTYPE_F16)) return MOBA_ERR_UNSUPPORTED;
   if (S <= 0 || H <= 0 || K < 0 || F < 0 || N <= 0 || B <= 0 || hist_bound < 0 || self_tiles <= 0) return MOBA_ERR_ARG;
   if (((uintptr_t)q & 15) || ((uintptr_t)k & 15) || ((uintptr_t)v & 15) || ((uintptr_t)part_o & 15)) return MOBA_ERR_ARG;
-  if ((int64_t)S * H * (K + 1) >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
-  const int64_t total = (K > 0 ? hist_bound : 0) + self_tiles * H;
+  int key_split_log2 = 0;
+  while ((1 << key_split_log2) < key_split) ++key_split_log2;
+  if (key_split < 1 || key_split > kMaxKeySplit || (1 << key_split_log2) != key_split) return MOBA_ERR_ARG;
+  if (K == 0) key_split = 1, key_split_log2 = 0;  // (no history tiles: nothing to cut)
+  if ((int64_t)S * H * (K + 1) * key_split >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
+  const int64_t total = (K > 0 ? hist_bound * key_split : 0) + self_tiles * H;
   if (total >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
   // one workgroup of eight waves per CU (what the kernel's registers allow), all resident at once and drawing
   // tiles from the queues; a multiple of 8 so that every XCD starts on its own queue with as many
   const int cus = resident_compute_units();
   if (cus <= 0) return MOBA_ERR_LAUNCH;
-  int64_t grid = ((int64_t)cus + 7) / 8 * 8;
   // with fewer than a few tiles per resident workgroup the queues do not pay: one workgroup per id then
   // (a negative grid tells the launcher)
-  if (total < 8 * grid) grid = -((total + 8 * kXcdBlock - 1) / (8 * kXcdBlock) * (8 * kXcdBlock));
+  const int64_t grid = fwd_grid(total, cus);
+  // the parts are tiles of the one-workgroup-per-id form only, whole key tiles each
+  if (key_split > 1 && (grid > 0 || B % (TN * key_split) != 0)) return MOBA_ERR_ARG;
   TileTables t;
   t.seg_off = seg_off; t.tile_off = tile_off; t.seg_dest = seg_dest; t.fchunk_tok = fchunk_tok;
   t.chunk_tok = chunk_tok; t.self_tile_prefix = self_tile_prefix;
@@ -811,6 +876,10 @@ extern "C" int moba_fwd_partials(const void* q, const void* k, const void* v, vo
   t.hist_bound = (K > 0) ? (int)hist_bound : 0;
   t.self_total = (int)(self_tiles * H);
   if (!set_layout(t, strides)) return MOBA_ERR_ARG;
+  t.key_split_log2 = key_split_log2;
+  t.part_stride = (int)(S * H * (K + 1));
+  t.xcd_block_log2 = fwd_xcd_block_log2(total);
+  t.self_first = key_split > 1;
   hipStream_t st = (hipStream_t)stream;
   return dtype == MOBA_DTYPE_F16
              ? launch_partials<F16>(q, k, v, part_o, part_lse, t, D, softmax_scale, grid, queues, redo, st)
@@ -818,19 +887,21 @@ extern "C" int moba_fwd_partials(const void* q, const void* k, const void* v, vo
 }
 
 extern "C" int moba_fwd_merge(const void* part_o, const float* part_lse, const int32_t* sel, void* out, float* lse,
-                              int64_t S, int H, int D, int K, int dtype, void* stream) {
+                              int64_t S, int H, int D, int K, int key_split, int dtype, void* stream) {
   LaunchCheck launch_check;
   if (!part_o || !part_lse || !out || !lse || (K > 0 && !sel)) return MOBA_ERR_ARG;
+  if (key_split < 1 || key_split > kMaxKeySplit) return MOBA_ERR_ARG;
+  if (K == 0) key_split = 1;
   if (D != kHeadDim || (dtype != MOBA_DTYPE_BF16 && dtype != MOBA_DTYPE_F16)) return MOBA_ERR_UNSUPPORTED;
   if (S <= 0 || H <= 0 || K < 0 || ((uintptr_t)part_o & 15) || ((uintptr_t)out & 15)) return MOBA_ERR_ARG;
   const int64_t rows = S * H;
   const dim3 grid((unsigned)((rows + 15) / 16));
   if (dtype == MOBA_DTYPE_F16)
     hipLaunchKernelGGL(moba_merge_kernel<F16>, grid, dim3(256), 0, (hipStream_t)stream, (const f16*)part_o, part_lse,
-                       sel, (f16*)out, lse, rows, K + 1);
+                       sel, (f16*)out, lse, rows, K + 1, key_split);
   else
     hipLaunchKernelGGL(moba_merge_kernel<Bf16>, grid, dim3(256), 0, (hipStream_t)stream, (const bf16*)part_o,
-                       part_lse, sel, (bf16*)out, lse, rows, K + 1);
+                       part_lse, sel, (bf16*)out, lse, rows, K + 1, key_split);
   return launch_check.result();
 }
 
@@ -840,11 +911,11 @@ extern "C" int moba_fwd(const void* q, const void* k, const void* v, void* part_
                         const int32_t* seg_dest, const int32_t* fchunk_tok, const int32_t* chunk_tok,
                         const int32_t* self_tile_prefix, const int32_t* tile_seg, const int32_t* self_tile_chunk,
                         void* out, float* lse, int64_t S, int H, int Hkv, int D, int K, int F, int N, int B,
-                        int64_t hist_bound, int64_t self_tiles, const int64_t* strides, int32_t* queues,
-                        int32_t* redo, float softmax_scale, int dtype, void* stream) {
+                        int64_t hist_bound, int64_t self_tiles, int key_split, const int64_t* strides,
+                        int32_t* queues, int32_t* redo, float softmax_scale, int dtype, void* stream) {
   int rc = moba_fwd_partials(q, k, v, part_o, part_lse, seg_off, tile_off, seg_dest, fchunk_tok, chunk_tok,
                              self_tile_prefix, tile_seg, self_tile_chunk, S, H, Hkv, D, K, F, N, B, hist_bound,
-                             self_tiles, strides, queues, redo, softmax_scale, dtype, stream);
+                             self_tiles, key_split, strides, queues, redo, softmax_scale, dtype, stream);
   if (rc != MOBA_OK) return rc;
-  return moba_fwd_merge(part_o, part_lse, sel, out, lse, S, H, D, K, dtype, stream);
+  return moba_fwd_merge(part_o, part_lse, sel, out, lse, S, H, D, K, key_split, dtype, stream);
 }

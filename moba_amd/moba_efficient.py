@@ -270,7 +270,9 @@ def _forward(q, k, v, plan: MobaPlan, timer: Optional[StageTimer] = None, scale:
     # the forward kernel's tile counters, then the list of tiles its fixed-reference softmax hands to the kernel
     # that tracks the running maximum (count first; the call zeroes the counters and the count).
     bound = plan.hist_tile_bound(H, FWD_TILE_ROWS)
-    rows = S * H * (K + 1)
+    # small problems: the keys of every history tile in `split` parts, each with slots of its own
+    split = 1 if plan.fallback else int(lib.moba_fwd_key_split(S, H, K, plan.chunk_size, bound, plan.fwd_self_tiles))
+    rows = S * H * (K + 1) * split
     n_ints = 8 + 1 + bound + plan.fwd_self_tiles * H
     ws = torch.empty(rows * D * q.element_size() + rows * 4 + n_ints * 4, dtype=torch.uint8, device=dev)
     part_o = ws[:rows * D * q.element_size()].view(q.dtype).view(rows, D)
@@ -282,12 +284,12 @@ def _forward(q, k, v, plan: MobaPlan, timer: Optional[StageTimer] = None, scale:
                                          _ptr(tile_off), _ptr(seg_dest), _ptr(t.get("fchunk_tok")),
                                          _ptr(t["chunk_tok"]), _ptr(t["fwd_self_tile_prefix"]), _ptr(tile_seg),
                                          _ptr(t["fwd_self_tile_chunk"]), S, H, Hkv, D, K, plan.F, plan.N,
-                                         plan.chunk_size, bound, plan.fwd_self_tiles, _strides(q, k),
+                                         plan.chunk_size, bound, plan.fwd_self_tiles, split, _strides(q, k),
                                          _ptr(queues), _ptr(redo), scale, _dtype_code(q), _stream(dev)),
                    "moba_fwd_partials")
     with span("fwd_merge"):
         _lib.check(lib.moba_fwd_merge(_ptr(part_o), _ptr(part_lse), _ptr(sel), _ptr(out), _ptr(lse), S, H, D, K,
-                                      _dtype_code(q), _stream(dev)), "moba_fwd_merge")
+                                      split, _dtype_code(q), _stream(dev)), "moba_fwd_merge")
     return out, lse, sel, seg_off, tile_off, seg_dest, tile_seg
 
 

@@ -164,24 +164,28 @@ def test_forward_vs_oracle(batch, seqlen, heads, B, topk):
 
 
 # ------------------------------------------------------------------ LSE merge alone
-@pytest.mark.parametrize("K,dtype", [(2, torch.bfloat16), (11, torch.bfloat16), (20, torch.float16)])
-def test_merge_of_random_partials(K, dtype):
+@pytest.mark.parametrize("K,dtype,parts", [(2, torch.bfloat16, 1), (11, torch.bfloat16, 1), (20, torch.float16, 1),
+                                           (3, torch.bfloat16, 2), (17, torch.float16, 4)])
+def test_merge_of_random_partials(K, dtype, parts):
     """moba_fwd_merge on random per-slot partials (some slots absent, log-sum-exps far apart)
-    against the merge algebra of the oracle (moba/moba_efficient.py:130-168)."""
+    against the merge algebra of the oracle (moba/moba_efficient.py:130-168).  parts > 1: every history slot
+    holds that many partials (key_split of the forward), the self slot one."""
     import ctypes
     import math
     from moba_amd import _lib
     lib = _lib.load()
     S, H, K1 = 300, 3, K + 1
     g = torch.Generator().manual_seed(K)
-    part_o = torch.randn((S * H * K1, 128), generator=g).to(dtype)
-    lse_nat = torch.randn((S * H, K1), generator=g) * 6                    # natural-log LSE of each slot
+    part_o = torch.randn((parts, S * H * K1, 128), generator=g).to(dtype)
+    lse_nat = torch.randn((parts, S * H, K1), generator=g) * 6             # natural-log LSE of each slot
     sel = torch.randint(0, 50, (S, H, K), generator=g, dtype=torch.int32)
     sel[torch.rand((S, H, K), generator=g) < 0.3] = -1                     # absent slots
     part_o_dev = part_o.cuda()
-    # absent slots hold garbage in the real buffers: poison them
+    # absent slots hold garbage in the real buffers (and so do parts 1.. of the self slot): poison them
     absent = torch.cat([torch.zeros((S * H, 1), dtype=torch.bool), (sel < 0).view(S * H, K)], dim=1)
-    part_o_dev.view(S * H, K1, 128)[absent.cuda()] = float("nan")
+    absent = absent.unsqueeze(0).repeat(parts, 1, 1)
+    absent[1:, :, 0] = True
+    part_o_dev.view(parts, S * H, K1, 128)[absent.cuda()] = float("nan")
     part_lse = (lse_nat / math.log(2.0)).float()                           # the kernels keep it in the log2 domain
     part_lse_dev = part_lse.clone()
     part_lse_dev[absent] = float("nan")
@@ -190,11 +194,13 @@ def test_merge_of_random_partials(K, dtype):
     lse = torch.empty((S, H), dtype=torch.float32, device="cuda")
     p = lambda t: ctypes.c_void_p(t.data_ptr())
     code = _lib.DTYPE_F16 if dtype == torch.float16 else _lib.DTYPE_BF16
-    _lib.check(lib.moba_fwd_merge(p(part_o_dev), p(part_lse_dev), p(sel.cuda()), p(out), p(lse), S, H, 128, K, code,
-                                  ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)), "moba_fwd_merge")
+    _lib.check(lib.moba_fwd_merge(p(part_o_dev), p(part_lse_dev), p(sel.cuda()), p(out), p(lse), S, H, 128, K, parts,
+                                  code, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)), "moba_fwd_merge")
     lses = lse_nat.clone()
     lses[absent] = float("-inf")
-    want, want_lse = O.merge_partials(part_o.float().view(S * H, K1, 128).permute(1, 0, 2), lses.t())
+    # (the parts of a slot are slots like any other to the merge algebra)
+    want, want_lse = O.merge_partials(part_o.float().view(parts, S * H, K1, 128).permute(0, 2, 1, 3).reshape(parts * K1, S * H, 128),
+                                      lses.permute(0, 2, 1).reshape(parts * K1, S * H))
     assert (out.float().cpu().view(S * H, 128) - want).abs().max() < 2e-2
     assert (lse.cpu().view(-1) - want_lse).abs().max() < 1e-3
 
@@ -216,8 +222,10 @@ def test_moba_fwd_entry_point(batch, seqlen, heads, B, topk, dtype):
     lib = _lib.load()
     S, H, D = q.shape
     K, t, dev = plan.K, plan.tables, qg.device
-    part_o = torch.empty((S * H * (K + 1), D), dtype=dtype, device=dev)
-    part_lse = torch.empty((S * H * (K + 1),), dtype=torch.float32, device=dev)
+    bound = plan.hist_tile_bound(H, 256)
+    split = 1 if plan.fallback else lib.moba_fwd_key_split(S, H, K, plan.chunk_size, bound, plan.fwd_self_tiles)  # as the operator
+    part_o = torch.empty((split * S * H * (K + 1), D), dtype=dtype, device=dev)
+    part_lse = torch.empty((split * S * H * (K + 1),), dtype=torch.float32, device=dev)
     out = torch.zeros((S, H, D), dtype=dtype, device=dev)
     lse = torch.zeros((S, H), dtype=torch.float32, device=dev)
     queues = torch.empty(8, dtype=torch.int32, device=dev)
@@ -225,7 +233,7 @@ def test_moba_fwd_entry_point(batch, seqlen, heads, B, topk, dtype):
     _lib.check(lib.moba_fwd(p(qg), p(kg), p(vg), p(part_o), p(part_lse), p(sel), p(seg_off), p(tile_off), p(seg_dest),
                             p(t.get("fchunk_tok")), p(t["chunk_tok"]), p(t["fwd_self_tile_prefix"]), p(tile_seg),
                             p(t["fwd_self_tile_chunk"]), p(out), p(lse), S, H, H, D, K, plan.F, plan.N, plan.chunk_size,
-                            plan.hist_tile_bound(H, 256), plan.fwd_self_tiles, None, p(queues), None, 0.0, E._dtype_code(qg),
+                            bound, plan.fwd_self_tiles, split, None, p(queues), None, 0.0, E._dtype_code(qg),
                             E._stream(dev)), "moba_fwd")
     torch.cuda.synchronize()
     assert torch.equal(out, want_out) and torch.equal(lse, want_lse)
@@ -237,7 +245,7 @@ def test_moba_fwd_entry_point(batch, seqlen, heads, B, topk, dtype):
 
 
 # ------------------------------------------------------------------ fixed-reference softmax and its redo list
-def _attention_stage(q, k, v, plan, aux, with_redo):
+def _attention_stage(q, k, v, plan, aux, with_redo, key_split=1):
     """moba_fwd on prepared selection/lists; returns (out, lse, number of tiles sent to the redo list or None)."""
     from moba_amd import _lib
     from moba_amd import moba_efficient as E
@@ -245,8 +253,9 @@ def _attention_stage(q, k, v, plan, aux, with_redo):
     sel, seg_off, tile_off, seg_dest, tile_seg = aux
     S, H, D = q.shape
     K, t, dev = plan.K, plan.tables, q.device
-    part_o = torch.empty((S * H * (K + 1), D), dtype=q.dtype, device=dev)
-    part_lse = torch.empty((S * H * (K + 1),), dtype=torch.float32, device=dev)
+    # (poisoned: a part that the kernel does not write, or a slot the merge must not read, shows)
+    part_o = torch.full((key_split * S * H * (K + 1), D), float("nan"), dtype=q.dtype, device=dev)
+    part_lse = torch.full((key_split * S * H * (K + 1),), float("nan"), dtype=torch.float32, device=dev)
     out = torch.zeros((S, H, D), dtype=q.dtype, device=dev)
     lse = torch.zeros((S, H), dtype=torch.float32, device=dev)
     queues = torch.empty(8, dtype=torch.int32, device=dev)
@@ -256,7 +265,7 @@ def _attention_stage(q, k, v, plan, aux, with_redo):
     _lib.check(lib.moba_fwd(p(q), p(k), p(v), p(part_o), p(part_lse), p(sel), p(seg_off), p(tile_off), p(seg_dest),
                             p(t.get("fchunk_tok")), p(t["chunk_tok"]), p(t["fwd_self_tile_prefix"]), p(tile_seg),
                             p(t["fwd_self_tile_chunk"]), p(out), p(lse), S, H, H, D, K, plan.F, plan.N, plan.chunk_size,
-                            plan.hist_tile_bound(H, 256), plan.fwd_self_tiles, None, p(queues), p(redo), 0.0,
+                            plan.hist_tile_bound(H, 256), plan.fwd_self_tiles, key_split, None, p(queues), p(redo), 0.0,
                             E._dtype_code(q), E._stream(dev)), "moba_fwd")
     torch.cuda.synchronize()
     if redo is None:
@@ -265,6 +274,50 @@ def _attention_stage(q, k, v, plan, aux, with_redo):
     ids = redo[1:1 + n].cpu()
     assert 0 <= n <= tiles and ids.unique().numel() == n and bool(((ids >= 0) & (ids < tiles)).all())
     return out, lse, n
+
+
+@pytest.mark.parametrize("seqlens,heads,B,topk,dtype", [([8192], 2, 1024, 3, torch.bfloat16),
+                                                         ([3000, 5000, 777], 3, 512, 2, torch.float16),
+                                                         ([16384], 1, 2048, 3, torch.bfloat16),
+                                                         ([4000], 2, 192, 3, torch.bfloat16)])
+def test_history_keys_cut_into_parts(seqlens, heads, B, topk, dtype):
+    """key_split of moba_fwd: every history tile's keys in 2, 4 or 8 parts (tiles of their own whose partials the
+    merge takes as further slots).  The result must agree with the uncut one within rounding and with the oracle
+    on the same selection; what moba_fwd_key_split proposes must be accepted; values the call cannot serve are
+    refused."""
+    from moba_amd import _lib
+    from moba_amd import moba_efficient as E
+    lib = _lib.load()
+    _note("key parts", seqlens, heads, B, topk, dtype)
+    cu = [0] + [int(x) for x in np.cumsum(seqlens)]
+    S = cu[-1]
+    g = torch.Generator().manual_seed(sum(seqlens) + heads)
+    q, k, v = (torch.randn((S, heads, 128), generator=g).to(dtype) for _ in range(3))
+    plan = _plan(cu, B, topk)
+    qg, kg, vg = q.cuda(), k.cuda(), v.cuda()
+    sel = E.gate_topk(qg, E.chunk_mean(kg, plan), plan)
+    aux = (sel,) + tuple(E.build_lists(sel, plan))
+    out1, lse1, _ = _attention_stage(qg, kg, vg, plan, aux, False, 1)
+    ref, ref_lse, _ = O.moba_attn_varlen_oracle(q, k, v, cu, max(seqlens), B, topk, sel=sel.cpu(), return_aux=True)
+    proposed = lib.moba_fwd_key_split(S, heads, plan.K, B, plan.hist_tile_bound(heads, 256), plan.fwd_self_tiles)
+    _note("  proposed", proposed)
+    assert proposed in (1, 2, 4, 8) and B % (64 * proposed) == 0
+    for split in (2, 4, 8):
+        if B % (64 * split):
+            with pytest.raises(RuntimeError):
+                _attention_stage(qg, kg, vg, plan, aux, False, split)
+            continue
+        out, lse, _ = _attention_stage(qg, kg, vg, plan, aux, False, split)
+        assert torch.isfinite(out.float()).all() and torch.isfinite(lse).all()
+        d = (out.float() - out1.float()).abs()
+        assert d.max() < 2e-2 and d.mean() < 2e-4, (split, d.max().item(), d.mean().item())
+        assert (lse - lse1).abs().max() < 1e-3
+        err = (out.cpu().float() - ref).abs()
+        assert err.max() < 2e-2 and err.mean() < 2e-3, (split, err.max().item(), err.mean().item())
+        assert (lse.cpu() - ref_lse).abs().max() < 2e-3
+    for bad in (0, 3, 16):
+        with pytest.raises(RuntimeError):
+            _attention_stage(qg, kg, vg, plan, aux, False, bad)
 
 
 @pytest.mark.parametrize("spread", [1.0, 8.0])
