@@ -8,54 +8,73 @@
 // mean is reproducible bit for bit (fp64 -> fp32 -> element type, round to nearest even).
 //
 // Stage 1: grid (F, token splits, column blocks); each thread owns 8 adjacent
-//          columns of the [H*D] token row and sums its token split.
+//          columns of the [H*D] token row and sums its share of a token split.
 // Stage 2: sums the splits in order, divides by B, rounds.
 #include <mutex>
 #include "common.h"
 
 namespace moba {
 
+// cpb_log2: the workgroup's 256 threads are 1 << cpb_log2 column groups (8 adjacent columns each) times
+// 256 >> cpb_log2 token lanes: a row narrower than 2048 elements still occupies every lane, and the token lanes'
+// sums are added through LDS (exact sums: the order does not matter).
 template <class E>
 __global__ __launch_bounds__(256) void chunk_mean_partial_kernel(
     const typename E::elem* __restrict__ k, const int* __restrict__ fchunk_tok, double* __restrict__ partial,
     int HD8 /* H*D/8 */, int D8 /* D/8 */, int B, int nsplit, int tok_per_split, int64_t row_stride,
-    int64_t head_stride, int batch_rows, int64_t batch_stride) {
+    int64_t head_stride, int batch_rows, int64_t batch_stride, int cpb_log2) {
   MOBA_ELEM_TYPES(E)
-  const int col = blockIdx.z * 256 + threadIdx.x;
-  if (col >= HD8) return;
+  __shared__ double red[256 * 8];
+  const int cpb = 1 << cpb_log2, lanes = 256 >> cpb_log2;
+  const int tl = threadIdx.x >> cpb_log2;
+  const int col = blockIdx.z * cpb + (threadIdx.x & (cpb - 1));
+  const bool col_ok = col < HD8;
   const int split = blockIdx.y;
   const int f = blockIdx.x;  // the only grid dimension without a 65535 limit
   const int t0 = split * tok_per_split;
   const int t1 = min(B, t0 + tok_per_split);
-  const int head = col / D8;
+  const int head = col_ok ? col / D8 : 0;
   // (a chunk lies inside one sequence, hence inside one batch entry of a batched layout)
   const int tok0 = fchunk_tok[f];
   const int be = batch_rows ? tok0 / batch_rows : 0;
-  const elem* src = k + be * batch_stride + ((int64_t)(tok0 - be * batch_rows) + t0) * row_stride + head * head_stride +
-                    (col - head * D8) * 8;
+  const elem* src = k + be * batch_stride + ((int64_t)(tok0 - be * batch_rows) + t0 + tl) * row_stride +
+                    head * head_stride + (col_ok ? col - head * D8 : 0) * 8;
+  const int64_t step = (int64_t)lanes * row_stride;
   double acc[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.0;
-  int t = t0;
-  for (; t + 8 <= t1; t += 8) {
-    elem8 x[8];
+  int t = t0 + tl;
+  if (col_ok) {
+    for (; t + 7 * lanes < t1; t += 8 * lanes) {
+      elem8 x[8];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) x[u] = __builtin_nontemporal_load(reinterpret_cast<const elem8*>(src + u * row_stride));
-    src += 8 * row_stride;
+      for (int u = 0; u < 8; ++u) x[u] = __builtin_nontemporal_load(reinterpret_cast<const elem8*>(src + u * step));
+      src += 8 * step;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      // sums of 16-bit float values are exact in fp64 whatever the order
-      const double a = ((double)(float)x[0][e] + (double)(float)x[1][e]) + ((double)(float)x[2][e] + (double)(float)x[3][e]);
-      const double b = ((double)(float)x[4][e] + (double)(float)x[5][e]) + ((double)(float)x[6][e] + (double)(float)x[7][e]);
-      acc[e] += a + b;
+      for (int e = 0; e < 8; ++e) {
+        // sums of 16-bit float values are exact in fp64 whatever the order
+        const double a = ((double)(float)x[0][e] + (double)(float)x[1][e]) + ((double)(float)x[2][e] + (double)(float)x[3][e]);
+        const double b = ((double)(float)x[4][e] + (double)(float)x[5][e]) + ((double)(float)x[6][e] + (double)(float)x[7][e]);
+        acc[e] += a + b;
+      }
+    }
+    for (; t < t1; t += lanes) {
+      elem8 x0 = *reinterpret_cast<const elem8*>(src);
+      src += step;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] += (double)(float)x0[e];
     }
   }
-  for (; t < t1; ++t) {
-    elem8 x0 = *reinterpret_cast<const elem8*>(src);
-    src += row_stride;
+  if (lanes > 1) {  // (uniform)
 #pragma unroll
-    for (int e = 0; e < 8; ++e) acc[e] += (double)(float)x0[e];
+    for (int e = 0; e < 8; ++e) red[e * 256 + threadIdx.x] = acc[e];
+    __syncthreads();
+    if (tl != 0) return;
+    for (int l = 1; l < lanes; ++l)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] += red[e * 256 + (l << cpb_log2) + threadIdx.x];
   }
+  if (!col_ok) return;
   double* dst = partial + ((int64_t)(f * nsplit + split) * HD8 + col) * 8;
 #pragma unroll
   for (int e = 0; e < 8; ++e) dst[e] = acc[e];
@@ -86,11 +105,22 @@ __global__ __launch_bounds__(256) void chunk_mean_finish_kernel(
   double acc[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.0;
-  for (int s = 0; s < nsplit; ++s) {
-    const double* src = partial + ((int64_t)(f * nsplit + s) * HD8 + col) * 8;
+  const double* src = partial + ((int64_t)f * nsplit * HD8 + col) * 8;
+  const int64_t step = (int64_t)HD8 * 8;
+  int s = 0;
+  for (; s + 4 <= nsplit; s += 4) {  // four splits' loads in flight together (nsplit is a power of two)
+    double x[4][8];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) x[u][e] = src[u * step + e];
+    src += 4 * step;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] += (x[0][e] + x[1][e]) + (x[2][e] + x[3][e]);
+  }
+  for (; s < nsplit; ++s, src += step)
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[e] += src[e];
-  }
   elem8 o;
   const double inv = (double)B;
 #pragma unroll
@@ -102,12 +132,20 @@ __global__ __launch_bounds__(256) void chunk_mean_finish_kernel(
 
 using namespace moba;
 
+// column groups per workgroup (as a power of two): all 256 threads for rows of 2048 elements or more
+static int pick_cpb_log2(int HD8) {
+  int c = 0;
+  while (c < 8 && (1 << c) < HD8) ++c;
+  return c;
+}
 static int pick_nsplit(int HD8, int F, int B) {
-  const int colblocks = (HD8 + 255) / 256;
+  const int cpb_log2 = pick_cpb_log2(HD8);
+  const int colblocks = (HD8 + (1 << cpb_log2) - 1) >> cpb_log2;
+  const int lanes = 256 >> cpb_log2;
   int nsplit = 1;
   // enough workgroups to keep every CU's memory pipeline full (8 row loads in flight per lane),
   // few enough that the fp64 partial sums stay a small fraction of the traffic
-  while ((int64_t)colblocks * F * nsplit < 1536 && B / (nsplit * 2) >= 64) nsplit *= 2;
+  while ((int64_t)colblocks * F * nsplit < 1536 && B / (nsplit * 2) >= 64 && B / (nsplit * 2) >= 8 * lanes) nsplit *= 2;
   return nsplit;
 }
 
@@ -123,17 +161,18 @@ static int launch_chunk_mean(const void* k, const int32_t* fchunk_tok, void* kba
   LaunchCheck launch_check;
   const int HD8 = H * D / 8;
   const int tps = (B + nsplit - 1) / nsplit;
-  dim3 grid(F, nsplit, (HD8 + 255) / 256);
+  const int cpb_log2 = pick_cpb_log2(HD8);
+  dim3 grid(F, nsplit, (HD8 + (1 << cpb_log2) - 1) >> cpb_log2);
   const int64_t n = (int64_t)F * HD8;
   const dim3 fgrid((unsigned)((n + 255) / 256));
   if (dtype == MOBA_DTYPE_F16) {
     hipLaunchKernelGGL(chunk_mean_partial_kernel<F16>, grid, dim3(256), 0, st, (const f16*)k, fchunk_tok, partial,
-                       HD8, D / 8, B, nsplit, tps, kts, khs, batch_rows, kbs);
+                       HD8, D / 8, B, nsplit, tps, kts, khs, batch_rows, kbs, cpb_log2);
     hipLaunchKernelGGL(chunk_mean_finish_kernel<F16>, fgrid, dim3(256), 0, st, (const double*)partial, (f16*)kbar,
                        HD8, B, nsplit, F);
   } else {
     hipLaunchKernelGGL(chunk_mean_partial_kernel<Bf16>, grid, dim3(256), 0, st, (const bf16*)k, fchunk_tok, partial,
-                       HD8, D / 8, B, nsplit, tps, kts, khs, batch_rows, kbs);
+                       HD8, D / 8, B, nsplit, tps, kts, khs, batch_rows, kbs, cpb_log2);
     hipLaunchKernelGGL(chunk_mean_finish_kernel<Bf16>, fgrid, dim3(256), 0, st, (const double*)partial, (bf16*)kbar,
                        HD8, B, nsplit, F);
   }

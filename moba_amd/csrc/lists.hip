@@ -218,6 +218,86 @@ __global__ __launch_bounds__(256) void lists_tile_seg_kernel(const int* __restri
   tile_seg[t] = t < tile_off[FH] ? upper_row(tile_off, FH, t) : -1;
 }
 
+// Few segments and few tiles: what lists_segments_kernel (or lists_tile_counts_kernel, when `base` is null and
+// seg_off is given), the scan of the tile counts and lists_tile_seg_kernel do, in one workgroup with the counts
+// in LDS -- three dependent launches of a few microseconds each are most of the list stage of a small problem.
+constexpr int kTailMaxSegments = 4096, kTailMaxTiles = 16384;
+__global__ __launch_bounds__(1024) void lists_tail_kernel(const int* __restrict__ base, const int* __restrict__ pair_off,
+                                                          int* __restrict__ seg_off, int* __restrict__ tile_off,
+                                                          int* __restrict__ tile_seg, int F, int H, int tile_rows,
+                                                          int bound) {
+  __shared__ int off[kTailMaxSegments + 1];
+  __shared__ int wsum[16];
+  const int FH = F * H, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // this thread's four consecutive segments: list starts (written out when they come from the counts), tile counts
+  int v[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int fh = tid * 4 + e;
+    v[e] = 0;
+    if (fh < FH) {
+      int start, end;
+      if (base) {
+        const int f = fh / H, h = fh % H;
+        const int p0 = pair_off[f];
+        const int nq = pair_off[f + 1] - p0;
+        start = base[p0 * H + h * nq];
+        end = base[p0 * H + (h + 1) * nq];
+        seg_off[fh] = start;
+      } else {
+        start = seg_off[fh];
+        end = seg_off[fh + 1];
+      }
+      v[e] = (end - start + tile_rows - 1) / tile_rows;
+    } else if (fh == FH && base) {
+      seg_off[fh] = base[pair_off[F] * H];
+    }
+  }
+  const int tsum = v[0] + v[1] + v[2] + v[3];
+  int inc = tsum;  // inclusive scan across the wave, then across the waves
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const int t = __shfl_up(inc, o, 64);
+    if (lane >= o) inc += t;
+  }
+  if (lane == 63) wsum[wave] = inc;
+  __syncthreads();
+  int woff = 0, total = 0;
+#pragma unroll
+  for (int w = 0; w < 16; ++w) {
+    const int x = wsum[w];
+    if (w < wave) woff += x;
+    total += x;
+  }
+  int run = woff + inc - tsum;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int fh = tid * 4 + e;
+    if (fh < FH) {
+      off[fh] = run;
+      tile_off[fh] = run;
+    }
+    run += v[e];
+  }
+  if (tid == 0) {
+    off[FH] = total;
+    tile_off[FH] = total;
+  }
+  __syncthreads();
+  for (int t = tid; t < bound; t += 1024) {
+    int seg = -1;
+    if (t < total) {
+      int lo = 0, hi = FH;  // off[lo] <= t < off[hi]
+      while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (off[mid] <= t) lo = mid; else hi = mid;
+      }
+      seg = lo;
+    }
+    tile_seg[t] = seg;
+  }
+}
+
 }  // namespace moba
 
 using namespace moba;
@@ -257,6 +337,11 @@ extern "C" int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, co
   else if (K <= 64) MOBA_FILL(64)
   else return MOBA_ERR_LIMIT;
 #undef MOBA_FILL
+  if ((int64_t)F * H < kTailMaxSegments && hist_bound <= kTailMaxTiles) {
+    hipLaunchKernelGGL(lists_tail_kernel, dim3(1), dim3(1024), 0, st, (const int*)cnt, pair_off, seg_off, tile_off,
+                       tile_seg, F, H, tile_rows, (int)hist_bound);
+    return launch_check.result();
+  }
   hipLaunchKernelGGL(lists_segments_kernel, dim3((F * H + 1 + 255) / 256), dim3(256), 0, st, (const int*)cnt,
                      pair_off, seg_off, tile_off, F, H, tile_rows);
   hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(1024), 0, st, tile_off, F * H);
@@ -274,6 +359,11 @@ extern "C" int moba_tile_tables(const int32_t* seg_off, int32_t* tile_off, int32
   if (H <= 0 || F <= 0 || tile_rows <= 0 || hist_bound <= 0 || hist_bound >= 0x7fffffffLL) return MOBA_ERR_ARG;
   if ((int64_t)F * H >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
   hipStream_t st = (hipStream_t)stream;
+  if ((int64_t)F * H < kTailMaxSegments && hist_bound <= kTailMaxTiles) {
+    hipLaunchKernelGGL(lists_tail_kernel, dim3(1), dim3(1024), 0, st, (const int*)nullptr, (const int*)nullptr,
+                       const_cast<int*>(seg_off), tile_off, tile_seg, F, H, tile_rows, (int)hist_bound);
+    return launch_check.result();
+  }
   hipLaunchKernelGGL(lists_tile_counts_kernel, dim3((F * H + 255) / 256), dim3(256), 0, st, seg_off, tile_off, F * H,
                      tile_rows);
   hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(1024), 0, st, tile_off, F * H);

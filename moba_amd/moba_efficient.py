@@ -32,8 +32,15 @@ def _ptr(t: Optional[torch.Tensor]):
     return ctypes.c_void_p(0 if t is None else t.data_ptr())
 
 
+# the current stream's handle without building a torch.cuda.Stream object (a few microseconds per stage otherwise)
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(device) -> ctypes.c_void_p:
-    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+    if _raw_stream is None:
+        return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+    index = device.index
+    return ctypes.c_void_p(_raw_stream(torch.cuda.current_device() if index is None else index))
 
 
 def _dtype_code(t: torch.Tensor) -> int:
@@ -346,6 +353,13 @@ class _MobaAttention(torch.autograd.Function):
         return dq, dk, dv, None, None, None
 
 
+def _attend(q, k, v, plan, timer=None, scale=0.0):
+    """(out, lse): through autograd when a gradient may be asked for, straight to the kernels otherwise."""
+    if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad):
+        return _MobaAttention.apply(q, k, v, plan, timer, scale)
+    return _forward(q, k, v, plan, timer, scale)[:2]
+
+
 def moba_attn_varlen(
     q: torch.Tensor,
     k: torch.Tensor,
@@ -401,7 +415,7 @@ def moba_attn_batched(query, key, value, moba_chunk_size, moba_topk):
     _check_qkv(query.select(0, 0).transpose(0, 1), key.select(0, 0).transpose(0, 1), value.select(0, 0).transpose(0, 1),
                gqa=True)
     plan = make_plan(cu_seqlens, moba_chunk_size, moba_topk, device=query.device)
-    return _MobaAttention.apply(query, key, value, plan)[0]
+    return _attend(query, key, value, plan)[0]
 
 
 # lets moba_layer skip the key/value head expansion when it drives this operator
@@ -424,7 +438,7 @@ def moba_attn_varlen_with_lse(q, k, v, cu_seqlens, max_seqlen, moba_chunk_size, 
     if head_dim < HEAD_DIM:
         pad = (0, HEAD_DIM - head_dim)
         q, k, v = (torch.nn.functional.pad(x, pad) for x in (q, k, v))
-        out, lse = _MobaAttention.apply(q, k, v, plan, timer, head_dim ** -0.5)
+        out, lse = _attend(q, k, v, plan, timer, head_dim ** -0.5)
         return out[..., :head_dim].contiguous(), lse
     q, k, v = _in_place(q, k, v)
-    return _MobaAttention.apply(q, k, v, plan, timer)
+    return _attend(q, k, v, plan, timer)
