@@ -127,7 +127,24 @@ __global__ __launch_bounds__(256) void gate_topk_kernel(
       __syncthreads();
     }
   }
-  if (s < S && head_ok) {
+  // The four waves hold the lists of four consecutive heads of the same 64 tokens: K ints per (token, head) that
+  // lie 4K ints in a row per token in sel.  Through LDS, so that the workgroup stores those runs with consecutive
+  // lanes on consecutive ints (a lane storing its own K ints touches a cache line for 4K bytes of it).
+  __syncthreads();  // (the score tile is read out)
+  int* stage = reinterpret_cast<int*>(&sc[0][0][0]);  // [64 tokens][4 heads][K]
+  if (4 * 64 * K <= (int)(sizeof(sc) / sizeof(int))) {  // (uniform; K <= 33)
+#pragma unroll
+    for (int j = 0; j < KMAX; ++j)
+      if (j < K) stage[(lane * 4 + wave) * K + j] = top.idx[j];
+    __syncthreads();
+    const int run = 4 * K;                       // ints per token in this workgroup's four heads
+    const int heads_here = min(4, H - blockIdx.y * 4);
+    for (int i = threadIdx.x; i < 64 * run; i += 256) {
+      const int tk = i / run, w = i - tk * run;  // token of the tile, int within its run
+      if (tok0 + tk < S && w < heads_here * K)
+        sel[((int64_t)(tok0 + tk) * H + blockIdx.y * 4) * K + w] = stage[i];
+    }
+  } else if (s < S && head_ok) {
     int* dst = sel + ((int64_t)s * H + h) * K;
 #pragma unroll
     for (int j = 0; j < KMAX; ++j)
