@@ -122,6 +122,7 @@ def test_float16(batch, seqlen, heads, B, topk):
     (4, 2048, 8, 2, 128, 2, torch.float16),
     (1, 2048, 4, 2, 128, 1, torch.bfloat16),     # fallback: full causal attention
     (2, 65536, 8, 2, 1024, 4, torch.float16),    # enough tiles for the resident-workgroup kernels, fp16
+    (1, 8192, 2, 1, 1024, 3, torch.float16),     # few tiles: the forward cuts the history tiles' keys into parts
 ])
 def test_grouped_query(batch, seqlen, heads, kv_heads, B, topk, dtype):
     """k, v with fewer heads: same result (bit for bit in the forward) as expanding them with
@@ -156,6 +157,7 @@ def test_grouped_query(batch, seqlen, heads, kv_heads, B, topk, dtype):
     (2, 1500, 6, 3, 100, 4, torch.float16),
     (4, 2048, 8, 2, 128, 2, torch.float16),
     (1, 2048, 4, 2, 128, 1, torch.bfloat16),     # fallback: full causal attention
+    (1, 8192, 2, 1, 1024, 3, torch.bfloat16),    # few tiles: the forward cuts the history tiles' keys into parts
 ])
 def test_grouped_query_vs_oracle(batch, seqlen, heads, kv_heads, B, topk, dtype):
     """The grouped-query operator against the oracle run on key/value heads expanded with repeat_interleave
