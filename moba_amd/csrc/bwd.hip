@@ -492,18 +492,17 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
   const uint32_t lds_base = lds_addr(smem);
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   const int ld_rin = lane >> 4, ld_pc = lane & 15;
-  // Row lookups run one stage ahead of the copies: fetch_rows(qi) starts the loads of the
-  // gather-list entries of stage qi (self stages need none), issue_stage(qi) turns them into
-  // tokens and issues the copies.  Rows past the end repeat the last row.
-  int raw[5];  // rows 4*(4*i + wave) + lane/16 for i < 4 (Q and dO copies), row = lane (lse, delta)
+  // Row lookups run one stage ahead of the copies: fetch_rows(qi) starts the load of the gather-list entries of
+  // stage qi (self stages need none), prepare_stage(qi) turns them into tokens.  Rows past the end repeat the last
+  // row.  A lane looks up row `lane` of the stage (the row whose lse and delta it copies); the 16 rows whose Q and
+  // dO this wave copies, 4*(4*i + wave) + lane/16 for i < 4, are among those 64: their tokens come from the
+  // lanes that hold them (ds_bpermute), one lookup and one division per lane and stage instead of five.
+  int raw = 0;
   auto fetch_rows = [&](int qi) __attribute__((always_inline)) {
     if (qi < nself || qi >= ntile) return;
-    const int base = (qi - nself) * TQ;
-    const int* src = p.t.seg_dest + list_base;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) raw[i] = src[min(base + 4 * (4 * i + wave_u) + ld_rin, list_rows - 1)];
-    raw[4] = src[min(base + lane, list_rows - 1)];
+    raw = p.t.seg_dest[list_base + min((qi - nself) * TQ + lane, list_rows - 1)];
   };
+  const int row_src_lane4 = (4 * wave_u + ld_rin) * 4;  // 4 x the lane that holds row 4*(4*0 + wave) + lane/16
   uint64_t q_lane_base = 0, do_lane_base = 0;  // this lane's 16 bytes in token 0's row of q and dO, head h
   auto set_lane_bases = [&]() __attribute__((always_inline)) {
     const int c16 = ld_pc ^ (ld_rin << 2) ^ (wave_u & 3);  // sw_col16(4*slab + ld_rin, ld_pc) for slab = 4*i + wave
@@ -512,14 +511,12 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
   };
   int toks[5];  // tokens of the rows of the stage whose copies are being issued
   auto prepare_stage = [&](int qi) __attribute__((always_inline)) {
-    if (qi < nself) {
+    // (a list entry is (token*H + h)*K1 + 1 + slot with H*K1 >= 2: the quotient by H*K1 is the high word of the
+    // product with the magic number, shifted; exact for entries below 2^31)
+    toks[4] = qi < nself ? c0 + key0 + min(qi * TQ + lane, self_rows - 1)
+                         : (int)(__umulhi((uint32_t)raw, p.hk_magic) >> (p.hk_shift - 32));
 #pragma unroll
-      for (int i = 0; i < 4; ++i) toks[i] = c0 + key0 + min(qi * TQ + 4 * (4 * i + wave_u) + ld_rin, self_rows - 1);
-      toks[4] = c0 + key0 + min(qi * TQ + lane, self_rows - 1);
-    } else {
-#pragma unroll
-      for (int i = 0; i < 5; ++i) toks[i] = (int)(((uint64_t)(uint32_t)raw[i] * p.hk_magic) >> p.hk_shift);
-    }
+    for (int i = 0; i < 4; ++i) toks[i] = __builtin_amdgcn_ds_bpermute(row_src_lane4 + 64 * i, toks[4]);
   };
   // part g of the 8 row copies of a stage (slab g/2 of Q for even g, of dO for odd g); the last part also
   // brings the softmax statistics.  A copy instruction occupies the wave for tens of cycles while the
@@ -713,8 +710,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
   if (q_end == q_first) continue;  // (uniform)
   set_lane_bases();
   __syncthreads();  // every wave is done with the LDS stages of the previous head
-#pragma unroll
-  for (int i = 0; i < 5; ++i) raw[i] = 0;
+  raw = 0;
   fetch_rows(q_first);
   issue_stage(q_first, 0);
   fetch_rows(q_first + 1);
@@ -860,7 +856,8 @@ static int launch_bwd(const void* dout, const void* q, const void* k, const void
   // division by H*K1 as a multiplication: with s = 31 + ceil(log2 d) and m = floor(2^s / d) + 1 the
   // error m*d - 2^s is at most d <= 2^(s-31), so n*m >> s is the exact quotient for n < 2^31; m < 2^32
   const uint64_t hk = (uint64_t)H * (K + 1);
-  uint32_t lg = 0;
+  uint32_t lg = 1;  // (at least 1: the kernels take the product's high word and shift by hk_shift - 32; a list entry
+                    // exists only with K >= 1, hence H*K1 >= 2)
   while ((1ull << lg) < hk) ++lg;
   p.hk_shift = 31 + lg;
   p.hk_magic = (uint32_t)((1ull << p.hk_shift) / hk + 1);
