@@ -55,7 +55,7 @@ extern "C" {
 
 enum { MOBA_DTYPE_BF16 = 0, MOBA_DTYPE_F16 = 1 };
 
-#define MOBA_ABI_VERSION 108 /* the signatures below; moba_version() returns the number the library was built with */
+#define MOBA_ABI_VERSION 109 /* the signatures below; moba_version() returns the number the library was built with */
 int moba_version(void);
 const char* moba_strerror(int code);
 
@@ -106,10 +106,14 @@ int moba_plan_sizes(const moba_plan_t* plan, int H, int Hkv, int D, moba_sizes_t
  *   k          [S,H,D] elem (H here is the number of key/value heads); strides[2], strides[3] apply
  *   fchunk_tok [F] int32, first token of each filtered chunk
  *   kbar       [F,H,D] elem out (the mean rounded once to the element type)
- *   workspace  moba_chunk_mean_workspace_bytes() bytes, 8-byte aligned */
+ *   workspace  moba_chunk_mean_workspace_bytes() bytes, 8-byte aligned
+ *   clear      optional: clear_ints int32 of the caller's that the call zeroes on the way -- the cnt array that
+ *              moba_gate_topk then adds its counts into, one launch less than clearing it separately; NULL, 0
+ *              for none.  (Not done when F = 0: there are no lists to count then.) */
 size_t moba_chunk_mean_workspace_bytes(int H, int D, int F, int B);
 int moba_chunk_mean(const void* k, const int32_t* fchunk_tok, void* kbar, void* workspace, int64_t S, int H, int D,
-                    int F, int B, const int64_t* strides, int dtype, void* stream);
+                    int F, int B, const int64_t* strides, int dtype, int32_t* clear, int64_t clear_ints,
+                    void* stream);
 
 /* moba_chunk_mean for callers that cannot allocate or bring a workspace (code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and
@@ -129,10 +133,14 @@ int moba_chunk_mean_static(const void* k, const int32_t* fchunk_tok, void* kbar,
  *   sel        [S,H,K] int32 out: filtered-chunk ids, descending score, -1 padded
  *   scores_out optional [S,H,F] fp32, pre-filled with -inf by the caller; receives the
  *              score of every valid candidate (debug / test output), may be NULL
+ *   cnt        optional [P*H+1] int32, zero on entry (moba_chunk_mean's `clear`): receives, as a by-product, the
+ *              counts that moba_build_lists starts from (how many tokens of each query chunk and head picked
+ *              each chunk; pass counted = 1 there); needs pair_off [F+1], the table of moba_build_lists.
+ *              NULL: no counts.
  * K <= 64.  strides[0], strides[1] apply to q; kbar is packed [F,Hkv,D]. */
 int moba_gate_topk(const void* q, const void* kbar, const int32_t* cu_seqlens, const int32_t* seq_fbase, int32_t* sel,
-                   float* scores_out, int64_t S, int H, int Hkv, int D, int nseq, int F, int B, int K,
-                   const int64_t* strides, int dtype, void* stream);
+                   float* scores_out, const int32_t* pair_off, int32_t* cnt, int64_t S, int H, int Hkv, int D,
+                   int nseq, int F, int B, int K, const int64_t* strides, int dtype, void* stream);
 
 /* The selection step of moba/moba_efficient.py:365-371 alone, on caller-supplied
  * scores [S,H,F] fp32 (-inf = not a candidate).  Same routine as moba_gate_topk. */
@@ -144,7 +152,8 @@ int moba_topk_from_scores(const float* scores, int32_t* sel, int64_t S, int H, i
  *   chunk_tok [N+1], chunk_fb [N] (first filtered id of the chunk's sequence),
  *   chunk_local [N] (index of the chunk inside its sequence), pair_off [F+1]
  *   (prefix sum of the number of later chunks in the same sequence)   -- int32 tables
- *   cnt      [P*H+1] int32 scratch
+ *   cnt      [P*H+1] int32 scratch; with counted = 1 it holds on entry the counts moba_gate_topk left there
+ *            (the call then skips its own counting pass over sel), with counted = 0 its contents do not matter
  *   seg_off  [F*H+1] out, list start of segment (f,h);  tile_off [F*H+1] out, prefix
  *            sum of ceil(rows/tile_rows);  seg_dest [M] out, entries
  *            (token*H + h)*(K+1) + 1 + slot
@@ -155,7 +164,7 @@ int moba_topk_from_scores(const float* scores, int32_t* sel, int64_t S, int H, i
 int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, const int32_t* chunk_fb, const int32_t* chunk_local,
                      const int32_t* pair_off, int32_t* cnt, int32_t* seg_off, int32_t* tile_off, int32_t* seg_dest,
                      int32_t* tile_seg, int64_t S, int H, int K, int N, int F, int P, int cmax, int tile_rows,
-                     int64_t hist_bound, void* stream);
+                     int64_t hist_bound, int counted, void* stream);
 
 /* The tile tables of moba_build_lists alone, for another tile height: the forward and the backward kernels cut
  * the same gather lists into tiles of moba_fwd_tile_rows() and moba_bwd_tile_rows() rows.  No counterpart in the

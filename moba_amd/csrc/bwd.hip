@@ -83,8 +83,12 @@ template <class E>
 __global__ __launch_bounds__(256) void bwd_delta_kernel(const typename E::elem* __restrict__ dout,
                                                         const typename E::elem* __restrict__ out,
                                                         const float* __restrict__ lse, float* __restrict__ delta,
-                                                        float* __restrict__ lse2, int64_t rows) {
+                                                        float* __restrict__ lse2, int64_t rows,
+                                                        int* __restrict__ queues) {
   MOBA_ELEM_TYPES(E)
+  // the 16 tile counters of the two kernels that follow start at zero (here: one launch less than a kernel of its
+  // own, and, unlike a memset, safe to record into a graph)
+  if (blockIdx.x == 0 && threadIdx.x < 16) queues[threadIdx.x] = 0;
   const int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
   const int c8 = threadIdx.x & 15;
   float acc = 0.f;
@@ -870,8 +874,7 @@ static int launch_bwd(const void* dout, const void* q, const void* k, const void
     return MOBA_ERR_LAUNCH;
   const int64_t rows = S * H;
   hipLaunchKernelGGL(bwd_delta_kernel<E>, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st, (const elem*)dout,
-                     (const elem*)out, lse, delta, delta + S * H, rows);
-  hipLaunchKernelGGL(zero_queues_kernel, dim3(1), dim3(16), 0, st, queues, (int*)nullptr);  // a kernel, not a memset: graph safe
+                     (const elem*)out, lse, delta, delta + S * H, rows, queues);
   hipLaunchKernelGGL(bwd_dq_kernel<E>, dim3((unsigned)grid_q), dim3(256), kBwdDqLds, st, p);
   hipLaunchKernelGGL(bwd_dq_reduce_kernel<E>, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st,
                      (const elem*)part_dq, sel, (elem*)dq, rows, K + 1);

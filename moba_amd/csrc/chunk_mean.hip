@@ -22,9 +22,15 @@ template <class E>
 __global__ __launch_bounds__(256) void chunk_mean_partial_kernel(
     const typename E::elem* __restrict__ k, const int* __restrict__ fchunk_tok, double* __restrict__ partial,
     int HD8 /* H*D/8 */, int D8 /* D/8 */, int B, int nsplit, int tok_per_split, int64_t row_stride,
-    int64_t head_stride, int batch_rows, int64_t batch_stride, int cpb_log2) {
+    int64_t head_stride, int batch_rows, int64_t batch_stride, int cpb_log2, int* __restrict__ clear,
+    int64_t clear_ints) {
   MOBA_ELEM_TYPES(E)
   __shared__ double red[256 * 8];
+  if (clear) {  // an int array of the caller's to be zeroed on the way (the workgroups share it out)
+    const int64_t wg = blockIdx.x + (int64_t)gridDim.x * (blockIdx.y + (int64_t)gridDim.y * blockIdx.z);
+    const int64_t step = (int64_t)gridDim.x * gridDim.y * gridDim.z * 256;
+    for (int64_t i = wg * 256 + threadIdx.x; i < clear_ints; i += step) clear[i] = 0;
+  }
   const int cpb = 1 << cpb_log2, lanes = 256 >> cpb_log2;
   const int tl = threadIdx.x >> cpb_log2;
   const int col = blockIdx.z * cpb + (threadIdx.x & (cpb - 1));
@@ -157,7 +163,7 @@ extern "C" size_t moba_chunk_mean_workspace_bytes(int H, int D, int F, int B) {
 
 static int launch_chunk_mean(const void* k, const int32_t* fchunk_tok, void* kbar, double* partial, int H, int D,
                              int F, int B, int nsplit, int64_t kts, int64_t khs, int batch_rows, int64_t kbs, int dtype,
-                             hipStream_t st) {
+                             int* clear, int64_t clear_ints, hipStream_t st) {
   LaunchCheck launch_check;
   const int HD8 = H * D / 8;
   const int tps = (B + nsplit - 1) / nsplit;
@@ -167,12 +173,12 @@ static int launch_chunk_mean(const void* k, const int32_t* fchunk_tok, void* kba
   const dim3 fgrid((unsigned)((n + 255) / 256));
   if (dtype == MOBA_DTYPE_F16) {
     hipLaunchKernelGGL(chunk_mean_partial_kernel<F16>, grid, dim3(256), 0, st, (const f16*)k, fchunk_tok, partial,
-                       HD8, D / 8, B, nsplit, tps, kts, khs, batch_rows, kbs, cpb_log2);
+                       HD8, D / 8, B, nsplit, tps, kts, khs, batch_rows, kbs, cpb_log2, clear, clear_ints);
     hipLaunchKernelGGL(chunk_mean_finish_kernel<F16>, fgrid, dim3(256), 0, st, (const double*)partial, (f16*)kbar,
                        HD8, B, nsplit, F);
   } else {
     hipLaunchKernelGGL(chunk_mean_partial_kernel<Bf16>, grid, dim3(256), 0, st, (const bf16*)k, fchunk_tok, partial,
-                       HD8, D / 8, B, nsplit, tps, kts, khs, batch_rows, kbs, cpb_log2);
+                       HD8, D / 8, B, nsplit, tps, kts, khs, batch_rows, kbs, cpb_log2, clear, clear_ints);
     hipLaunchKernelGGL(chunk_mean_finish_kernel<Bf16>, fgrid, dim3(256), 0, st, (const double*)partial, (bf16*)kbar,
                        HD8, B, nsplit, F);
   }
@@ -200,15 +206,16 @@ static int check_chunk_mean_args(const void* k, const int32_t* fchunk_tok, void*
 
 extern "C" int moba_chunk_mean(const void* k, const int32_t* fchunk_tok, void* kbar, void* workspace,
                                int64_t S, int H, int D, int F, int B, const int64_t* strides, int dtype,
-                               void* stream) {
-  if (F == 0) return MOBA_OK;
+                               int32_t* clear, int64_t clear_ints, void* stream) {
+  if (clear_ints < 0 || (clear_ints > 0 && !clear)) return MOBA_ERR_ARG;
+  if (F == 0) return MOBA_OK;  // (nothing to clear for: without chunks there are no lists to count)
   int64_t kts = 0, khs = 0, kbs = 0;
   int kbr = 0;
   const int rc = check_chunk_mean_args(k, fchunk_tok, kbar, S, H, D, F, B, strides, dtype, kts, khs, kbr, kbs);
   if (rc != MOBA_OK) return rc;
   if (!workspace || ((uintptr_t)workspace & 7)) return MOBA_ERR_ARG;
   return launch_chunk_mean(k, fchunk_tok, kbar, (double*)workspace, H, D, F, B, pick_nsplit(H * D / 8, F, B), kts, khs,
-                           kbr, kbs, dtype, (hipStream_t)stream);
+                           kbr, kbs, dtype, clear_ints > 0 ? clear : nullptr, clear_ints, (hipStream_t)stream);
 }
 
 // ---- the same stage for callers that cannot allocate: the partial sums live in a fixed array of the library ----
@@ -251,5 +258,6 @@ extern "C" int moba_chunk_mean_static(const void* k, const int32_t* fchunk_tok, 
   while (nsplit > 1 && per_split * nsplit > kStaticPartialBytes) nsplit /= 2;
   double* partial = static_partials();
   if (!partial) return MOBA_ERR_LAUNCH;
-  return launch_chunk_mean(k, fchunk_tok, kbar, partial, H, D, F, B, nsplit, kts, khs, kbr, kbs, dtype, (hipStream_t)stream);
+  return launch_chunk_mean(k, fchunk_tok, kbar, partial, H, D, F, B, nsplit, kts, khs, kbr, kbs, dtype, nullptr, 0,
+                           (hipStream_t)stream);
 }

@@ -704,44 +704,48 @@ __global__ __launch_bounds__(256) void moba_merge_kernel(const typename E::elem*
   const int K = K1 - 1;
   const float* pl = part_lse + row * K1;
   const int* ps = sel + row * K;
-  const elem* po = part_o + row * K1 * kHeadDim + c8 * 8;
-  const elem* const po0 = po;  // the self slot: always written
+  const elem* po = part_o + row * K1 * kHeadDim + c8 * 8;  // the self slot: always written
   // Lane c8 of the row's group fetches the LSE and the presence of slot j0 + c8, so the slot
   // statistics cost one round trip per 16 slots; weights travel by lane shuffles.  Absent slots
   // are redirected to the self slot with weight 0, so the partial-output loads are unconditional and
   // eight of them are in flight together.  Slots are accumulated in ascending order.
   // With `parts` > 1 the history slots hold `parts` partials each (the forward cut the chunks' keys): those of
   // part g lie rows * K1 slot rows behind those of part g - 1; the self slot has part 0 only.
-  const int64_t part_rows = rows * K1;
+  // The parts are slots like any other: slot v of the parts * K1 is slot v % K1 of part v / K1, at slot row
+  // (v / K1) * rows * K1 + v % K1 of the row's first (an int: the buffers hold fewer than 2^31 slot rows).
+  const int nvirt = parts * K1;
+  const int part_rows = (int)(rows * K1);
   float mx = -INFINITY;
-  for (int part = 0; part < parts; ++part)
-    for (int j0 = 0; j0 < K1; j0 += 16) {
-      const int j = j0 + c8;
-      const bool ok = j < K1 && (j == 0 ? part == 0 : ps[j - 1] >= 0);
-      const float l = ok ? pl[part * part_rows + j] : -INFINITY;
-      mx = fmaxf(mx, l);
-    }
+  for (int v0 = 0; v0 < nvirt; v0 += 16) {
+    const int v = v0 + c8;
+    const int part = parts == 1 ? 0 : v / K1, j = v - part * K1;
+    const bool ok = v < nvirt && (j == 0 ? part == 0 : ps[j - 1] >= 0);
+    const float l = ok ? pl[(int64_t)part * part_rows + j] : -INFINITY;
+    mx = fmaxf(mx, l);
+  }
 #pragma unroll
   for (int o = 8; o >= 1; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 16));
   float acc[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.f;
   float wsum = 0.f;
-  for (int part = 0; part < parts; ++part, pl += part_rows, po += part_rows * kHeadDim)
-  for (int j0 = 0; j0 < K1; j0 += 16) {
-    const int j = j0 + c8;
-    const bool ok = j < K1 && (j == 0 ? part == 0 : ps[j - 1] >= 0);
-    const float wl = ok ? fast_exp2(pl[j] - mx) : 0.f;
-    const int nslot = min(16, K1 - j0);
+  for (int v0 = 0; v0 < nvirt; v0 += 16) {
+    const int v = v0 + c8;
+    const int part = parts == 1 ? 0 : v / K1, j = v - part * K1;
+    const bool ok = v < nvirt && (j == 0 ? part == 0 : ps[j - 1] >= 0);
+    const int at = part * part_rows + j;  // (0, the self slot, for a slot that is absent)
+    const float wl = ok ? fast_exp2(pl[(int64_t)part * part_rows + j] - mx) : 0.f;
+    const int at_ok = ok ? at : 0;
+    const int nslot = min(16, nvirt - v0);
     for (int u0 = 0; u0 < nslot; u0 += 8) {
       elem8 x[8];
       float w[8];
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
-        w[u] = __shfl(wl, u0 + u, 16);           // 0 for slots past K1 too (their lanes computed ok = false)
-        const elem* src = w[u] > 0.f ? po + (int64_t)(j0 + u0 + u) * kHeadDim : po0;
+        w[u] = __shfl(wl, u0 + u, 16);           // 0 for slots past the last too (their lanes computed ok = false)
+        const int where = parts == 1 ? (w[u] > 0.f ? v0 + u0 + u : 0) : __shfl(at_ok, u0 + u, 16);
         if (u0 + u < nslot)                      // uniform: no loads for slots that do not exist
-          x[u] = __builtin_nontemporal_load(reinterpret_cast<const elem8*>(src));
+          x[u] = __builtin_nontemporal_load(reinterpret_cast<const elem8*>(po + (int64_t)where * kHeadDim));
       }
 #pragma unroll
       for (int u = 0; u < 8; ++u) {

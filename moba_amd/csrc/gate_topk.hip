@@ -56,7 +56,7 @@ __global__ __launch_bounds__(256) void gate_topk_kernel(
     const typename E::elem* __restrict__ q, const typename E::elem* __restrict__ kbar, const int* __restrict__ cu_seqlens,
     const int* __restrict__ seq_fbase, int* __restrict__ sel, float* __restrict__ scores_out,
     int S, int H, int Hkv, int nseq, int F, int B, int K, int64_t q_tok_stride, int64_t q_head_stride,
-    int batch_rows, int64_t q_batch_stride) {
+    int batch_rows, int64_t q_batch_stride, const int* __restrict__ pair_off, int* __restrict__ cnt) {
   MOBA_ELEM_TYPES(E)
   __shared__ float sc[4][64][33];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -150,6 +150,46 @@ __global__ __launch_bounds__(256) void gate_topk_kernel(
     for (int j = 0; j < KMAX; ++j)
       if (j < K) dst[j] = top.idx[j];
   }
+  // The gather lists' counts as a by-product: how many tokens of a (query chunk, head) picked each earlier chunk,
+  // added into cnt[(chunk, head, query chunk)] (integer sums: the order of the additions does not matter).  A
+  // wave's 64 tokens lie in one query chunk, or in a few: one round per chunk, through a histogram in LDS.
+  if (!cnt) return;
+  __syncthreads();  // (the staged lists are stored)
+  constexpr int kHist = (int)(sizeof(sc) / sizeof(int)) / 4;
+  int* hist = reinterpret_cast<int*>(&sc[0][0][0]) + wave * kHist;
+  const bool counts = head_ok && s < S && c > 0;
+  uint64_t todo = __ballot(counts);
+  while (todo) {  // (wave-uniform)
+    const int leader = __ffsll((unsigned long long)todo) - 1;
+    const int cc = __shfl(c, leader, 64), cfb = __shfl(fb, leader, 64);
+    const bool mine = counts && c == cc && fb == cfb;
+    for (int w0 = 0; w0 < cc; w0 += kHist) {
+      const int wn = min(kHist, cc - w0);
+      for (int i = lane; i < wn; i += 64) hist[i] = 0;
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      if (mine) {
+#pragma unroll
+        for (int j = 0; j < KMAX; ++j) {
+          const int i = (j < K && top.idx[j] >= 0) ? top.idx[j] - cfb - w0 : -1;
+          if ((unsigned)i < (unsigned)wn) atomicAdd(&hist[i], 1);
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      for (int i = lane; i < wn; i += 64) {
+        const int n = hist[i];
+        if (n) {
+          const int f = cfb + w0 + i;
+          const int q0 = pair_off[f], nq = pair_off[f + 1] - q0;
+          atomicAdd(&cnt[q0 * H + h * nq + (cc - (w0 + i) - 1)], n);
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+    }
+    todo &= ~__ballot(mine);
+  }
 }
 
 // Selection alone, on scores supplied by the caller ([S, H, F] fp32, -inf where a
@@ -184,10 +224,11 @@ using namespace moba;
   else return MOBA_ERR_LIMIT;
 
 extern "C" int moba_gate_topk(const void* q, const void* kbar, const int32_t* cu_seqlens, const int32_t* seq_fbase,
-                              int32_t* sel, float* scores_out, int64_t S, int H, int Hkv, int D, int nseq, int F,
-                              int B, int K, const int64_t* strides, int dtype, void* stream) {
+                              int32_t* sel, float* scores_out, const int32_t* pair_off, int32_t* cnt, int64_t S, int H,
+                              int Hkv, int D, int nseq, int F, int B, int K, const int64_t* strides, int dtype,
+                              void* stream) {
   LaunchCheck launch_check;
-  if (!q || !kbar || !cu_seqlens || !seq_fbase || !sel) return MOBA_ERR_ARG;
+  if (!q || !kbar || !cu_seqlens || !seq_fbase || !sel || (cnt && !pair_off)) return MOBA_ERR_ARG;
   if (Hkv <= 0 || H % Hkv != 0) return MOBA_ERR_ARG;
   if (dtype != MOBA_DTYPE_BF16 && dtype != MOBA_DTYPE_F16) return MOBA_ERR_UNSUPPORTED;
   if (S <= 0 || S > 0x7fffffff - 64 || H <= 0 || nseq <= 0 || F <= 0 || B <= 0 || K <= 0) return MOBA_ERR_ARG;
@@ -204,10 +245,12 @@ extern "C" int moba_gate_topk(const void* q, const void* kbar, const int32_t* cu
 #define CALL(KM)                                                                                               \
   if (dtype == MOBA_DTYPE_F16)                                                                                 \
     hipLaunchKernelGGL((gate_topk_kernel<F16, KM>), grid, dim3(256), 0, st, (const f16*)q, (const f16*)kbar,   \
-                       cu_seqlens, seq_fbase, sel, scores_out, (int)S, H, Hkv, nseq, F, B, K, qts, qhs, qbr, qbs);  \
+                       cu_seqlens, seq_fbase, sel, scores_out, (int)S, H, Hkv, nseq, F, B, K, qts, qhs, qbr, qbs, \
+                       pair_off, cnt);                                                                         \
   else                                                                                                         \
     hipLaunchKernelGGL((gate_topk_kernel<Bf16, KM>), grid, dim3(256), 0, st, (const bf16*)q, (const bf16*)kbar, \
-                       cu_seqlens, seq_fbase, sel, scores_out, (int)S, H, Hkv, nseq, F, B, K, qts, qhs, qbr, qbs)
+                       cu_seqlens, seq_fbase, sel, scores_out, (int)S, H, Hkv, nseq, F, B, K, qts, qhs, qbr, qbs, \
+                       pair_off, cnt)
   MOBA_DISPATCH_K(K, CALL)
 #undef CALL
   return launch_check.result();

@@ -26,7 +26,8 @@ __device__ __forceinline__ int cnt_index(const int* __restrict__ pair_off, int f
   return p0 * H + h * nq + crel;
 }
 
-__global__ __launch_bounds__(256) void lists_count_kernel(
+template <int NT>  // threads per workgroup
+__global__ __launch_bounds__(NT) void lists_count_kernel(
     const int* __restrict__ sel, const int* __restrict__ chunk_tok, const int* __restrict__ chunk_fb,
     const int* __restrict__ chunk_local, const int* __restrict__ pair_off, int* __restrict__ cnt, int H, int K) {
   extern __shared__ int lds[];
@@ -35,9 +36,9 @@ __global__ __launch_bounds__(256) void lists_count_kernel(
   if (c == 0) return;
   const int fb = chunk_fb[cq];
   const int t0 = chunk_tok[cq], t1 = chunk_tok[cq + 1];
-  for (int i = threadIdx.x; i < c; i += 256) lds[i] = 0;
+  for (int i = threadIdx.x; i < c; i += NT) lds[i] = 0;
   __syncthreads();
-  for (int s = t0 + threadIdx.x; s < t1; s += 256) {
+  for (int s = t0 + threadIdx.x; s < t1; s += NT) {
     const int* src = sel + ((int64_t)s * H + h) * K;
     for (int j = 0; j < K; ++j) {
       const int i = src[j] - fb;
@@ -45,63 +46,40 @@ __global__ __launch_bounds__(256) void lists_count_kernel(
     }
   }
   __syncthreads();
-  for (int i = threadIdx.x; i < c; i += 256) cnt[cnt_index(pair_off, fb + i, h, H, c - i - 1)] = lds[i];
+  for (int i = threadIdx.x; i < c; i += NT) cnt[cnt_index(pair_off, fb + i, h, H, c - i - 1)] = lds[i];
 }
 
-template <int KC>  // compile-time bound on K: a lane keeps its token's picks in registers
-__global__ __launch_bounds__(256) void lists_fill_kernel(
+// the lanes of a wave see each other's LDS writes: a wave's LDS instructions execute in the order issued, so only
+// the compiler has to be held to that order
+__device__ __forceinline__ void wave_lds_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// KC: compile-time bound on K (a lane keeps its token's picks in registers); NW: waves of the workgroup, which
+// own consecutive NW-ths of the chunk.  base_of() returns the scanned count array, in global memory or in LDS;
+// it is called by the whole workgroup once the first loads of the picks are under way (it may synchronise).
+template <int KC, int NW, class BaseFn>
+__device__ __forceinline__ void lists_fill_body(
     const int* __restrict__ sel, const int* __restrict__ chunk_tok, const int* __restrict__ chunk_fb,
-    const int* __restrict__ chunk_local, const int* __restrict__ pair_off, const int* __restrict__ base,
-    int* __restrict__ seg_dest, int H, int K) {
-  extern __shared__ int lds[];
+    const int* __restrict__ chunk_local, const int* __restrict__ pair_off, BaseFn base_of,
+    int* __restrict__ seg_dest, int H, int K, int* lds) {
   const int cq = blockIdx.x, h = blockIdx.y;
   const int c = chunk_local[cq];
-  if (c == 0) return;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  int* pos = lds;                                            // [4][c] running list position per wave
-  unsigned* bits = reinterpret_cast<unsigned*>(lds + 4 * c);  // [4][c][2] lanes of the batch that picked i
+  int* pos = lds;                                             // [NW][c] running list position per wave
+  unsigned* bits = reinterpret_cast<unsigned*>(lds + NW * c);  // [NW][c][2] lanes of the batch that picked i
   const int fb = chunk_fb[cq];
   const int t0 = chunk_tok[cq], t1 = chunk_tok[cq + 1];
-  const int qlen = (t1 - t0 + 3) / 4;
+  const int qlen = (t1 - t0 + NW - 1) / NW;
   const int w0 = min(t1, t0 + wave * qlen), w1 = min(t1, w0 + qlen);
   const int K1 = K + 1;
-  for (int i = threadIdx.x; i < 4 * c; i += 256) {
-    pos[i] = 0;
-    bits[2 * i] = 0;
-    bits[2 * i + 1] = 0;
-  }
-  __syncthreads();
-  // per-wave counts
-  for (int s = w0 + lane; s < w1; s += 64) {
-    const int* src = sel + ((int64_t)s * H + h) * K;
-#pragma unroll
-    for (int j = 0; j < KC; ++j) {
-      if (j >= K) break;
-      const int i = src[j] - fb;
-      if ((unsigned)i < (unsigned)c) atomicAdd(&pos[wave * c + i], 1);
-    }
-  }
-  __syncthreads();
-  // counts -> start positions: global base of (f, h, this query chunk) plus the earlier waves
-  for (int i = threadIdx.x; i < c; i += 256) {
-    int run = base[cnt_index(pair_off, fb + i, h, H, c - i - 1)];
-#pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      const int n = pos[w * c + i];
-      pos[w * c + i] = run;
-      run += n;
-    }
-  }
-  __syncthreads();
-  const int nbatch = (qlen + 63) / 64;  // same for the four waves
-  int* wpos = pos + wave * c;
-  unsigned* wbits = bits + 2 * wave * c;
-  const uint64_t below = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
-  for (int bi = 0; bi < nbatch; ++bi) {
+  // candidate index of each pick of this lane's token in a batch of 64, -1 when it is not a list entry
+  auto load_picks = [&](int bi, int (&pick)[KC]) {
     const int s = w0 + bi * 64 + lane;
     const bool active = s < w1;
     const int* src = sel + ((int64_t)(active ? s : t0) * H + h) * K;
-    int pick[KC];  // candidate index of each pick, -1 when it is not a list entry
 #pragma unroll
     for (int j = 0; j < KC; ++j) {
       pick[j] = -1;
@@ -110,10 +88,62 @@ __global__ __launch_bounds__(256) void lists_fill_kernel(
         if (active && (unsigned)i < (unsigned)c) pick[j] = i;
       }
     }
+  };
+  constexpr int kKept = 2;  // the picks of the first batches stay in registers from the counting pass on
+  int kept[kKept][KC];
+#pragma unroll
+  for (int bi = 0; bi < kKept; ++bi) load_picks(bi, kept[bi]);
+  const int* base = base_of();
+  if (c == 0) return;  // (the whole workgroup)
+  for (int i = threadIdx.x; i < NW * c; i += NW * 64) {
+    pos[i] = 0;
+    bits[2 * i] = 0;
+    bits[2 * i + 1] = 0;
+  }
+  __syncthreads();
+  const int nbatch = (qlen + 63) / 64;  // same for all waves
+  // per-wave counts
+  for (int bi = 0; bi < nbatch; ++bi) {
+    int pick[KC];
+    if (bi < kKept) {
+#pragma unroll
+      for (int j = 0; j < KC; ++j) pick[j] = bi == 0 ? kept[0][j] : kept[1][j];
+    } else {
+      load_picks(bi, pick);
+    }
+#pragma unroll
+    for (int j = 0; j < KC; ++j)
+      if (pick[j] >= 0) atomicAdd(&pos[wave * c + pick[j]], 1);
+  }
+  __syncthreads();
+  // counts -> start positions: global base of (f, h, this query chunk) plus the earlier waves
+  for (int i = threadIdx.x; i < c; i += NW * 64) {
+    int run = base[cnt_index(pair_off, fb + i, h, H, c - i - 1)];
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+      const int n = pos[w * c + i];
+      pos[w * c + i] = run;
+      run += n;
+    }
+  }
+  __syncthreads();
+  // from here on a wave works on its own positions and lane masks only
+  int* wpos = pos + wave * c;
+  unsigned* wbits = bits + 2 * wave * c;
+  const uint64_t below = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+  for (int bi = 0; bi < nbatch; ++bi) {
+    const int s = w0 + bi * 64 + lane;
+    int pick[KC];
+    if (bi < kKept) {
+#pragma unroll
+      for (int j = 0; j < KC; ++j) pick[j] = bi == 0 ? kept[0][j] : kept[1][j];
+    } else {
+      load_picks(bi, pick);
+    }
 #pragma unroll
     for (int j = 0; j < KC; ++j)
       if (pick[j] >= 0) atomicOr(&wbits[2 * pick[j] + (lane >> 5)], 1u << (lane & 31));
-    __syncthreads();
+    wave_lds_sync();
 #pragma unroll
     for (int j = 0; j < KC; ++j) {
       if (pick[j] >= 0) {
@@ -123,7 +153,7 @@ __global__ __launch_bounds__(256) void lists_fill_kernel(
         seg_dest[wpos[i] + rank] = (s * H + h) * K1 + 1 + j;
       }
     }
-    __syncthreads();
+    wave_lds_sync();
 #pragma unroll
     for (int j = 0; j < KC; ++j) {
       if (pick[j] >= 0) {
@@ -136,8 +166,17 @@ __global__ __launch_bounds__(256) void lists_fill_kernel(
         }
       }
     }
-    __syncthreads();
+    wave_lds_sync();
   }
+}
+
+template <int KC>
+__global__ __launch_bounds__(256) void lists_fill_kernel(
+    const int* __restrict__ sel, const int* __restrict__ chunk_tok, const int* __restrict__ chunk_fb,
+    const int* __restrict__ chunk_local, const int* __restrict__ pair_off, const int* __restrict__ base,
+    int* __restrict__ seg_dest, int H, int K) {
+  extern __shared__ int lds[];
+  lists_fill_body<KC, 4>(sel, chunk_tok, chunk_fb, chunk_local, pair_off, [&] { return base; }, seg_dest, H, K, lds);
 }
 
 // exclusive prefix sum of a[0..n) in place, total stored at a[n]; one workgroup.
@@ -222,12 +261,11 @@ __global__ __launch_bounds__(256) void lists_tile_seg_kernel(const int* __restri
 // seg_off is given), the scan of the tile counts and lists_tile_seg_kernel do, in one workgroup with the counts
 // in LDS -- three dependent launches of a few microseconds each are most of the list stage of a small problem.
 constexpr int kTailMaxSegments = 4096, kTailMaxTiles = 16384;
-__global__ __launch_bounds__(1024) void lists_tail_kernel(const int* __restrict__ base, const int* __restrict__ pair_off,
-                                                          int* __restrict__ seg_off, int* __restrict__ tile_off,
-                                                          int* __restrict__ tile_seg, int F, int H, int tile_rows,
-                                                          int bound) {
-  __shared__ int off[kTailMaxSegments + 1];
-  __shared__ int wsum[16];
+// (off: kTailMaxSegments + 1 ints of LDS, wsum: 16; `base` may point into LDS)
+__device__ __forceinline__ void lists_tail_body(const int* base, const int* __restrict__ pair_off,
+                                                int* __restrict__ seg_off, int* __restrict__ tile_off,
+                                                int* __restrict__ tile_seg, int F, int H, int tile_rows, int bound,
+                                                int* off, int* wsum) {
   const int FH = F * H, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   // this thread's four consecutive segments: list starts (written out when they come from the counts), tile counts
   int v[4];
@@ -298,6 +336,69 @@ __global__ __launch_bounds__(1024) void lists_tail_kernel(const int* __restrict_
   }
 }
 
+__global__ __launch_bounds__(1024) void lists_tail_kernel(const int* __restrict__ base, const int* __restrict__ pair_off,
+                                                          int* __restrict__ seg_off, int* __restrict__ tile_off,
+                                                          int* __restrict__ tile_seg, int F, int H, int tile_rows,
+                                                          int bound) {
+  __shared__ int off[kTailMaxSegments + 1];
+  __shared__ int wsum[16];
+  lists_tail_body(base, pair_off, seg_off, tile_off, tile_seg, F, H, tile_rows, bound, off, wsum);
+}
+
+// Small problems (few counts, few segments, few tiles, few workgroups): the scan, the fill and the tail in one
+// launch.  Every workgroup scans the whole count array for itself into LDS (cheaper than a launch that does it
+// once); workgroups (cq < N, h) fill their part of the lists with 16 waves, workgroup (N, 0) writes the segment and
+// tile tables, which depend on the scanned counts only.
+constexpr int kFusedMaxCounts = 4096, kFusedMaxCand = 128;
+template <int KC>
+__global__ __launch_bounds__(1024) void lists_fill_tail_kernel(
+    const int* __restrict__ sel, const int* __restrict__ chunk_tok, const int* __restrict__ chunk_fb,
+    const int* __restrict__ chunk_local, const int* __restrict__ pair_off, const int* __restrict__ cnt,
+    int* __restrict__ seg_dest, int* __restrict__ seg_off, int* __restrict__ tile_off, int* __restrict__ tile_seg,
+    int N, int H, int K, int F, int PH, int tile_rows, int bound) {
+  __shared__ int sbase[kFusedMaxCounts + 1];
+  // the tail's tile starts, or the fill's positions and lane masks: 16 waves x 3 ints per candidate chunk
+  __shared__ int off[kFusedMaxCand * 48 > kTailMaxSegments + 1 ? kFusedMaxCand * 48 : kTailMaxSegments + 1];
+  __shared__ int wsum[16];
+  if (blockIdx.x == N && blockIdx.y != 0) return;
+  auto scanned_counts = [&]() -> const int* {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int i0 = tid * 4;
+    int v[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = (i0 + e < PH) ? cnt[i0 + e] : 0;
+    const int tsum = v[0] + v[1] + v[2] + v[3];
+    int inc = tsum;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int t = __shfl_up(inc, o, 64);
+      if (lane >= o) inc += t;
+    }
+    if (lane == 63) wsum[wave] = inc;
+    __syncthreads();
+    int woff = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) {
+      const int x = wsum[w];
+      if (w < wave) woff += x;
+      total += x;
+    }
+    int run = woff + inc - tsum;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if (i0 + e < PH) sbase[i0 + e] = run;
+      run += v[e];
+    }
+    if (tid == 0) sbase[PH] = total;
+    __syncthreads();
+    return sbase;
+  };
+  if (blockIdx.x == N)
+    lists_tail_body(scanned_counts(), pair_off, seg_off, tile_off, tile_seg, F, H, tile_rows, bound, off, wsum);
+  else
+    lists_fill_body<KC, 16>(sel, chunk_tok, chunk_fb, chunk_local, pair_off, scanned_counts, seg_dest, H, K, off);
+}
+
 }  // namespace moba
 
 using namespace moba;
@@ -308,7 +409,7 @@ extern "C" int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, co
                                 const int32_t* chunk_local, const int32_t* pair_off, int32_t* cnt,
                                 int32_t* seg_off, int32_t* tile_off, int32_t* seg_dest, int32_t* tile_seg,
                                 int64_t S, int H, int K, int N, int F, int P, int cmax, int tile_rows,
-                                int64_t hist_bound, void* stream) {
+                                int64_t hist_bound, int counted, void* stream) {
   LaunchCheck launch_check;
   if (!sel || !chunk_tok || !chunk_fb || !chunk_local || !pair_off || !cnt || !seg_off || !tile_off || !seg_dest ||
       !tile_seg)
@@ -319,8 +420,23 @@ extern "C" int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, co
   if (H > 65535 || (size_t)cmax * 48 > 160 * 1024) return MOBA_ERR_LIMIT;
   hipStream_t st = (hipStream_t)stream;
   dim3 grid(N, H);
-  hipLaunchKernelGGL(lists_count_kernel, grid, dim3(256), (size_t)cmax * 4, st, sel, chunk_tok, chunk_fb,
-                     chunk_local, pair_off, cnt, H, K);
+  const bool small_tail = (int64_t)F * H < kTailMaxSegments && hist_bound <= kTailMaxTiles;
+  if (small_tail && (int64_t)P * H <= kFusedMaxCounts && cmax <= kFusedMaxCand && (int64_t)N * H <= 512 && K <= 16) {
+    if (!counted)
+      hipLaunchKernelGGL(lists_count_kernel<1024>, grid, dim3(1024), (size_t)cmax * 4, st, sel, chunk_tok, chunk_fb,
+                         chunk_local, pair_off, cnt, H, K);
+#define MOBA_FILL_TAIL(KC)                                                                                       \
+  hipLaunchKernelGGL(lists_fill_tail_kernel<KC>, dim3(N + 1, H), dim3(1024), 0, st, sel, chunk_tok, chunk_fb,    \
+                     chunk_local, pair_off, (const int*)cnt, seg_dest, seg_off, tile_off, tile_seg, N, H, K, F,  \
+                     P * H, tile_rows, (int)hist_bound)
+    if (K <= 4) MOBA_FILL_TAIL(4);
+    else MOBA_FILL_TAIL(16);
+#undef MOBA_FILL_TAIL
+    return launch_check.result();
+  }
+  if (!counted)
+    hipLaunchKernelGGL(lists_count_kernel<256>, grid, dim3(256), (size_t)cmax * 4, st, sel, chunk_tok, chunk_fb,
+                       chunk_local, pair_off, cnt, H, K);
   hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(1024), 0, st, cnt, P * H);
   // more than 64 KiB of dynamic LDS has to be asked for explicitly
 #define MOBA_FILL(KC)                                                                                          \
@@ -337,7 +453,7 @@ extern "C" int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, co
   else if (K <= 64) MOBA_FILL(64)
   else return MOBA_ERR_LIMIT;
 #undef MOBA_FILL
-  if ((int64_t)F * H < kTailMaxSegments && hist_bound <= kTailMaxTiles) {
+  if (small_tail) {
     hipLaunchKernelGGL(lists_tail_kernel, dim3(1), dim3(1024), 0, st, (const int*)cnt, pair_off, seg_off, tile_off,
                        tile_seg, F, H, tile_rows, (int)hist_bound);
     return launch_check.result();

@@ -132,8 +132,9 @@ def _check_qkv(q, k, v, gqa=False):
 
 
 # ----------------------------------------------------------------------------- stages
-def chunk_mean(k: torch.Tensor, plan: MobaPlan) -> torch.Tensor:
-    """kbar [F, H, D] in k's dtype: mean of K over every filtered chunk (exact sum, rounded once)."""
+def chunk_mean(k: torch.Tensor, plan: MobaPlan, clear: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """kbar [F, H, D] in k's dtype: mean of K over every filtered chunk (exact sum, rounded once).
+    `clear`: an int32 tensor the call zeroes on the way (the counts array of gate_topk)."""
     lib = _lib.load()
     S, H, D = _dims(k)
     if not _addressable(k):
@@ -142,14 +143,17 @@ def chunk_mean(k: torch.Tensor, plan: MobaPlan) -> torch.Tensor:
     nbytes = lib.moba_chunk_mean_workspace_bytes(H, D, plan.F, plan.chunk_size)
     ws = torch.empty(nbytes // 8, dtype=torch.float64, device=k.device)
     _lib.check(lib.moba_chunk_mean(_ptr(k), _ptr(plan.tables["fchunk_tok"]), _ptr(kbar), _ptr(ws), S, H, D, plan.F,
-                                   plan.chunk_size, _strides(None, k), _dtype_code(k), _stream(k.device)),
+                                   plan.chunk_size, _strides(None, k), _dtype_code(k), _ptr(clear),
+                                   0 if clear is None else clear.numel(), _stream(k.device)),
                "moba_chunk_mean")
     return kbar
 
 
-def gate_topk(q: torch.Tensor, kbar: torch.Tensor, plan: MobaPlan, return_scores: bool = False):
+def gate_topk(q: torch.Tensor, kbar: torch.Tensor, plan: MobaPlan, return_scores: bool = False,
+              cnt: Optional[torch.Tensor] = None):
     """sel [S, H, K] int32: selected filtered-chunk ids per (token, head), -1 padded.
-    kbar may have fewer heads than q (grouped-query attention)."""
+    kbar may have fewer heads than q (grouped-query attention).  `cnt` (list_buffers()[0], zeroed): receives
+    the counts build_lists starts from."""
     lib = _lib.load()
     S, H, D = _dims(q)
     Hkv = kbar.shape[1]
@@ -160,8 +164,9 @@ def gate_topk(q: torch.Tensor, kbar: torch.Tensor, plan: MobaPlan, return_scores
     if return_scores:
         scores = torch.full((S, H, plan.F), float("-inf"), dtype=torch.float32, device=q.device)
     _lib.check(lib.moba_gate_topk(_ptr(q), _ptr(kbar), _ptr(plan.tables["cu_seqlens"]), _ptr(plan.tables["seq_fbase"]),
-                                  _ptr(sel), _ptr(scores), S, H, Hkv, D, plan.nseq, plan.F, plan.chunk_size, plan.K,
-                                  _strides(q, None), _dtype_code(q), _stream(q.device)), "moba_gate_topk")
+                                  _ptr(sel), _ptr(scores), _ptr(plan.tables["pair_off"]), _ptr(cnt), S, H, Hkv, D,
+                                  plan.nseq, plan.F, plan.chunk_size, plan.K, _strides(q, None), _dtype_code(q),
+                                  _stream(q.device)), "moba_gate_topk")
     return (sel, scores) if return_scores else sel
 
 
@@ -176,26 +181,33 @@ def topk_from_scores(scores: torch.Tensor, K: int) -> torch.Tensor:
     return sel
 
 
-def build_lists(sel: torch.Tensor, plan: MobaPlan, tile_rows: int = FWD_TILE_ROWS):
-    """(seg_off [F*H+1], tile_off [F*H+1], seg_dest [M], tile_seg [tile bound]) int32 -- see csrc/lists.hip.
-    The tile tables cut the lists into tiles of `tile_rows` rows (the forward kernel's by default)."""
-    lib = _lib.load()
-    S, H, K = sel.shape
-    dev = sel.device
-    M = plan.pairs_per_head * H
-    bound = plan.hist_tile_bound(H, tile_rows)
-    # one allocation for the five arrays (each start a multiple of 4 ints)
-    sizes = [plan.P * H + 1, plan.F * H + 1, plan.F * H + 1, max(M, 1), bound]
+def list_buffers(plan: MobaPlan, H: int, device, tile_rows: int = FWD_TILE_ROWS):
+    """(cnt [P*H+1], seg_off [F*H+1], tile_off [F*H+1], seg_dest [M], tile_seg [tile bound]) int32, uninitialised:
+    the arrays of build_lists, in one allocation (each start a multiple of 4 ints)."""
+    sizes = [plan.P * H + 1, plan.F * H + 1, plan.F * H + 1, max(plan.pairs_per_head * H, 1),
+             plan.hist_tile_bound(H, tile_rows)]
     starts = [0]
     for n in sizes:
         starts.append(starts[-1] + (n + 3) // 4 * 4)
-    buf = torch.empty(starts[-1], dtype=torch.int32, device=dev)
-    cnt, seg_off, tile_off, seg_dest, tile_seg = (buf[a:a + n] for a, n in zip(starts, sizes))
+    buf = torch.empty(starts[-1], dtype=torch.int32, device=device)
+    return tuple(buf[a:a + n] for a, n in zip(starts, sizes))
+
+
+def build_lists(sel: torch.Tensor, plan: MobaPlan, tile_rows: int = FWD_TILE_ROWS, buffers=None, counted=False):
+    """(seg_off [F*H+1], tile_off [F*H+1], seg_dest [M], tile_seg [tile bound]) int32 -- see csrc/lists.hip.
+    The tile tables cut the lists into tiles of `tile_rows` rows (the forward kernel's by default).
+    `buffers`: list_buffers() of the same plan, heads and tile_rows; `counted`: their cnt already holds the
+    counts, left there by gate_topk."""
+    lib = _lib.load()
+    S, H, K = sel.shape
+    dev = sel.device
+    bound = plan.hist_tile_bound(H, tile_rows)
+    cnt, seg_off, tile_off, seg_dest, tile_seg = buffers if buffers is not None else list_buffers(plan, H, dev, tile_rows)
     t = plan.tables
     _lib.check(lib.moba_build_lists(_ptr(sel), _ptr(t["chunk_tok"]), _ptr(t["chunk_fb"]), _ptr(t["chunk_local"]),
                                     _ptr(t["pair_off"]), _ptr(cnt), _ptr(seg_off), _ptr(tile_off), _ptr(seg_dest),
                                     _ptr(tile_seg), S, H, K, plan.N, plan.F, plan.P, plan.cmax, tile_rows, bound,
-                                    _stream(dev)), "moba_build_lists")
+                                    1 if counted else 0, _stream(dev)), "moba_build_lists")
     return seg_off, tile_off, seg_dest, tile_seg
 
 
@@ -265,12 +277,14 @@ def _forward(q, k, v, plan: MobaPlan, timer: Optional[StageTimer] = None, scale:
     if plan.fallback:
         sel = seg_off = tile_off = seg_dest = tile_seg = None
     else:
+        # the lists' counts are a by-product of the gate: the chunk mean clears the array, the gate adds to it
+        lists = list_buffers(plan, H, dev)
         with span("chunk_mean"):
-            kbar = chunk_mean(k, plan)
+            kbar = chunk_mean(k, plan, clear=lists[0])
         with span("gate_topk"):
-            sel = gate_topk(q, kbar, plan)
+            sel = gate_topk(q, kbar, plan, cnt=lists[0])
         with span("build_lists"):
-            seg_off, tile_off, seg_dest, tile_seg = build_lists(sel, plan)
+            seg_off, tile_off, seg_dest, tile_seg = build_lists(sel, plan, buffers=lists, counted=True)
     out = torch.empty((S, H, D), dtype=q.dtype, device=dev)
     lse = torch.empty((S, H), dtype=torch.float32, device=dev)
     # One allocation for the scratch of the attention stage: the per-slot partial outputs, their log-sum-exps,
@@ -340,12 +354,15 @@ class _MobaAttention(torch.autograd.Function):
         ctx.aux = (sel, seg_off, seg_dest)
         ctx.save_for_backward(q, k, v, out, lse)
         ctx.mark_non_differentiable(lse)
+        ctx.set_materialize_grads(False)  # no zero-filled gradient for lse on the way back
         return out, lse
 
     @staticmethod
     def backward(ctx, dout, _dlse):
         q, k, v, out, lse = ctx.saved_tensors
         sel, seg_off, seg_dest = ctx.aux
+        if dout is None:
+            return None, None, None, None, None, None
         dq, dk, dv = _backward(_aligned(dout.to(q.dtype)), q, k, v, out, lse, sel, seg_off, seg_dest, ctx.plan, ctx.scale)
         if q.dim() == 4:   # gradients in the layout of the batched inputs: views of the packed results
             b, _, l, d = q.shape

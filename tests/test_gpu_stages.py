@@ -107,15 +107,32 @@ def test_topk_from_injected_scores_bit_exact(K):
 
 
 # ------------------------------------------------------------------ gather lists
-@pytest.mark.parametrize("batch,seqlen,heads,B,topk", [(1, 2048, 2, 128, 3), (5, 3000, 3, 100, 4), (2, 9000, 1, 64, 12)])
-def test_gather_lists(batch, seqlen, heads, B, topk):
+# (the last case: more candidate chunks than one pass of the gate's LDS histogram holds)
+@pytest.mark.parametrize("counted", [False, True])
+@pytest.mark.parametrize("batch,seqlen,heads,B,topk", [(1, 2048, 2, 128, 3), (5, 3000, 3, 100, 4), (2, 9000, 1, 64, 12),
+                                                       (3, 5000, 5, 192, 2), (1, 140817, 1, 64, 2)])
+def test_gather_lists(batch, seqlen, heads, B, topk, counted):
+    """The lists from the counting pass of moba_build_lists, and from the counts the gate leaves as a by-product
+    in an array that the chunk mean cleared."""
     from moba_amd import moba_efficient as E
-    _note("lists", batch, seqlen, heads, B, topk)
+    _note("lists", batch, seqlen, heads, B, topk, counted)
     q, k, v, _, cu, _ = make_case(batch, seqlen, heads, seed=4)
     plan = _plan(cu, B, topk)
     kbar = O.chunk_mean(k, cu, B)
-    sel = E.gate_topk(q.cuda(), kbar.cuda(), plan)
-    seg_off, tile_off, seg_dest, tile_seg = (x.cpu().numpy() for x in E.build_lists(sel, plan))
+    if counted:
+        buffers = E.list_buffers(plan, heads, torch.device("cuda"))
+        for b in buffers:
+            b.fill_(0x5A5A5A5A)
+        assert torch.equal(E.chunk_mean(k.cuda(), plan, clear=buffers[0]).cpu(), kbar)
+        assert int(buffers[0].abs().max()) == 0 and int(buffers[1][0]) == 0x5A5A5A5A
+        sel = E.gate_topk(q.cuda(), kbar.cuda(), plan, cnt=buffers[0])
+        assert int(buffers[0].sum()) == plan.pairs_per_head * heads
+        assert torch.equal(sel, E.gate_topk(q.cuda(), kbar.cuda(), plan))
+        lists = E.build_lists(sel, plan, buffers=buffers, counted=True)
+    else:
+        sel = E.gate_topk(q.cuda(), kbar.cuda(), plan)
+        lists = E.build_lists(sel, plan)
+    seg_off, tile_off, seg_dest, tile_seg = (x.cpu().numpy() for x in lists)
     sel = sel.cpu()
     counts, offs, rows, slots = O.gather_lists(sel, plan.F)
     H, K1 = heads, plan.K + 1
