@@ -31,7 +31,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of moba_fwd_kernel from rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled by a copy
 # kernel of known size (profiles/moba_fwd_128k_hbm_traffic.txt); measured for the headline workload only
-FWD_KERNEL_TRAFFIC_BYTES = {"cfg4_L131072_h32_c4096_k12": 51.15e9}
+FWD_KERNEL_TRAFFIC_BYTES = {"cfg4_L131072_h32_c4096_k12": 51.3e9}
 
 WORKLOADS = {
     # name: (seq lens or None, heads, kv_heads, chunk, topk, normalise, backward)
