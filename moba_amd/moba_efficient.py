@@ -265,52 +265,108 @@ class _NoSpan:
         return False
 
 
+_NO_SPAN = _NoSpan()
+
+
+class _Geometry:
+    """What a forward call needs besides its tensors, worked out once per (plan, heads, head_dim, element size):
+    buffer sizes, the carving of the two scratch allocations, the key split and the tables' addresses."""
+
+    def __init__(self, plan: MobaPlan, lib, H: int, D: int, esize: int):
+        S, K = plan.S, plan.K
+        self.tptr = {name: _ptr(t) for name, t in plan.tables.items()}
+        self.null = ctypes.c_void_p(0)
+        self.bound = plan.hist_tile_bound(H, FWD_TILE_ROWS)
+        if plan.fallback:
+            self.split = 1
+        else:
+            self.split = int(lib.moba_fwd_key_split(S, H, K, plan.chunk_size, self.bound, plan.fwd_self_tiles))
+        # lists: cnt, seg_off, tile_off, seg_dest, tile_seg (int32, each start a multiple of 4 ints)
+        sizes = [plan.P * H + 1, plan.F * H + 1, plan.F * H + 1, max(plan.pairs_per_head * H, 1), self.bound]
+        self.list_sizes = sizes
+        starts = [0]
+        for n in sizes:
+            starts.append(starts[-1] + (n + 3) // 4 * 4)
+        self.list_starts = starts
+        # attention scratch: per-slot partial outputs, their log-sum-exps, the kernel's 8 tile counters, then
+        # the list of tiles its fixed-reference softmax hands to the kernel that tracks the running maximum
+        # (count first; the call zeroes the counters and the count)
+        rows = S * H * (K + 1) * self.split
+        self.rows = rows
+        self.part_o_bytes = rows * D * esize
+        self.scratch_ints = 8 + 1 + self.bound + plan.fwd_self_tiles * H
+        self.ws_bytes = self.part_o_bytes + rows * 4 + self.scratch_ints * 4
+        self.mean_ws = {}  # kv heads -> fp64 elements of the chunk mean's workspace
+        self.bwd = {}      # kv heads -> sizes of the backward's scratch
+
+
+def _geometry(plan: MobaPlan, lib, H: int, D: int, esize: int) -> _Geometry:
+    key = (H, D, esize)
+    g = plan.memo.get(key)
+    if g is None:
+        g = plan.memo[key] = _Geometry(plan, lib, H, D, esize)
+    return g
+
+
 def _forward(q, k, v, plan: MobaPlan, timer: Optional[StageTimer] = None, scale: float = 0.0):
-    """q, k, v: [tokens, heads, 128], or batched [batch, heads, tokens, 128] (read in place, see _dims)."""
+    """q, k, v: [tokens, heads, 128], or batched [batch, heads, tokens, 128] (read in place, see _dims), already
+    addressable (_in_place).  Returns (out, lse, sel, seg_off, tile_off, seg_dest, tile_seg).
+    The stages are those of chunk_mean(), gate_topk(), build_lists() above, called on precomputed sizes and
+    addresses: at small shapes a forward is bound by the host's time per call."""
     lib = _lib.load()
     S, H, D = _dims(q)
     Hkv = _dims(k)[1]
     dev = q.device
     K = plan.K
-    t = plan.tables
-    span = (lambda name: timer.span(name, dev)) if timer is not None else (lambda name: _NoSpan())
+    g = _geometry(plan, lib, H, D, q.element_size())
+    tp, null = g.tptr, g.null
+    span = (lambda name: timer.span(name, dev)) if timer is not None else (lambda name: _NO_SPAN)
+    stream, code, strides = _stream(dev), _dtype_code(q), _strides(q, k)
+    qp, kp, vp = _ptr(q), _ptr(k), _ptr(v)
     if plan.fallback:
         sel = seg_off = tile_off = seg_dest = tile_seg = None
+        selp = seg_offp = tile_offp = seg_destp = tile_segp = null
     else:
+        mean_ws = g.mean_ws.get(Hkv)
+        if mean_ws is None:
+            mean_ws = g.mean_ws[Hkv] = lib.moba_chunk_mean_workspace_bytes(Hkv, D, plan.F, plan.chunk_size) // 8
+        kbar = torch.empty((plan.F, Hkv, D), dtype=q.dtype, device=dev)
+        ws = torch.empty(mean_ws, dtype=torch.float64, device=dev)
+        sel = torch.empty((S, H, K), dtype=torch.int32, device=dev)
+        lists = torch.empty(g.list_starts[-1], dtype=torch.int32, device=dev)
+        base = lists.data_ptr()
+        cntp, seg_offp, tile_offp, seg_destp, tile_segp = (ctypes.c_void_p(base + 4 * a) for a in g.list_starts[:5])
+        seg_off, tile_off, seg_dest, tile_seg = (lists[a:a + n] for a, n in zip(g.list_starts[1:5], g.list_sizes[1:]))
+        selp, kbarp = _ptr(sel), _ptr(kbar)
         # the lists' counts are a by-product of the gate: the chunk mean clears the array, the gate adds to it
-        lists = list_buffers(plan, H, dev)
         with span("chunk_mean"):
-            kbar = chunk_mean(k, plan, clear=lists[0])
+            _lib.check(lib.moba_chunk_mean(kp, tp["fchunk_tok"], kbarp, _ptr(ws), S, Hkv, D, plan.F, plan.chunk_size,
+                                           strides, code, cntp, g.list_sizes[0], stream), "moba_chunk_mean")
         with span("gate_topk"):
-            sel = gate_topk(q, kbar, plan, cnt=lists[0])
+            _lib.check(lib.moba_gate_topk(qp, kbarp, tp["cu_seqlens"], tp["seq_fbase"], selp, null, tp["pair_off"],
+                                          cntp, S, H, Hkv, D, plan.nseq, plan.F, plan.chunk_size, K, strides, code,
+                                          stream), "moba_gate_topk")
         with span("build_lists"):
-            seg_off, tile_off, seg_dest, tile_seg = build_lists(sel, plan, buffers=lists, counted=True)
+            _lib.check(lib.moba_build_lists(selp, tp["chunk_tok"], tp["chunk_fb"], tp["chunk_local"], tp["pair_off"],
+                                            cntp, seg_offp, tile_offp, seg_destp, tile_segp, S, H, K, plan.N, plan.F,
+                                            plan.P, plan.cmax, FWD_TILE_ROWS, g.bound, 1, stream), "moba_build_lists")
     out = torch.empty((S, H, D), dtype=q.dtype, device=dev)
     lse = torch.empty((S, H), dtype=torch.float32, device=dev)
-    # One allocation for the scratch of the attention stage: the per-slot partial outputs, their log-sum-exps,
-    # the forward kernel's tile counters, then the list of tiles its fixed-reference softmax hands to the kernel
-    # that tracks the running maximum (count first; the call zeroes the counters and the count).
-    bound = plan.hist_tile_bound(H, FWD_TILE_ROWS)
-    # small problems: the keys of every history tile in `split` parts, each with slots of its own
-    split = 1 if plan.fallback else int(lib.moba_fwd_key_split(S, H, K, plan.chunk_size, bound, plan.fwd_self_tiles))
-    rows = S * H * (K + 1) * split
-    n_ints = 8 + 1 + bound + plan.fwd_self_tiles * H
-    ws = torch.empty(rows * D * q.element_size() + rows * 4 + n_ints * 4, dtype=torch.uint8, device=dev)
-    part_o = ws[:rows * D * q.element_size()].view(q.dtype).view(rows, D)
-    part_lse = ws[rows * D * q.element_size():][:rows * 4].view(torch.float32)
-    scratch = ws[rows * D * q.element_size() + rows * 4:].view(torch.int32)
-    queues, redo = scratch[:8], (scratch[8:] if FIXED_REFERENCE else None)
+    ws2 = torch.empty(g.ws_bytes, dtype=torch.uint8, device=dev)
+    base = ws2.data_ptr()
+    part_op = ctypes.c_void_p(base)
+    part_lsep = ctypes.c_void_p(base + g.part_o_bytes)
+    queuesp = ctypes.c_void_p(base + g.part_o_bytes + g.rows * 4)
+    redop = ctypes.c_void_p(base + g.part_o_bytes + g.rows * 4 + 32) if FIXED_REFERENCE else null
     with span("fwd_partials"):
-        _lib.check(lib.moba_fwd_partials(_ptr(q), _ptr(k), _ptr(v), _ptr(part_o), _ptr(part_lse), _ptr(seg_off),
-                                         _ptr(tile_off), _ptr(seg_dest), _ptr(t.get("fchunk_tok")),
-                                         _ptr(t["chunk_tok"]), _ptr(t["fwd_self_tile_prefix"]), _ptr(tile_seg),
-                                         _ptr(t["fwd_self_tile_chunk"]), S, H, Hkv, D, K, plan.F, plan.N,
-                                         plan.chunk_size, bound, plan.fwd_self_tiles, split, _strides(q, k),
-                                         _ptr(queues), _ptr(redo), scale, _dtype_code(q), _stream(dev)),
-                   "moba_fwd_partials")
+        _lib.check(lib.moba_fwd_partials(qp, kp, vp, part_op, part_lsep, seg_offp, tile_offp, seg_destp,
+                                         tp.get("fchunk_tok", null), tp["chunk_tok"], tp["fwd_self_tile_prefix"],
+                                         tile_segp, tp["fwd_self_tile_chunk"], S, H, Hkv, D, K, plan.F, plan.N,
+                                         plan.chunk_size, g.bound, plan.fwd_self_tiles, g.split, strides, queuesp,
+                                         redop, scale, code, stream), "moba_fwd_partials")
     with span("fwd_merge"):
-        _lib.check(lib.moba_fwd_merge(_ptr(part_o), _ptr(part_lse), _ptr(sel), _ptr(out), _ptr(lse), S, H, D, K,
-                                      split, _dtype_code(q), _stream(dev)), "moba_fwd_merge")
+        _lib.check(lib.moba_fwd_merge(part_op, part_lsep, selp, _ptr(out), _ptr(lse), S, H, D, K, g.split, code,
+                                      stream), "moba_fwd_merge")
     return out, lse, sel, seg_off, tile_off, seg_dest, tile_seg
 
 
@@ -320,26 +376,41 @@ def _backward(dout, q, k, v, out, lse, sel, seg_off, seg_dest, plan: MobaPlan, s
     Hkv = _dims(k)[1]
     dev = q.device
     K = plan.K
-    t = plan.tables
-    # the backward kernels cut the gather lists into tiles of their own height
-    tile_off, tile_seg = (None, None) if plan.fallback else tile_tables(seg_off, plan, H, TILE_ROWS)
+    g = _geometry(plan, lib, H, D, q.element_size())
+    tp, null = g.tptr, g.null
+    stream = _stream(dev)
+    # One allocation for the call's scratch, every part a multiple of 16 bytes: the per-slot partial dQ, delta and
+    # the log2 lse, the 16 tile counters of the two kernels (zeroed by the call), the backward kernels' own tile
+    # tables (they cut the gather lists into tiles of their own height) and, for small problems, the fp32 sums of
+    # the parts the dK/dV kernel cuts its key tiles into (0 bytes otherwise)
+    b = g.bwd.get(Hkv)
+    if b is None:
+        bound = plan.hist_tile_bound(H, TILE_ROWS)
+        kv_bytes = int(lib.moba_bwd_dkv_scratch_bytes(S, Hkv, plan.self_tiles))
+        sizes = [S * H * (K + 1) * D * q.element_size(), 2 * S * H * 4, 64,
+                 0 if plan.fallback else (plan.F * H + 1) * 4, 0 if plan.fallback else bound * 4, kv_bytes]
+        starts = [0]
+        for n in sizes:
+            starts.append(starts[-1] + (n + 15) // 16 * 16)
+        b = g.bwd[Hkv] = (bound, kv_bytes, starts)
+    bound, kv_bytes, starts = b
+    ws = torch.empty(starts[-1], dtype=torch.uint8, device=dev)
+    base = ws.data_ptr()
+    part_dqp, deltap, queuesp, tile_offp, tile_segp, kvp = (ctypes.c_void_p(base + a) for a in starts[:6])
+    if plan.fallback:
+        tile_offp = tile_segp = null
+    else:
+        _lib.check(lib.moba_tile_tables(_ptr(seg_off), tile_offp, tile_segp, H, plan.F, TILE_ROWS, bound, stream),
+                   "moba_tile_tables")
     dq = torch.empty((S, H, D), dtype=q.dtype, device=dev)  # packed, whatever the strides of q, k, v
     dk = torch.empty((S, Hkv, D), dtype=k.dtype, device=dev)
     dv = torch.empty((S, Hkv, D), dtype=v.dtype, device=dev)
-    delta = torch.empty((2, S, H), dtype=torch.float32, device=dev)
-    part_dq = torch.empty((S * H * (K + 1), D), dtype=q.dtype, device=dev)
-    queues = torch.empty(16, dtype=torch.int32, device=dev)  # tile counters of the two backward kernels (zeroed there)
-    # small problems: the fp32 sums of the parts the dK/dV kernel cuts its key tiles into (0 bytes otherwise)
-    kv_bytes = int(lib.moba_bwd_dkv_scratch_bytes(S, Hkv, plan.self_tiles))
-    kv_scratch = torch.empty(kv_bytes, dtype=torch.uint8, device=dev) if kv_bytes else None
     _lib.check(lib.moba_bwd(_ptr(dout), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(sel), _ptr(seg_off),
-                            _ptr(tile_off), _ptr(seg_dest), _ptr(t.get("fchunk_tok")), _ptr(t["chunk_tok"]),
-                            _ptr(t["self_tile_prefix"]), _ptr(tile_seg), _ptr(t["self_tile_chunk"]),
-                            _ptr(t.get("chunk_fid")), _ptr(delta), _ptr(part_dq), _ptr(dq), _ptr(dk), _ptr(dv),
-                            S, H, Hkv, D, K, plan.F, plan.N, plan.chunk_size, plan.hist_tile_bound(H),
-                            plan.self_tiles, _strides(q, k), _ptr(queues), _ptr(kv_scratch), kv_bytes, scale,
-                            _dtype_code(q), _stream(dev)),
-               "moba_bwd")
+                            tile_offp, _ptr(seg_dest), tp.get("fchunk_tok", null), tp["chunk_tok"],
+                            tp["self_tile_prefix"], tile_segp, tp["self_tile_chunk"], tp.get("chunk_fid", null),
+                            deltap, part_dqp, _ptr(dq), _ptr(dk), _ptr(dv), S, H, Hkv, D, K, plan.F, plan.N,
+                            plan.chunk_size, plan.hist_tile_bound(H), plan.self_tiles, _strides(q, k), queuesp,
+                            kvp if kv_bytes else null, kv_bytes, scale, _dtype_code(q), stream), "moba_bwd")
     return dq, dk, dv
 
 

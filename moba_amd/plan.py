@@ -41,6 +41,7 @@ class MobaPlan:
     flops_per_head: float
     tables: Dict[str, torch.Tensor] = field(default_factory=dict)
     host: Dict[str, np.ndarray] = field(default_factory=dict)
+    memo: Dict[tuple, object] = field(default_factory=dict)  # what callers derive once per plan (sizes, pointers)
 
     def hist_tile_bound(self, H: int, rows: int = TILE_ROWS) -> int:
         """Upper bound on the number of history tiles of `rows` rows (every segment may end in a partial tile)."""
