@@ -55,7 +55,7 @@ extern "C" {
 
 enum { MOBA_DTYPE_BF16 = 0, MOBA_DTYPE_F16 = 1 };
 
-#define MOBA_ABI_VERSION 109 /* the signatures below; moba_version() returns the number the library was built with */
+#define MOBA_ABI_VERSION 110 /* the signatures below; moba_version() returns the number the library was built with */
 int moba_version(void);
 const char* moba_strerror(int code);
 
@@ -228,7 +228,12 @@ int moba_fwd(const void* q, const void* k, const void* v, void* part_o, float* p
  *   tile_off, tile_seg, self_tile_prefix, self_tile_chunk, hist_bound, self_tiles: as in moba_fwd_partials, but for
  *   tiles of moba_bwd_tile_rows() rows (moba_tile_tables makes the first two from seg_off)
  *   chunk_fid [N] int32: filtered id of each chunk, -1 for the last chunk of a sequence
- *   delta [2,S,H] fp32 scratch (rowsum(dO*O), then the LSE in the log2 domain); part_dq [S*H*(K+1), D] elem scratch (the per-slot dQ, rounded as the per-chunk dQ that flash-attn returns to the reference is)
+ *   delta [2,S,H] fp32 scratch (rowsum(dO*O), then the LSE in the log2 domain); part_dq [dq_key_split*S*H*(K+1), D]
+ *   elem scratch (the per-slot dQ, rounded as the per-chunk dQ that flash-attn returns to the reference is)
+ *   dq_key_split: 1, or for small problems the power of two (up to 8) that moba_bwd_dq_key_split() names: the dQ
+ *              kernel then cuts the keys of every history tile into that many parts, each a tile with slot rows of
+ *              its own (as key_split does in the forward), and takes its self tiles first.  B must be a multiple
+ *              of 64 * dq_key_split (MOBA_ERR_ARG otherwise).
  *   dq, dk, dv: out; dk and dv of a key/value head sum over its query heads
  *   queues [16] int32 scratch: tile counters of the dQ and dK/dV kernels (as in moba_fwd_partials)
  *   dkv_scratch: moba_bwd_dkv_scratch_bytes(S, Hkv, self_tiles) bytes, 16-byte aligned, or null.  With few key tiles
@@ -237,13 +242,14 @@ int moba_fwd(const void* q, const void* k, const void* v, void* part_o, float* p
  *              without the scratch, or when the query returns 0, every tile is one piece.
  *   softmax_scale: as in the forward call */
 size_t moba_bwd_dkv_scratch_bytes(int64_t S, int Hkv, int64_t self_tiles);
+int moba_bwd_dq_key_split(int64_t S, int H, int K, int B, int64_t hist_bound, int64_t self_tiles);
 int moba_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out, const float* lse,
              const int32_t* sel, const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest,
              const int32_t* fchunk_tok, const int32_t* chunk_tok, const int32_t* self_tile_prefix,
              const int32_t* tile_seg, const int32_t* self_tile_chunk, const int32_t* chunk_fid, float* delta,
              void* part_dq, void* dq, void* dk, void* dv, int64_t S, int H, int Hkv, int D, int K, int F, int N, int B,
-             int64_t hist_bound, int64_t self_tiles, const int64_t* strides, int32_t* queues, void* dkv_scratch,
-             int64_t dkv_scratch_bytes, float softmax_scale, int dtype, void* stream);
+             int64_t hist_bound, int64_t self_tiles, int dq_key_split, const int64_t* strides, int32_t* queues,
+             void* dkv_scratch, int64_t dkv_scratch_bytes, float softmax_scale, int dtype, void* stream);
 
 /* Decode: one query token per sequence against the key/value cache.  Replaces the
  * flash_attn_func call of the adapter's decode branch, moba/wrapper.py:76-82 (full attention

@@ -45,8 +45,9 @@ _SIGNATURES = {
     "moba_fwd": (c_int, [c_void_p] * 16 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_int64,
                                           c_int, c_strides, c_void_p, c_void_p, c_float, c_int, c_void_p]),
     "moba_bwd_dkv_scratch_bytes": (ctypes.c_size_t, [c_int64, c_int, c_int64]),
+    "moba_bwd_dq_key_split": (c_int, [c_int64, c_int, c_int, c_int, c_int64, c_int64]),
     "moba_bwd": (c_int, [c_void_p] * 21 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_int64,
-                                          c_strides, c_void_p, c_void_p, c_int64, c_float, c_int, c_void_p]),
+                                          c_int, c_strides, c_void_p, c_void_p, c_int64, c_float, c_int, c_void_p]),
     "moba_decode_splits": (c_int, [c_int, c_int, c_int]),
     "moba_decode": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_int64] * 4 + [c_float, c_int, c_void_p]),
 }
@@ -70,7 +71,7 @@ class SizesStruct(ctypes.Structure):
     _fields_ = [(n, c_int64) for n in ("kbar_elems", "chunk_mean_workspace_bytes", "sel_ints", "cnt_ints", "seg_off_ints",
                                        "seg_dest_ints", "fwd_hist_bound", "bwd_hist_bound", "part_rows", "redo_ints",
                                        "lse_floats", "delta_floats")]
-ABI_VERSION = 109  # MOBA_ABI_VERSION of include/moba_hip.h, the signatures above
+ABI_VERSION = 110  # MOBA_ABI_VERSION of include/moba_hip.h, the signatures above
 DTYPE_BF16, DTYPE_F16 = 0, 1
 
 

@@ -122,26 +122,56 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams<E> p) {
   // The draw for the next tile is in flight while the current one is computed.
   int queue = blockIdx.x & 7, empty_queues = 0;
   int drawn_next = 0;  // thread 0: the counter value drawn for the next tile
-  if (tid == 0) drawn_next = __hip_atomic_fetch_add(p.queues + queue, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  // (With few tiles per workgroup a tile drawn ahead is a tile that waits for its holder while other workgroups
+  // run out of work: the draw is made when the tile is due then, two microseconds that nothing hides.)
+  const bool draw_ahead = !p.t.self_first;
+  if (tid == 0 && draw_ahead)
+    drawn_next = __hip_atomic_fetch_add(p.queues + queue, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   while (true) {
   __syncthreads();  // the previous tile is done with LDS, and every wave has read the previous draw
-  if (tid == 0) *reinterpret_cast<int*>(smem + kDqIdSlot) = drawn_next;
+  if (tid == 0) {
+    if (!draw_ahead)
+      drawn_next = __hip_atomic_fetch_add(p.queues + queue, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    *reinterpret_cast<int*>(smem + kDqIdSlot) = drawn_next;
+  }
   __syncthreads();
   const int drawn = __builtin_amdgcn_readfirstlane(*reinterpret_cast<const int*>(smem + kDqIdSlot));
   const int64_t id = ((int64_t)(drawn / kXcdBlock) * 8 + queue) * kXcdBlock + (drawn % kXcdBlock);
-  const bool past_end = id >= (int64_t)p.t.hist_bound + p.t.self_total;
+  const int ks = p.t.key_split_log2;
+  const bool past_end = id >= ((int64_t)p.t.hist_bound << ks) + p.t.self_total;
   if (past_end) {
     queue = (queue + 1) & 7;
     if (++empty_queues == 8) break;
   } else {
     empty_queues = 0;
   }
-  if (tid == 0) drawn_next = __hip_atomic_fetch_add(p.queues + queue, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (tid == 0 && draw_ahead)
+    drawn_next = __hip_atomic_fetch_add(p.queues + queue, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   if (past_end) continue;
 
   Tile t;
   const int r = wave * 32 + n;
-  if (!decode_tile(p.t, (int)id, wave, r, t)) continue;  // an unused id below hist_bound
+  // With few tiles per workgroup (self_first) the self tiles take the first ids -- the longest of them are as
+  // long as a history tile, and drawn last they would run alone at the end -- and the keys of a history tile
+  // are cut into 1 << ks parts that are tiles of their own, each with slot rows of its own for its partial dQ
+  // (part g of a slot row lies g * part_stride rows behind part 0; bwd_dq_reduce_kernel adds them up).
+  int logical = (int)id, key_part = 0;
+  if (p.t.self_first) {
+    if (logical < p.t.self_total) {
+      logical += p.t.hist_bound;
+    } else {
+      logical -= p.t.self_total;
+      key_part = logical & ((1 << ks) - 1);
+      logical >>= ks;
+    }
+  }
+  if (!decode_tile_head(p.t, logical, t)) continue;  // an unused id below hist_bound
+  if (t.base >= 0) {
+    t.nkeys >>= ks;
+    t.kv_tok0 += key_part * t.nkeys;
+  }
+  decode_tile_rows(p.t, wave, r, t);
+  t.dest += key_part * p.t.part_stride;
   const int h = t.h, nkeys = t.nkeys, kv_tok0 = t.kv_tok0, limit = t.limit;
   const bool row_valid = r < t.row_count;
 
@@ -381,7 +411,8 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams<E> p) {
 template <class E>
 __global__ __launch_bounds__(256) void bwd_dq_reduce_kernel(const typename E::elem* __restrict__ part_dq,
                                                             const int* __restrict__ sel,
-                                                            typename E::elem* __restrict__ dq, int64_t rows, int K1) {
+                                                            typename E::elem* __restrict__ dq, int64_t rows, int K1,
+                                                            int parts) {
   MOBA_ELEM_TYPES(E)
   const int64_t row_raw = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
   const bool row_ok = row_raw < rows;
@@ -394,18 +425,25 @@ __global__ __launch_bounds__(256) void bwd_dq_reduce_kernel(const typename E::el
   for (int e = 0; e < 8; ++e) acc[e] = 0.f;
   const elem* src = part_dq + row * K1 * kHeadDim + c8 * 8;
   // lane c8 fetches the presence of slot j0 + c8; absent slots are redirected to slot 0 and
-  // multiplied by 0, so the loads of eight slots are unconditional and in flight together
-  for (int j0 = 0; j0 < K1; j0 += 16) {
-    const int j = j0 + c8;
-    const float present = (j < K1 && (j == 0 || ps[j - 1] >= 0)) ? 1.f : 0.f;
-    const int nslot = min(16, K1 - j0);
+  // multiplied by 0, so the loads of eight slots are unconditional and in flight together.
+  // With parts, slot v of the parts * K1 is slot v % K1 of part v / K1, rows * K1 slot rows behind the part
+  // before (an int: the buffer holds fewer than 2^31 slot rows); the self slot exists in part 0 only.
+  const int nvirt = parts * K1;
+  const int part_rows = (int)(rows * K1);
+  for (int j0 = 0; j0 < nvirt; j0 += 16) {
+    const int v = j0 + c8;
+    const int part = parts == 1 ? 0 : v / K1, j = v - part * K1;
+    const bool ok = v < nvirt && (j == 0 ? part == 0 : ps[j - 1] >= 0);
+    const float present = ok ? 1.f : 0.f;
+    const int at = ok ? part * part_rows + j : 0;
+    const int nslot = min(16, nvirt - j0);
     for (int u0 = 0; u0 < nslot; u0 += 8) {
       elem8 a[8];
       float w[8];
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
         w[u] = __shfl(present, u0 + u, 16);
-        const int jj = w[u] > 0.f ? j0 + u0 + u : 0;
+        const int jj = parts == 1 ? (w[u] > 0.f ? j0 + u0 + u : 0) : __shfl(at, u0 + u, 16);
         if (u0 + u < nslot)  // uniform: no loads for slots that do not exist
           a[u] = __builtin_nontemporal_load(reinterpret_cast<const elem8*>(src + (int64_t)jj * kHeadDim));
       }
@@ -877,7 +915,7 @@ static int launch_bwd(const void* dout, const void* q, const void* k, const void
                      (const elem*)out, lse, delta, delta + S * H, rows, queues);
   hipLaunchKernelGGL(bwd_dq_kernel<E>, dim3((unsigned)grid_q), dim3(256), kBwdDqLds, st, p);
   hipLaunchKernelGGL(bwd_dq_reduce_kernel<E>, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st,
-                     (const elem*)part_dq, sel, (elem*)dq, rows, K + 1);
+                     (const elem*)part_dq, sel, (elem*)dq, rows, K + 1, 1 << t.key_split_log2);
   if (batched) hipLaunchKernelGGL((bwd_dkv_kernel<E, true>), dim3((unsigned)grid_kv), dim3(256), kBwdDkvLds, st, p);
   else hipLaunchKernelGGL((bwd_dkv_kernel<E, false>), dim3((unsigned)grid_kv), dim3(256), kBwdDkvLds, st, p);
   if (dkv_split > 1)
@@ -905,14 +943,29 @@ extern "C" size_t moba_bwd_dkv_scratch_bytes(int64_t S, int Hkv, int64_t self_ti
   return split > 1 ? (size_t)tiles * split * (2 * TM * kHeadDim) * sizeof(float) : 0;
 }
 
+// Parts per history tile of the dQ kernel (a power of two).  With fewer tiles than workgroup slots to fill a few
+// times over, a tile of 128 rows x B keys is too coarse a unit: the kernel's time is then two such tiles in a row
+// on some workgroups while others idle.  Every part keeps at least 512 keys; part_dq grows by the same factor.
+extern "C" int moba_bwd_dq_key_split(int64_t S, int H, int K, int B, int64_t hist_bound, int64_t self_tiles) {
+  const int cus = resident_compute_units();
+  if (cus <= 0 || S <= 0 || H <= 0 || K <= 0 || B <= 0 || hist_bound <= 0 || self_tiles <= 0) return 1;
+  const int64_t slots = 2 * (((int64_t)cus + 7) / 8 * 8), own = self_tiles * H;
+  int split = 1;
+  while (split < 8 && B % (64 * 2 * split) == 0 && B / (2 * split) >= 512 &&
+         own + hist_bound * 2 * split <= 3 * slots && S * H * (K + 1) * 2 * split < 0x7fffffffLL)
+    split *= 2;
+  return split;
+}
+
 extern "C" int moba_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out,
                         const float* lse, const int32_t* sel, const int32_t* seg_off, const int32_t* tile_off,
                         const int32_t* seg_dest, const int32_t* fchunk_tok, const int32_t* chunk_tok,
                         const int32_t* self_tile_prefix, const int32_t* tile_seg, const int32_t* self_tile_chunk,
                         const int32_t* chunk_fid, float* delta, void* part_dq,
                         void* dq, void* dk, void* dv, int64_t S, int H, int Hkv, int D, int K, int F, int N, int B,
-                        int64_t hist_bound, int64_t self_tiles, const int64_t* strides, int32_t* queues,
-                        void* dkv_scratch, int64_t dkv_scratch_bytes, float softmax_scale, int dtype, void* stream) {
+                        int64_t hist_bound, int64_t self_tiles, int dq_key_split, const int64_t* strides,
+                        int32_t* queues, void* dkv_scratch, int64_t dkv_scratch_bytes, float softmax_scale, int dtype,
+                        void* stream) {
   if (!dout || !q || !k || !v || !out || !lse || !chunk_tok || !self_tile_prefix || !self_tile_chunk || !delta ||
       !part_dq || !dq || !dk || !dv || !queues)
     return MOBA_ERR_ARG;
@@ -924,8 +977,10 @@ extern "C" int moba_bwd(const void* dout, const void* q, const void* k, const vo
   const void* ptrs[] = {dout, q, k, v, out, part_dq, dq, dk, dv};
   for (const void* x : ptrs)
     if ((uintptr_t)x & 15) return MOBA_ERR_ARG;
-  if ((int64_t)S * H * (K + 1) >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
-  const int64_t total_q = (K > 0 ? hist_bound : 0) + self_tiles * H;
+  if (dq_key_split < 1 || dq_key_split > 8 || (dq_key_split & (dq_key_split - 1))) return MOBA_ERR_ARG;
+  if (dq_key_split > 1 && (K == 0 || B % (64 * dq_key_split) != 0)) return MOBA_ERR_ARG;
+  if ((int64_t)S * H * (K + 1) * dq_key_split >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
+  const int64_t total_q = (K > 0 ? hist_bound * dq_key_split : 0) + self_tiles * H;
   // the dK/dV kernel: one workgroup per CU, resident, drawing its tiles from the queues
   const int cus = resident_compute_units();
   if (cus <= 0) return MOBA_ERR_LAUNCH;
@@ -941,6 +996,10 @@ extern "C" int moba_bwd(const void* dout, const void* q, const void* k, const vo
   t.hist_bound = (K > 0) ? (int)hist_bound : 0;
   t.self_total = (int)(self_tiles * H);
   if (!set_layout(t, strides)) return MOBA_ERR_ARG;
+  // the dQ kernel's order of tiles and its parts per history tile (the dK/dV kernel has parts of its own)
+  t.self_first = dq_key_split > 1 || total_q < 8 * grid_q;
+  while ((1 << t.key_split_log2) < dq_key_split) ++t.key_split_log2;
+  t.part_stride = (int)(S * H * (K + 1));
   // the key tiles are cut into parts only if the caller brought the scratch for their sums
   const int64_t kv_tiles = self_tiles * Hkv;
   int dkv_split = dkv_split_for(S, kv_tiles);

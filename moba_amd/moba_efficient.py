@@ -387,13 +387,15 @@ def _backward(dout, q, k, v, out, lse, sel, seg_off, seg_dest, plan: MobaPlan, s
     if b is None:
         bound = plan.hist_tile_bound(H, TILE_ROWS)
         kv_bytes = int(lib.moba_bwd_dkv_scratch_bytes(S, Hkv, plan.self_tiles))
-        sizes = [S * H * (K + 1) * D * q.element_size(), 2 * S * H * 4, 64,
+        # small problems: the keys of every history tile of the dQ kernel in `split` parts with slots of their own
+        split = 1 if plan.fallback else int(lib.moba_bwd_dq_key_split(S, H, K, plan.chunk_size, bound, plan.self_tiles))
+        sizes = [split * S * H * (K + 1) * D * q.element_size(), 2 * S * H * 4, 64,
                  0 if plan.fallback else (plan.F * H + 1) * 4, 0 if plan.fallback else bound * 4, kv_bytes]
         starts = [0]
         for n in sizes:
             starts.append(starts[-1] + (n + 15) // 16 * 16)
-        b = g.bwd[Hkv] = (bound, kv_bytes, starts)
-    bound, kv_bytes, starts = b
+        b = g.bwd[Hkv] = (bound, kv_bytes, starts, split)
+    bound, kv_bytes, starts, split = b
     ws = torch.empty(starts[-1], dtype=torch.uint8, device=dev)
     base = ws.data_ptr()
     part_dqp, deltap, queuesp, tile_offp, tile_segp, kvp = (ctypes.c_void_p(base + a) for a in starts[:6])
@@ -409,7 +411,7 @@ def _backward(dout, q, k, v, out, lse, sel, seg_off, seg_dest, plan: MobaPlan, s
                             tile_offp, _ptr(seg_dest), tp.get("fchunk_tok", null), tp["chunk_tok"],
                             tp["self_tile_prefix"], tile_segp, tp["self_tile_chunk"], tp.get("chunk_fid", null),
                             deltap, part_dqp, _ptr(dq), _ptr(dk), _ptr(dv), S, H, Hkv, D, K, plan.F, plan.N,
-                            plan.chunk_size, plan.hist_tile_bound(H), plan.self_tiles, _strides(q, k), queuesp,
+                            plan.chunk_size, bound, plan.self_tiles, split, _strides(q, k), queuesp,
                             kvp if kv_bytes else null, kv_bytes, scale, _dtype_code(q), stream), "moba_bwd")
     return dq, dk, dv
 

@@ -307,6 +307,59 @@ def test_backward_is_deterministic():
         assert torch.equal(a, b)
 
 
+def test_history_tiles_of_dq_cut_into_parts():
+    """With few tiles per workgroup the dQ kernel cuts the keys of every history tile into parts that are tiles of
+    their own, each leaving its partial dQ in slot rows of its own: 1, 2 and 4 parts give the same out, dk and dv
+    bit for bit and a dq that differs by the rounding of the parts' partial sums only; dq lies within the tolerance
+    of the oracle for each.  Three sequences with partial last chunks, grouped-query heads."""
+    from moba_amd import _lib, moba_attn_varlen_gqa
+    from moba_amd import moba_efficient as E
+    from moba_amd.plan import make_plan
+    heads, kv_heads, B, topk = 2, 1, 1024, 3
+    q, _, _, do, cu, mx = make_case(3, 16384, heads, seed=23)
+    _, k, v, _, _, _ = make_case(3, 16384, kv_heads, seed=24)
+    cu_t = torch.tensor(cu, dtype=torch.int32, device="cuda")
+    lib = _lib.load()
+    plan = make_plan(cu_t, B, topk)
+    proposed = lib.moba_bwd_dq_key_split(16384, heads, plan.K, B, plan.hist_tile_bound(heads), plan.self_tiles)
+    assert proposed in (1, 2, 4, 8) and (proposed == 2 or "MOBA_RESIDENT_CUS" in os.environ)
+
+    def run(split):
+        real = lib.moba_bwd_dq_key_split
+        plan.memo.clear()   # (the operator keeps the split with the plan)
+        try:
+            lib.moba_bwd_dq_key_split = lambda *a: split
+            qg, kg, vg = (x.cuda().requires_grad_(True) for x in (q, k, v))
+            out = moba_attn_varlen_gqa(qg, kg, vg, cu_t, mx, B, topk)
+            out.backward(do.cuda())
+        finally:
+            lib.moba_bwd_dq_key_split = real
+            plan.memo.clear()
+        return out.detach(), qg.grad, kg.grad, vg.grad
+
+    whole, two, four = run(1), run(2), run(4)
+    for cut in (two, four):
+        assert torch.equal(cut[0], whole[0]) and torch.equal(cut[2], whole[2]) and torch.equal(cut[3], whole[3])
+        e = (cut[1].float() - whole[1].float()).abs()
+        assert 0 < e.max() <= 2.0 ** -6 * whole[1].float().abs().max(), e.max().item()
+    again = run(2)
+    assert torch.equal(again[1], two[1])
+    with pytest.raises(RuntimeError, match="moba_bwd"):
+        run(3)           # not a power of two
+    with pytest.raises(RuntimeError, match="moba_bwd"):
+        run(32)          # B is not a multiple of 64 * 32 (and 8 is the most)
+    sel = E.gate_topk(q.cuda(), E.chunk_mean(k.cuda(), plan), plan).cpu()
+    qc = q.clone().requires_grad_(True)
+    rep = heads // kv_heads
+    ref = O.moba_attn_varlen_oracle(qc, torch.repeat_interleave(k, rep, dim=1), torch.repeat_interleave(v, rep, dim=1),
+                                    cu, mx, B, topk, sel=sel)
+    ref.backward(do.float())
+    for got in (whole, two, four):
+        e = (got[1].cpu().float() - qc.grad.float()).abs()
+        scale = qc.grad.abs().max().clamp_min(1.0)
+        assert e.max() < MAX_ABS * scale and e.mean() < MEAN_ABS, (e.max().item(), e.mean().item())
+
+
 def test_key_tiles_cut_into_parts():
     """With few key tiles (here 16384 tokens x 1 key/value head = 128 tiles on 256 compute units) the dK/dV kernel
     cuts every tile into parts that leave fp32 sums for a reduction kernel: grouped-query heads, three sequences
