@@ -59,6 +59,9 @@ struct BwdParams {
   // which bwd_dkv_reduce_kernel adds up in a fixed order.  dkv_split = 1: whole tiles, dk and dv written directly.
   float* part_dkv;
   int dkv_split;
+  // 3: eight queues, one per XCD (tiles that share rows or keys run behind one L2); 0: one queue for all, for a
+  // problem of few tiles per workgroup, whose ids come longest tile first: whoever is free takes the longest left
+  int queues_log2;
 };
 
 // which 128-key tile of which key/value head: the forward's self-tile enumeration over Hkv heads
@@ -120,7 +123,8 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams<E> p) {
   // consecutive ids (tiles that share a K/V chunk behind one L2), and a workgroup whose queue is empty
   // goes on with the next XCD's: the XCDs differ in speed by a few percent and finish together this way.
   // The draw for the next tile is in flight while the current one is computed.
-  int queue = blockIdx.x & 7, empty_queues = 0;
+  const int ql = p.queues_log2, qmask = (1 << ql) - 1;  // eight queues, or one for a problem of few tiles
+  int queue = blockIdx.x & qmask, empty_queues = 0;
   int drawn_next = 0;  // thread 0: the counter value drawn for the next tile
   // (With few tiles per workgroup a tile drawn ahead is a tile that waits for its holder while other workgroups
   // run out of work: the draw is made when the tile is due then, two microseconds that nothing hides.)
@@ -136,12 +140,12 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams<E> p) {
   }
   __syncthreads();
   const int drawn = __builtin_amdgcn_readfirstlane(*reinterpret_cast<const int*>(smem + kDqIdSlot));
-  const int64_t id = ((int64_t)(drawn / kXcdBlock) * 8 + queue) * kXcdBlock + (drawn % kXcdBlock);
+  const int64_t id = (((int64_t)(drawn / kXcdBlock) << ql) + queue) * kXcdBlock + (drawn % kXcdBlock);
   const int ks = p.t.key_split_log2;
   const bool past_end = id >= ((int64_t)p.t.hist_bound << ks) + p.t.self_total;
   if (past_end) {
-    queue = (queue + 1) & 7;
-    if (++empty_queues == 8) break;
+    queue = (queue + 1) & qmask;
+    if (++empty_queues > qmask) break;
   } else {
     empty_queues = 0;
   }
@@ -478,7 +482,8 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
   // (chunk, head) that gather the same Q and dO rows, run side by side behind one L2 -- and a workgroup whose
   // queue is empty goes on with the next XCD's, so that the XCDs, which differ in speed by a few percent,
   // finish together.  A tile runs for about a millisecond: the draw (one atomic, two barriers) is free.
-  int queue = blockIdx.x & 7, empty_queues = 0;
+  const int ql = p.queues_log2, qmask = (1 << ql) - 1;
+  int queue = blockIdx.x & qmask, empty_queues = 0;
   while (true) {
   __syncthreads();  // every wave is done with the LDS of the previous tile and has read the previous draw
   if (tid == 0)
@@ -486,11 +491,11 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
         __hip_atomic_fetch_add(p.queues + 8 + queue, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   __syncthreads();
   const int drawn = __builtin_amdgcn_readfirstlane(*reinterpret_cast<const int*>(smem + kDkvIdSlot));
-  const int64_t id = ((int64_t)(drawn / kXcdBlock) * 8 + queue) * kXcdBlock + (drawn % kXcdBlock);
+  const int64_t id = (((int64_t)(drawn / kXcdBlock) << ql) + queue) * kXcdBlock + (drawn % kXcdBlock);
   const int split = p.dkv_split;
   if (id >= (int64_t)(p.t.self_total / rep) * split) {
-    queue = (queue + 1) & 7;
-    if (++empty_queues == 8) break;
+    queue = (queue + 1) & qmask;
+    if (++empty_queues > qmask) break;
     continue;
   }
   empty_queues = 0;
@@ -891,6 +896,7 @@ static int launch_bwd(const void* dout, const void* q, const void* k, const void
   p.queues = queues;
   p.part_dkv = part_dkv;
   p.dkv_split = dkv_split;
+  p.queues_log2 = t.self_first ? 0 : 3;
   p.t = t;
   p.scale = softmax_scale > 0.f ? softmax_scale : (float)(1.0 / sqrt((double)D));
   p.scale_log2 = softmax_scale > 0.f ? (float)(1.4426950408889634 * (double)softmax_scale)
