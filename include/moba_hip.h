@@ -237,7 +237,7 @@ int moba_fwd(const void* q, const void* k, const void* v, void* part_o, float* p
  *   dq, dk, dv: out; dk and dv of a key/value head sum over its query heads
  *   queues [16] int32 scratch: tile counters of the dQ and dK/dV kernels (as in moba_fwd_partials)
  *   dkv_scratch: moba_bwd_dkv_scratch_bytes(S, Hkv, self_tiles) bytes, 16-byte aligned, or null.  With few key tiles
- *              (fewer than two per compute unit, S >= 16384) the dK/dV kernel cuts each into up to 4 parts that run
+ *              (fewer than two per compute unit, S >= 4096) the dK/dV kernel cuts each into up to 4 parts that run
  *              side by side and leave fp32 sums there, added up in a fixed order (deterministic all the same);
  *              without the scratch, or when the query returns 0, every tile is one piece.
  *   softmax_scale: as in the forward call */

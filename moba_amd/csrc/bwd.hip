@@ -934,10 +934,10 @@ extern "C" int moba_bwd_tile_rows(void) { return TM; }
 // Parts per key tile of the dK/dV kernel.  With fewer tiles than two per compute unit the tiles of the first
 // chunks of a sequence, whose gather lists are the longest, set the kernel's time while most of the chip is
 // idle: they are cut into parts then (at most 4: every part leaves 128 KiB of fp32 sums to be added up).
-// Problems below 16384 tokens are too short for the parts' extra traffic to pay.
+// Problems below 4096 tokens are too short for the parts' extra traffic to pay.
 static int dkv_split_for(int64_t S, int64_t tiles) {
   const int cus = resident_compute_units();
-  if (cus <= 0 || tiles <= 0 || tiles >= 2 * (int64_t)cus || S < 16384) return 1;
+  if (cus <= 0 || tiles <= 0 || tiles >= 2 * (int64_t)cus || S < 4096) return 1;
   const int64_t r = (3 * (int64_t)cus + tiles - 1) / tiles;
   return (int)(r < 1 ? 1 : (r > 4 ? 4 : r));
 }
