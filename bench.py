@@ -278,11 +278,12 @@ def main():
     if args.decode:
         result["decode"] = bench_decode(dev, S if len(cu) == 2 else max_seqlen, H)
     if others:
-        # the other BASELINE configurations, a few steps each (cfg5: BASELINE asks for the forward; the backward runs too)
+        # the other BASELINE configurations, 200 steps of the two small ones, a few of the others
+        # (cfg5: BASELINE asks for the forward; the backward runs too)
         del q, k, v
         torch.cuda.empty_cache()
         result["other_configs"] = {}
-        for name, steps, warmup in (("cfg1_L4096_h4_c512_k3", 20, 5), ("cfg2_L32768_h1_c2048_k3", 20, 5),
+        for name, steps, warmup in (("cfg1_L4096_h4_c512_k3", 200, 20), ("cfg2_L32768_h1_c2048_k3", 200, 20),
                                     ("cfg3_varlen8_h32_c2048_k3", 3, 1), ("cfg5_L1048576_h32_c4096_k12", 2, 1)):
             result["other_configs"][name] = quick_measure(name, dev, steps, warmup, backward=True)
             torch.cuda.empty_cache()
