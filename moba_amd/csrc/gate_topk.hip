@@ -152,7 +152,7 @@ __global__ __launch_bounds__(256) void gate_topk_kernel(
   }
   // The gather lists' counts as a by-product: how many tokens of a (query chunk, head) picked each earlier chunk,
   // added into cnt[(chunk, head, query chunk)] (integer sums: the order of the additions does not matter).  A
-  // wave's 64 tokens lie in one query chunk, or in a few: one round per chunk, through a histogram in LDS.
+  // wave's 64 tokens lie in one query chunk, or in a few: one pass per chunk, through a histogram in LDS.
   if (!cnt) return;
   __syncthreads();  // (the staged lists are stored)
   constexpr int kHist = (int)(sizeof(sc) / sizeof(int)) / 4;
