@@ -101,10 +101,11 @@ __device__ __forceinline__ float round_to_odd_f32(double x) {
 }
 
 template <class E>
-__global__ __launch_bounds__(256) void chunk_mean_finish_kernel(
+__global__ __launch_bounds__(64) void chunk_mean_finish_kernel(
     const double* __restrict__ partial, typename E::elem* __restrict__ kbar, int HD8, int B, int nsplit, int F) {
   MOBA_ELEM_TYPES(E)
-  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;  // over F * HD8
+  // (one wave per workgroup: a small problem's few hundred outputs then spread over several compute units)
+  const int64_t idx = (int64_t)blockIdx.x * 64 + threadIdx.x;  // over F * HD8
   if (idx >= (int64_t)F * HD8) return;
   const int f = (int)(idx / HD8);
   const int col = (int)(idx % HD8);
@@ -170,16 +171,16 @@ static int launch_chunk_mean(const void* k, const int32_t* fchunk_tok, void* kba
   const int cpb_log2 = pick_cpb_log2(HD8);
   dim3 grid(F, nsplit, (HD8 + (1 << cpb_log2) - 1) >> cpb_log2);
   const int64_t n = (int64_t)F * HD8;
-  const dim3 fgrid((unsigned)((n + 255) / 256));
+  const dim3 fgrid((unsigned)((n + 63) / 64));
   if (dtype == MOBA_DTYPE_F16) {
     hipLaunchKernelGGL(chunk_mean_partial_kernel<F16>, grid, dim3(256), 0, st, (const f16*)k, fchunk_tok, partial,
                        HD8, D / 8, B, nsplit, tps, kts, khs, batch_rows, kbs, cpb_log2, clear, clear_ints);
-    hipLaunchKernelGGL(chunk_mean_finish_kernel<F16>, fgrid, dim3(256), 0, st, (const double*)partial, (f16*)kbar,
+    hipLaunchKernelGGL(chunk_mean_finish_kernel<F16>, fgrid, dim3(64), 0, st, (const double*)partial, (f16*)kbar,
                        HD8, B, nsplit, F);
   } else {
     hipLaunchKernelGGL(chunk_mean_partial_kernel<Bf16>, grid, dim3(256), 0, st, (const bf16*)k, fchunk_tok, partial,
                        HD8, D / 8, B, nsplit, tps, kts, khs, batch_rows, kbs, cpb_log2, clear, clear_ints);
-    hipLaunchKernelGGL(chunk_mean_finish_kernel<Bf16>, fgrid, dim3(256), 0, st, (const double*)partial, (bf16*)kbar,
+    hipLaunchKernelGGL(chunk_mean_finish_kernel<Bf16>, fgrid, dim3(64), 0, st, (const double*)partial, (bf16*)kbar,
                        HD8, B, nsplit, F);
   }
   return launch_check.result();
