@@ -55,7 +55,7 @@ extern "C" {
 
 enum { MOBA_DTYPE_BF16 = 0, MOBA_DTYPE_F16 = 1 };
 
-#define MOBA_ABI_VERSION 110 /* the signatures below; moba_version() returns the number the library was built with */
+#define MOBA_ABI_VERSION 111 /* the signatures below; moba_version() returns the number the library was built with */
 int moba_version(void);
 const char* moba_strerror(int code);
 
@@ -160,11 +160,15 @@ int moba_topk_from_scores(const float* scores, int32_t* sel, int64_t S, int H, i
  *   tile_seg [hist_bound] out: segment f*H + h of every history tile id, -1 past the last tile
  * cmax = most chunks in a sequence minus one; tile_rows = rows per tile of the kernel that will read tile_off and
  * tile_seg (moba_fwd_tile_rows() or moba_bwd_tile_rows()); hist_bound: an upper bound on the number of tiles,
- * e.g. M / tile_rows + F * H. */
+ * e.g. M / tile_rows + F * H.
+ * tile_rows_b, tile_off_b [F*H+1], tile_seg_b [hist_bound_b]: optional second pair of tile tables for another tile
+ * height (what moba_tile_tables would make from seg_off: a caller that will run the backward asks for its tables
+ * here and saves that launch on small problems); tile_off_b NULL for none. */
 int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, const int32_t* chunk_fb, const int32_t* chunk_local,
                      const int32_t* pair_off, int32_t* cnt, int32_t* seg_off, int32_t* tile_off, int32_t* seg_dest,
                      int32_t* tile_seg, int64_t S, int H, int K, int N, int F, int P, int cmax, int tile_rows,
-                     int64_t hist_bound, int counted, void* stream);
+                     int64_t hist_bound, int counted, int tile_rows_b, int32_t* tile_off_b, int32_t* tile_seg_b,
+                     int64_t hist_bound_b, void* stream);
 
 /* The tile tables of moba_build_lists alone, for another tile height: the forward and the backward kernels cut
  * the same gather lists into tiles of moba_fwd_tile_rows() and moba_bwd_tile_rows() rows.  No counterpart in the

@@ -33,7 +33,8 @@ _SIGNATURES = {
     "moba_gate_topk": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_strides, c_int, c_void_p]),
     "moba_topk_from_scores": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_void_p]),
-    "moba_build_lists": (c_int, [c_void_p] * 10 + [c_int64] + [c_int] * 7 + [c_int64, c_int, c_void_p]),
+    "moba_build_lists": (c_int, [c_void_p] * 10 + [c_int64] + [c_int] * 7 + [c_int64, c_int, c_int, c_void_p, c_void_p,
+                                                                             c_int64, c_void_p]),
     "moba_tile_tables": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int64, c_void_p]),
     "moba_fwd_tile_rows": (c_int, []),
     "moba_bwd_tile_rows": (c_int, []),
@@ -71,7 +72,7 @@ class SizesStruct(ctypes.Structure):
     _fields_ = [(n, c_int64) for n in ("kbar_elems", "chunk_mean_workspace_bytes", "sel_ints", "cnt_ints", "seg_off_ints",
                                        "seg_dest_ints", "fwd_hist_bound", "bwd_hist_bound", "part_rows", "redo_ints",
                                        "lse_floats", "delta_floats")]
-ABI_VERSION = 110  # MOBA_ABI_VERSION of include/moba_hip.h, the signatures above
+ABI_VERSION = 111  # MOBA_ABI_VERSION of include/moba_hip.h, the signatures above
 DTYPE_BF16, DTYPE_F16 = 0, 1
 
 

@@ -355,7 +355,8 @@ __global__ __launch_bounds__(1024) void lists_fill_tail_kernel(
     const int* __restrict__ sel, const int* __restrict__ chunk_tok, const int* __restrict__ chunk_fb,
     const int* __restrict__ chunk_local, const int* __restrict__ pair_off, const int* __restrict__ cnt,
     int* __restrict__ seg_dest, int* __restrict__ seg_off, int* __restrict__ tile_off, int* __restrict__ tile_seg,
-    int N, int H, int K, int F, int PH, int tile_rows, int bound) {
+    int N, int H, int K, int F, int PH, int tile_rows, int bound, int tile_rows_b, int* __restrict__ tile_off_b,
+    int* __restrict__ tile_seg_b, int bound_b) {
   __shared__ int sbase[kFusedMaxCounts + 1];
   // the tail's tile starts, or the fill's positions and lane masks: 16 waves x 3 ints per candidate chunk
   __shared__ int off[kFusedMaxCand * 48 > kTailMaxSegments + 1 ? kFusedMaxCand * 48 : kTailMaxSegments + 1];
@@ -393,9 +394,14 @@ __global__ __launch_bounds__(1024) void lists_fill_tail_kernel(
     __syncthreads();
     return sbase;
   };
-  if (blockIdx.x == N)
-    lists_tail_body(scanned_counts(), pair_off, seg_off, tile_off, tile_seg, F, H, tile_rows, bound, off, wsum);
-  else
+  if (blockIdx.x == N) {
+    const int* base = scanned_counts();
+    lists_tail_body(base, pair_off, seg_off, tile_off, tile_seg, F, H, tile_rows, bound, off, wsum);
+    if (tile_off_b) {  // the same lists cut into tiles of another height (the backward kernels')
+      __syncthreads();
+      lists_tail_body(base, pair_off, seg_off, tile_off_b, tile_seg_b, F, H, tile_rows_b, bound_b, off, wsum);
+    }
+  } else
     lists_fill_body<KC, 16>(sel, chunk_tok, chunk_fb, chunk_local, pair_off, scanned_counts, seg_dest, H, K, off);
 }
 
@@ -403,32 +409,50 @@ __global__ __launch_bounds__(1024) void lists_fill_tail_kernel(
 
 using namespace moba;
 
+static void launch_tile_tables(const int32_t* seg_off, int32_t* tile_off, int32_t* tile_seg, int H, int F,
+                               int tile_rows, int64_t hist_bound, hipStream_t st) {
+  if ((int64_t)F * H < kTailMaxSegments && hist_bound <= kTailMaxTiles) {
+    hipLaunchKernelGGL(lists_tail_kernel, dim3(1), dim3(1024), 0, st, (const int*)nullptr, (const int*)nullptr,
+                       const_cast<int*>(seg_off), tile_off, tile_seg, F, H, tile_rows, (int)hist_bound);
+    return;
+  }
+  hipLaunchKernelGGL(lists_tile_counts_kernel, dim3((F * H + 255) / 256), dim3(256), 0, st, seg_off, tile_off, F * H,
+                     tile_rows);
+  hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(1024), 0, st, tile_off, F * H);
+  hipLaunchKernelGGL(lists_tile_seg_kernel, dim3((unsigned)((hist_bound + 255) / 256)), dim3(256), 0, st,
+                     (const int*)tile_off, tile_seg, F * H, (int)hist_bound);
+}
+
 // Limits: chunks per sequence minus one (cmax) is bounded by the LDS the fill pass
 // needs, 48 bytes per candidate chunk.
 extern "C" int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, const int32_t* chunk_fb,
                                 const int32_t* chunk_local, const int32_t* pair_off, int32_t* cnt,
                                 int32_t* seg_off, int32_t* tile_off, int32_t* seg_dest, int32_t* tile_seg,
                                 int64_t S, int H, int K, int N, int F, int P, int cmax, int tile_rows,
-                                int64_t hist_bound, int counted, void* stream) {
+                                int64_t hist_bound, int counted, int tile_rows_b, int32_t* tile_off_b,
+                                int32_t* tile_seg_b, int64_t hist_bound_b, void* stream) {
   LaunchCheck launch_check;
   if (!sel || !chunk_tok || !chunk_fb || !chunk_local || !pair_off || !cnt || !seg_off || !tile_off || !seg_dest ||
       !tile_seg)
     return MOBA_ERR_ARG;
   if (hist_bound <= 0 || hist_bound >= 0x7fffffffLL) return MOBA_ERR_ARG;
+  if (tile_off_b && (!tile_seg_b || tile_rows_b <= 0 || hist_bound_b <= 0 || hist_bound_b >= 0x7fffffffLL))
+    return MOBA_ERR_ARG;
   if (S <= 0 || H <= 0 || K <= 0 || N <= 0 || F <= 0 || P <= 0 || cmax <= 0 || tile_rows <= 0) return MOBA_ERR_ARG;
   if ((int64_t)S * H * (K + 1) >= 0x7fffffffLL || (int64_t)P * H >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
   if (H > 65535 || (size_t)cmax * 48 > 160 * 1024) return MOBA_ERR_LIMIT;
   hipStream_t st = (hipStream_t)stream;
   dim3 grid(N, H);
   const bool small_tail = (int64_t)F * H < kTailMaxSegments && hist_bound <= kTailMaxTiles;
-  if (small_tail && (int64_t)P * H <= kFusedMaxCounts && cmax <= kFusedMaxCand && (int64_t)N * H <= 512 && K <= 16) {
+  if (small_tail && (int64_t)P * H <= kFusedMaxCounts && cmax <= kFusedMaxCand && (int64_t)N * H <= 512 && K <= 16 &&
+      (!tile_off_b || hist_bound_b <= kTailMaxTiles)) {
     if (!counted)
       hipLaunchKernelGGL(lists_count_kernel<1024>, grid, dim3(1024), (size_t)cmax * 4, st, sel, chunk_tok, chunk_fb,
                          chunk_local, pair_off, cnt, H, K);
 #define MOBA_FILL_TAIL(KC)                                                                                       \
   hipLaunchKernelGGL(lists_fill_tail_kernel<KC>, dim3(N + 1, H), dim3(1024), 0, st, sel, chunk_tok, chunk_fb,    \
                      chunk_local, pair_off, (const int*)cnt, seg_dest, seg_off, tile_off, tile_seg, N, H, K, F,  \
-                     P * H, tile_rows, (int)hist_bound)
+                     P * H, tile_rows, (int)hist_bound, tile_rows_b, tile_off_b, tile_seg_b, (int)hist_bound_b)
     if (K <= 4) MOBA_FILL_TAIL(4);
     else MOBA_FILL_TAIL(16);
 #undef MOBA_FILL_TAIL
@@ -456,13 +480,14 @@ extern "C" int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, co
   if (small_tail) {
     hipLaunchKernelGGL(lists_tail_kernel, dim3(1), dim3(1024), 0, st, (const int*)cnt, pair_off, seg_off, tile_off,
                        tile_seg, F, H, tile_rows, (int)hist_bound);
-    return launch_check.result();
+  } else {
+    hipLaunchKernelGGL(lists_segments_kernel, dim3((F * H + 1 + 255) / 256), dim3(256), 0, st, (const int*)cnt,
+                       pair_off, seg_off, tile_off, F, H, tile_rows);
+    hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(1024), 0, st, tile_off, F * H);
+    hipLaunchKernelGGL(lists_tile_seg_kernel, dim3((unsigned)((hist_bound + 255) / 256)), dim3(256), 0, st,
+                       (const int*)tile_off, tile_seg, F * H, (int)hist_bound);
   }
-  hipLaunchKernelGGL(lists_segments_kernel, dim3((F * H + 1 + 255) / 256), dim3(256), 0, st, (const int*)cnt,
-                     pair_off, seg_off, tile_off, F, H, tile_rows);
-  hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(1024), 0, st, tile_off, F * H);
-  hipLaunchKernelGGL(lists_tile_seg_kernel, dim3((unsigned)((hist_bound + 255) / 256)), dim3(256), 0, st,
-                     (const int*)tile_off, tile_seg, F * H, (int)hist_bound);
+  if (tile_off_b) launch_tile_tables(seg_off, tile_off_b, tile_seg_b, H, F, tile_rows_b, hist_bound_b, st);
   return launch_check.result();
 }
 
@@ -474,16 +499,6 @@ extern "C" int moba_tile_tables(const int32_t* seg_off, int32_t* tile_off, int32
   if (!seg_off || !tile_off || !tile_seg) return MOBA_ERR_ARG;
   if (H <= 0 || F <= 0 || tile_rows <= 0 || hist_bound <= 0 || hist_bound >= 0x7fffffffLL) return MOBA_ERR_ARG;
   if ((int64_t)F * H >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
-  hipStream_t st = (hipStream_t)stream;
-  if ((int64_t)F * H < kTailMaxSegments && hist_bound <= kTailMaxTiles) {
-    hipLaunchKernelGGL(lists_tail_kernel, dim3(1), dim3(1024), 0, st, (const int*)nullptr, (const int*)nullptr,
-                       const_cast<int*>(seg_off), tile_off, tile_seg, F, H, tile_rows, (int)hist_bound);
-    return launch_check.result();
-  }
-  hipLaunchKernelGGL(lists_tile_counts_kernel, dim3((F * H + 255) / 256), dim3(256), 0, st, seg_off, tile_off, F * H,
-                     tile_rows);
-  hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(1024), 0, st, tile_off, F * H);
-  hipLaunchKernelGGL(lists_tile_seg_kernel, dim3((unsigned)((hist_bound + 255) / 256)), dim3(256), 0, st,
-                     (const int*)tile_off, tile_seg, F * H, (int)hist_bound);
+  launch_tile_tables(seg_off, tile_off, tile_seg, H, F, tile_rows, hist_bound, (hipStream_t)stream);
   return launch_check.result();
 }

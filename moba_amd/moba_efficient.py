@@ -193,22 +193,29 @@ def list_buffers(plan: MobaPlan, H: int, device, tile_rows: int = FWD_TILE_ROWS)
     return tuple(buf[a:a + n] for a, n in zip(starts, sizes))
 
 
-def build_lists(sel: torch.Tensor, plan: MobaPlan, tile_rows: int = FWD_TILE_ROWS, buffers=None, counted=False):
+def build_lists(sel: torch.Tensor, plan: MobaPlan, tile_rows: int = FWD_TILE_ROWS, buffers=None, counted=False,
+                second_tile_rows: int = 0):
     """(seg_off [F*H+1], tile_off [F*H+1], seg_dest [M], tile_seg [tile bound]) int32 -- see csrc/lists.hip.
     The tile tables cut the lists into tiles of `tile_rows` rows (the forward kernel's by default).
     `buffers`: list_buffers() of the same plan, heads and tile_rows; `counted`: their cnt already holds the
-    counts, left there by gate_topk."""
+    counts, left there by gate_topk; `second_tile_rows`: also return (tile_off, tile_seg) for tiles of that height."""
     lib = _lib.load()
     S, H, K = sel.shape
     dev = sel.device
     bound = plan.hist_tile_bound(H, tile_rows)
     cnt, seg_off, tile_off, seg_dest, tile_seg = buffers if buffers is not None else list_buffers(plan, H, dev, tile_rows)
     t = plan.tables
+    second, second_args = (), (0, None, None, 0)
+    if second_tile_rows:
+        bound_b = plan.hist_tile_bound(H, second_tile_rows)
+        second = (torch.empty(plan.F * H + 1, dtype=torch.int32, device=dev),
+                  torch.empty(bound_b, dtype=torch.int32, device=dev))
+        second_args = (second_tile_rows, _ptr(second[0]), _ptr(second[1]), bound_b)
     _lib.check(lib.moba_build_lists(_ptr(sel), _ptr(t["chunk_tok"]), _ptr(t["chunk_fb"]), _ptr(t["chunk_local"]),
                                     _ptr(t["pair_off"]), _ptr(cnt), _ptr(seg_off), _ptr(tile_off), _ptr(seg_dest),
                                     _ptr(tile_seg), S, H, K, plan.N, plan.F, plan.P, plan.cmax, tile_rows, bound,
-                                    1 if counted else 0, _stream(dev)), "moba_build_lists")
-    return seg_off, tile_off, seg_dest, tile_seg
+                                    1 if counted else 0, *second_args, _stream(dev)), "moba_build_lists")
+    return (seg_off, tile_off, seg_dest, tile_seg) + second
 
 
 def tile_tables(seg_off: torch.Tensor, plan: MobaPlan, H: int, tile_rows: int):
@@ -288,6 +295,10 @@ class _Geometry:
         for n in sizes:
             starts.append(starts[-1] + (n + 3) // 4 * 4)
         self.list_starts = starts
+        # ... and, for a call that a backward will follow, the backward kernels' tile tables behind them
+        self.bwd_bound = plan.hist_tile_bound(H, TILE_ROWS)
+        self.bwd_starts = [starts[-1], starts[-1] + (plan.F * H + 1 + 3) // 4 * 4]
+        self.list_ints_with_bwd = self.bwd_starts[1] + self.bwd_bound
         # attention scratch: per-slot partial outputs, their log-sum-exps, the kernel's 8 tile counters, then
         # the list of tiles its fixed-reference softmax hands to the kernel that tracks the running maximum
         # (count first; the call zeroes the counters and the count)
@@ -308,9 +319,10 @@ def _geometry(plan: MobaPlan, lib, H: int, D: int, esize: int) -> _Geometry:
     return g
 
 
-def _forward(q, k, v, plan: MobaPlan, timer: Optional[StageTimer] = None, scale: float = 0.0):
+def _forward(q, k, v, plan: MobaPlan, timer: Optional[StageTimer] = None, scale: float = 0.0, bwd_tables=None):
     """q, k, v: [tokens, heads, 128], or batched [batch, heads, tokens, 128] (read in place, see _dims), already
     addressable (_in_place).  Returns (out, lse, sel, seg_off, tile_off, seg_dest, tile_seg).
+    bwd_tables: a list that receives the backward kernels' (tile_off, tile_seg), made on the way.
     The stages are those of chunk_mean(), gate_topk(), build_lists() above, called on precomputed sizes and
     addresses: at small shapes a forward is bound by the host's time per call."""
     lib = _lib.load()
@@ -333,8 +345,15 @@ def _forward(q, k, v, plan: MobaPlan, timer: Optional[StageTimer] = None, scale:
         kbar = torch.empty((plan.F, Hkv, D), dtype=q.dtype, device=dev)
         ws = torch.empty(mean_ws, dtype=torch.float64, device=dev)
         sel = torch.empty((S, H, K), dtype=torch.int32, device=dev)
-        lists = torch.empty(g.list_starts[-1], dtype=torch.int32, device=dev)
+        lists = torch.empty(g.list_starts[-1] if bwd_tables is None else g.list_ints_with_bwd, dtype=torch.int32,
+                            device=dev)
         base = lists.data_ptr()
+        if bwd_tables is None:
+            bwd_args = (0, null, null, 0)
+        else:
+            b0, b1 = g.bwd_starts
+            bwd_tables += [lists[b0:b0 + plan.F * H + 1], lists[b1:b1 + g.bwd_bound]]
+            bwd_args = (TILE_ROWS, ctypes.c_void_p(base + 4 * b0), ctypes.c_void_p(base + 4 * b1), g.bwd_bound)
         cntp, seg_offp, tile_offp, seg_destp, tile_segp = (ctypes.c_void_p(base + 4 * a) for a in g.list_starts[:5])
         seg_off, tile_off, seg_dest, tile_seg = (lists[a:a + n] for a, n in zip(g.list_starts[1:5], g.list_sizes[1:]))
         selp, kbarp = _ptr(sel), _ptr(kbar)
@@ -349,7 +368,8 @@ def _forward(q, k, v, plan: MobaPlan, timer: Optional[StageTimer] = None, scale:
         with span("build_lists"):
             _lib.check(lib.moba_build_lists(selp, tp["chunk_tok"], tp["chunk_fb"], tp["chunk_local"], tp["pair_off"],
                                             cntp, seg_offp, tile_offp, seg_destp, tile_segp, S, H, K, plan.N, plan.F,
-                                            plan.P, plan.cmax, FWD_TILE_ROWS, g.bound, 1, stream), "moba_build_lists")
+                                            plan.P, plan.cmax, FWD_TILE_ROWS, g.bound, 1, *bwd_args, stream),
+                       "moba_build_lists")
     out = torch.empty((S, H, D), dtype=q.dtype, device=dev)
     lse = torch.empty((S, H), dtype=torch.float32, device=dev)
     ws2 = torch.empty(g.ws_bytes, dtype=torch.uint8, device=dev)
@@ -370,7 +390,8 @@ def _forward(q, k, v, plan: MobaPlan, timer: Optional[StageTimer] = None, scale:
     return out, lse, sel, seg_off, tile_off, seg_dest, tile_seg
 
 
-def _backward(dout, q, k, v, out, lse, sel, seg_off, seg_dest, plan: MobaPlan, scale: float = 0.0):
+def _backward(dout, q, k, v, out, lse, sel, seg_off, seg_dest, plan: MobaPlan, scale: float = 0.0, tables=None):
+    """tables: the backward kernels' (tile_off, tile_seg) if the forward made them (made here otherwise)."""
     lib = _lib.load()
     S, H, D = _dims(q)
     Hkv = _dims(k)[1]
@@ -401,6 +422,8 @@ def _backward(dout, q, k, v, out, lse, sel, seg_off, seg_dest, plan: MobaPlan, s
     part_dqp, deltap, queuesp, tile_offp, tile_segp, kvp = (ctypes.c_void_p(base + a) for a in starts[:6])
     if plan.fallback:
         tile_offp = tile_segp = null
+    elif tables:
+        tile_offp, tile_segp = _ptr(tables[0]), _ptr(tables[1])
     else:
         _lib.check(lib.moba_tile_tables(_ptr(seg_off), tile_offp, tile_segp, H, plan.F, TILE_ROWS, bound, stream),
                    "moba_tile_tables")
@@ -421,10 +444,11 @@ class _MobaAttention(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q, k, v, plan, timer=None, scale=0.0):
-        out, lse, sel, seg_off, _, seg_dest, _ = _forward(q, k, v, plan, timer, scale)
+        tables = []  # the backward's tile tables, made by the forward's list stage
+        out, lse, sel, seg_off, _, seg_dest, _ = _forward(q, k, v, plan, timer, scale, bwd_tables=tables)
         ctx.plan = plan
         ctx.scale = scale
-        ctx.aux = (sel, seg_off, seg_dest)
+        ctx.aux = (sel, seg_off, seg_dest, tables)
         ctx.save_for_backward(q, k, v, out, lse)
         ctx.mark_non_differentiable(lse)
         ctx.set_materialize_grads(False)  # no zero-filled gradient for lse on the way back
@@ -433,10 +457,11 @@ class _MobaAttention(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dout, _dlse):
         q, k, v, out, lse = ctx.saved_tensors
-        sel, seg_off, seg_dest = ctx.aux
+        sel, seg_off, seg_dest, tables = ctx.aux
         if dout is None:
             return None, None, None, None, None, None
-        dq, dk, dv = _backward(_aligned(dout.to(q.dtype)), q, k, v, out, lse, sel, seg_off, seg_dest, ctx.plan, ctx.scale)
+        dq, dk, dv = _backward(_aligned(dout.to(q.dtype)), q, k, v, out, lse, sel, seg_off, seg_dest, ctx.plan, ctx.scale,
+                               tables)
         if q.dim() == 4:   # gradients in the layout of the batched inputs: views of the packed results
             b, _, l, d = q.shape
             dq, dk, dv = (g.view(b, l, -1, d).transpose(1, 2) for g in (dq, dk, dv))

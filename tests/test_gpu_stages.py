@@ -128,11 +128,11 @@ def test_gather_lists(batch, seqlen, heads, B, topk, counted):
         sel = E.gate_topk(q.cuda(), kbar.cuda(), plan, cnt=buffers[0])
         assert int(buffers[0].sum()) == plan.pairs_per_head * heads
         assert torch.equal(sel, E.gate_topk(q.cuda(), kbar.cuda(), plan))
-        lists = E.build_lists(sel, plan, buffers=buffers, counted=True)
+        lists = E.build_lists(sel, plan, buffers=buffers, counted=True, second_tile_rows=128)
     else:
         sel = E.gate_topk(q.cuda(), kbar.cuda(), plan)
-        lists = E.build_lists(sel, plan)
-    seg_off, tile_off, seg_dest, tile_seg = (x.cpu().numpy() for x in lists)
+        lists = E.build_lists(sel, plan, second_tile_rows=128)
+    seg_off, tile_off, seg_dest, tile_seg, second_off, second_seg = (x.cpu().numpy() for x in lists)
     sel = sel.cpu()
     counts, offs, rows, slots = O.gather_lists(sel, plan.F)
     H, K1 = heads, plan.K + 1
@@ -147,6 +147,8 @@ def test_gather_lists(batch, seqlen, heads, B, topk, counted):
     assert (fwd_rows, bwd_rows) == (256, 128)
     # the tile tables: the forward kernel's from moba_build_lists, the backward kernels' from moba_tile_tables
     bwd_off, bwd_seg = (x.cpu().numpy() for x in E.tile_tables(torch.from_numpy(seg_off).cuda(), plan, H, bwd_rows))
+    # ... or, for a caller that asks, from moba_build_lists as a second pair
+    assert np.array_equal(second_off, bwd_off) and np.array_equal(second_seg, bwd_seg)
     for rows_per_tile, toff, tseg in ((fwd_rows, tile_off, tile_seg), (bwd_rows, bwd_off, bwd_seg)):
         tiles = (counts + rows_per_tile - 1) // rows_per_tile
         assert np.array_equal(toff, np.concatenate([[0], np.cumsum(tiles)]))
