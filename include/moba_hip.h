@@ -91,7 +91,8 @@ typedef struct moba_sizes_t {
   int64_t seg_off_ints;                    /* [F*H + 1]; tile_off has the same size */
   int64_t seg_dest_ints;                   /* [M] */
   int64_t fwd_hist_bound, bwd_hist_bound;  /* sizes of the two tile_seg tables = the hist_bound arguments */
-  int64_t part_rows;                       /* S*H*(K+1): part_o, part_dq [part_rows, D] elem; part_lse [part_rows] fp32 */
+  int64_t part_rows;                       /* S*H*(K+1): part_o, part_dq [part_rows, D] elem; part_lse [part_rows] fp32
+                                              (times key_split for part_o, part_lse, times dq_key_split for part_dq) */
   int64_t redo_ints;
   int64_t lse_floats;                      /* [S, H] */
   int64_t delta_floats;                    /* [2, S, H] */
