@@ -55,7 +55,7 @@ extern "C" {
 
 enum { MOBA_DTYPE_BF16 = 0, MOBA_DTYPE_F16 = 1 };
 
-#define MOBA_ABI_VERSION 111 /* the signatures below; moba_version() returns the number the library was built with */
+#define MOBA_ABI_VERSION 112 /* the signatures below; moba_version() returns the number the library was built with */
 int moba_version(void);
 const char* moba_strerror(int code);
 
@@ -66,9 +66,20 @@ const char* moba_strerror(int code);
  * moba_plan fills `plan` (counts, table offsets and table_ints); moba_plan_fill does the same and writes the tables
  * into tables_host [plan->table_ints] int32, which the caller copies to the device once per batch layout: table X
  * then lives at device_base + plan->off_X (off_X = -1: the table does not exist in the full-attention fallback,
- * pass NULL).  Tables: cu_seqlens, chunk_tok [N+1], fwd_self_tile_prefix [N+1] / fwd_self_tile_chunk (the
- * self_tile_* arguments of moba_fwd*), self_tile_prefix / self_tile_chunk (those of moba_bwd), seq_fbase [nseq+1],
- * fchunk_tok [F], chunk_fb [N], chunk_local [N], pair_off [F+1], chunk_fid [N].
+ * pass NULL).
+ * Dense prefixes (dense = 1; no counterpart in the reference): a token in chunk c <= K of its sequence selects
+ * every earlier chunk, so what it attends is the plain causal prefix of its sequence.  The plan then makes the chunks
+ * 0..K of every sequence one *attention chunk* (dense_local = K) whose rows the kernels serve through their causal
+ * self path alone: one partial result instead of c + 1, no picks in sel (moba_gate_topk writes -1 for them), no
+ * list entries (pairs_per_head counts the other tokens' only).  The attended sets, and so the results up to
+ * rounding, are those of dense = 0, where every chunk is its own attention chunk (dense_local = 0, NA = N).
+ * It pays for problems of many tiles (ask moba_fwd_is_queued with the dense plan's counts); on a small problem the
+ * long causal tiles of a prefix would run alone at the end.
+ * Tables: cu_seqlens, chunk_tok [N+1], achunk_tok [NA+1] (first token of every attention chunk: the chunk_tok
+ * argument of moba_fwd* and moba_bwd), fwd_self_tile_prefix [NA+1] / fwd_self_tile_chunk (the self_tile_* arguments of
+ * moba_fwd*), self_tile_prefix [NA+1] / self_tile_chunk (those of moba_bwd), kv_tile_prefix [N+1] / kv_tile_chunk
+ * and chunk_self_end [N] (moba_bwd), seq_fbase [nseq+1], fchunk_tok [F], chunk_fb [N], chunk_local [N], pair_off [F+1],
+ * chunk_fid [N].
  * moba_plan_sizes gives, for H query and Hkv key/value heads, the size of every scratch buffer of the calls below. */
 typedef struct moba_plan_t {
   int64_t S;
@@ -76,11 +87,15 @@ typedef struct moba_plan_t {
   int32_t N, F, K, P, cmax;
   int32_t fallback;                        /* 1: full causal attention (K = 0, one "chunk" per sequence) */
   int32_t fwd_tile_rows, bwd_tile_rows;
+  int32_t dense_local;                     /* chunks 0..dense_local of a sequence are one attention chunk */
+  int32_t NA;                              /* attention chunks: the N argument of moba_fwd* and moba_bwd */
   int64_t pairs_per_head;                  /* M = pairs_per_head * H */
   int64_t fwd_self_tiles, bwd_self_tiles;  /* the self_tiles arguments of moba_fwd* and of moba_bwd */
+  int64_t kv_tiles;                        /* the kv_tiles argument of moba_bwd */
   double flops_per_head_per_dim;           /* forward flops = this * H * D */
-  int64_t off_cu_seqlens, off_chunk_tok, off_fwd_self_tile_prefix, off_fwd_self_tile_chunk, off_self_tile_prefix,
-      off_self_tile_chunk, off_seq_fbase, off_fchunk_tok, off_chunk_fb, off_chunk_local, off_pair_off, off_chunk_fid;
+  int64_t off_cu_seqlens, off_chunk_tok, off_achunk_tok, off_fwd_self_tile_prefix, off_fwd_self_tile_chunk,
+      off_self_tile_prefix, off_self_tile_chunk, off_kv_tile_prefix, off_kv_tile_chunk, off_chunk_self_end,
+      off_seq_fbase, off_fchunk_tok, off_chunk_fb, off_chunk_local, off_pair_off, off_chunk_fid;
   int64_t table_ints;
 } moba_plan_t;
 typedef struct moba_sizes_t {
@@ -97,8 +112,8 @@ typedef struct moba_sizes_t {
   int64_t lse_floats;                      /* [S, H] */
   int64_t delta_floats;                    /* [2, S, H] */
 } moba_sizes_t;
-int moba_plan(const int32_t* cu_seqlens_host, int nseq, int chunk, int topk, moba_plan_t* plan);
-int moba_plan_fill(const int32_t* cu_seqlens_host, int nseq, int chunk, int topk, moba_plan_t* plan,
+int moba_plan(const int32_t* cu_seqlens_host, int nseq, int chunk, int topk, int dense, moba_plan_t* plan);
+int moba_plan_fill(const int32_t* cu_seqlens_host, int nseq, int chunk, int topk, int dense, moba_plan_t* plan,
                    int32_t* tables_host);
 int moba_plan_sizes(const moba_plan_t* plan, int H, int Hkv, int D, moba_sizes_t* sizes);
 
@@ -138,10 +153,12 @@ int moba_chunk_mean_static(const void* k, const int32_t* fchunk_tok, void* kbar,
  *              counts that moba_build_lists starts from (how many tokens of each query chunk and head picked
  *              each chunk; pass counted = 1 there); needs pair_off [F+1], the table of moba_build_lists.
  *              NULL: no counts.
+ *   dense_local the plan's: the tokens of the chunks 0..dense_local of every sequence get no picks (-1) and no
+ *              counts; 0 for the reference's selection
  * K <= 64.  strides[0], strides[1] apply to q; kbar is packed [F,Hkv,D]. */
 int moba_gate_topk(const void* q, const void* kbar, const int32_t* cu_seqlens, const int32_t* seq_fbase, int32_t* sel,
                    float* scores_out, const int32_t* pair_off, int32_t* cnt, int64_t S, int H, int Hkv, int D,
-                   int nseq, int F, int B, int K, const int64_t* strides, int dtype, void* stream);
+                   int nseq, int F, int B, int K, int dense_local, const int64_t* strides, int dtype, void* stream);
 
 /* The selection step of moba/moba_efficient.py:365-371 alone, on caller-supplied
  * scores [S,H,F] fp32 (-inf = not a candidate).  Same routine as moba_gate_topk. */
@@ -164,12 +181,14 @@ int moba_topk_from_scores(const float* scores, int32_t* sel, int64_t S, int H, i
  * e.g. M / tile_rows + F * H.
  * tile_rows_b, tile_off_b [F*H+1], tile_seg_b [hist_bound_b]: optional second pair of tile tables for another tile
  * height (what moba_tile_tables would make from seg_off: a caller that will run the backward asks for its tables
- * here and saves that launch on small problems); tile_off_b NULL for none. */
+ * here and saves that launch on small problems); tile_off_b NULL for none.
+ * dense_local: the plan's -- the tokens of the chunks 0..dense_local of every sequence have no list entries (their
+ * picks in sel, if any, are ignored, and their counts are zero); 0 for the reference's lists. */
 int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, const int32_t* chunk_fb, const int32_t* chunk_local,
                      const int32_t* pair_off, int32_t* cnt, int32_t* seg_off, int32_t* tile_off, int32_t* seg_dest,
                      int32_t* tile_seg, int64_t S, int H, int K, int N, int F, int P, int cmax, int tile_rows,
                      int64_t hist_bound, int counted, int tile_rows_b, int32_t* tile_off_b, int32_t* tile_seg_b,
-                     int64_t hist_bound_b, void* stream);
+                     int64_t hist_bound_b, int dense_local, void* stream);
 
 /* The tile tables of moba_build_lists alone, for another tile height: the forward and the backward kernels cut
  * the same gather lists into tiles of moba_fwd_tile_rows() and moba_bwd_tile_rows() rows.  No counterpart in the
@@ -188,8 +207,10 @@ int moba_tile_tables(const int32_t* seg_off, int32_t* tile_off, int32_t* tile_se
  *              parts as further slots (part g of a slot row lies S*H*(K+1) rows behind part g-1).  Refused
  *              (MOBA_ERR_ARG) for problems large enough for the resident-workgroup kernel or when B is not a
  *              multiple of 64*key_split.  The same value goes to moba_fwd_partials and moba_fwd_merge.
- *   self_tile_prefix [N+1] int32: prefix sum of ceil(chunk_len / moba_fwd_tile_rows())
- *   self_tile_chunk [self_tile_prefix[N]] int32: the chunk of each of those tiles
+ *   chunk_tok [N+1], N: the attention chunks (the plan's achunk_tok and NA; the chunks themselves without dense
+ *              prefixes): the rows of one attend its keys causally, in tiles of moba_fwd_tile_rows() rows
+ *   self_tile_prefix [N+1] int32: prefix sum of ceil(attention chunk length / moba_fwd_tile_rows())
+ *   self_tile_chunk [self_tile_prefix[N]] int32: the attention chunk of each of those tiles
  *   tile_off, tile_seg: from moba_build_lists or moba_tile_tables with tile_rows = moba_fwd_tile_rows()
  *              (may be NULL when K = 0)
  *   out [S,H,D] elem, lse [S,H] fp32 (natural log)
@@ -219,6 +240,9 @@ int moba_fwd_partials(const void* q, const void* k, const void* v, void* part_o,
 int moba_fwd_merge(const void* part_o, const float* part_lse, const int32_t* sel, void* out, float* lse, int64_t S,
                    int H, int D, int K, int key_split, int dtype, void* stream);
 int moba_fwd_key_split(int64_t S, int H, int K, int B, int64_t hist_bound, int64_t self_tiles);
+/* 1 if moba_fwd_partials would run a problem of hist_bound + self_tiles * H tiles with resident workgroups drawing
+ * from the tile queues, 0 if with one workgroup per tile (no counterpart in the reference). */
+int moba_fwd_is_queued(int64_t hist_bound, int64_t self_tiles, int H);
 int moba_fwd(const void* q, const void* k, const void* v, void* part_o, float* part_lse, const int32_t* sel,
              const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest, const int32_t* fchunk_tok,
              const int32_t* chunk_tok, const int32_t* self_tile_prefix, const int32_t* tile_seg,
@@ -230,9 +254,14 @@ int moba_fwd(const void* q, const void* k, const void* v, void* part_o, float* p
  * autograd scatter of its gathered gradients.  Deterministic (no floating-point atomics).
  *   dout, q, out, dq [S,H,D] elem; k, v, dk, dv [S,Hkv,D] elem; lse [S,H] fp32 from the forward
  *   (`strides` applies to q, k, v; dout, out, dq, dk, dv are packed)
- *   tile_off, tile_seg, self_tile_prefix, self_tile_chunk, hist_bound, self_tiles: as in moba_fwd_partials, but for
- *   tiles of moba_bwd_tile_rows() rows (moba_tile_tables makes the first two from seg_off)
- *   chunk_fid [N] int32: filtered id of each chunk, -1 for the last chunk of a sequence
+ *   tile_off, tile_seg, chunk_tok, self_tile_prefix, self_tile_chunk, hist_bound, self_tiles, N: as in
+ *   moba_fwd_partials (attention chunks), but for tiles of moba_bwd_tile_rows() rows (moba_tile_tables makes the
+ *   first two from seg_off)
+ *   chunk_fid [chunks] int32: filtered id of each chunk, -1 for the last chunk of a sequence
+ *   kv_chunk_tok [chunks+1] (the plan's chunk_tok), kv_tile_prefix [chunks+1], kv_tile_chunk [kv_tiles],
+ *   chunk_self_end [chunks], kv_tiles: the key tiles of the dK/dV kernel, moba_bwd_tile_rows() keys of one chunk
+ *   each; the rows that attend a chunk's keys causally end at token chunk_self_end (the end of the chunk, or of
+ *   the dense prefix it belongs to), the others come from the chunk's gather list
  *   delta [2,S,H] fp32 scratch (rowsum(dO*O), then the LSE in the log2 domain); part_dq [dq_key_split*S*H*(K+1), D]
  *   elem scratch (the per-slot dQ, rounded as the per-chunk dQ that flash-attn returns to the reference is)
  *   dq_key_split: 1, or for small problems the power of two (up to 8) that moba_bwd_dq_key_split() names: the dQ
@@ -241,20 +270,22 @@ int moba_fwd(const void* q, const void* k, const void* v, void* part_o, float* p
  *              of 64 * dq_key_split (MOBA_ERR_ARG otherwise).
  *   dq, dk, dv: out; dk and dv of a key/value head sum over its query heads
  *   queues [16] int32 scratch: tile counters of the dQ and dK/dV kernels (as in moba_fwd_partials)
- *   dkv_scratch: moba_bwd_dkv_scratch_bytes(S, Hkv, self_tiles) bytes, 16-byte aligned, or null.  With few key tiles
+ *   dkv_scratch: moba_bwd_dkv_scratch_bytes(S, Hkv, kv_tiles) bytes, 16-byte aligned, or null.  With few key tiles
  *              (fewer than two per compute unit, S >= 4096) the dK/dV kernel cuts each into up to 4 parts that run
  *              side by side and leave fp32 sums there, added up in a fixed order (deterministic all the same);
  *              without the scratch, or when the query returns 0, every tile is one piece.
  *   softmax_scale: as in the forward call */
-size_t moba_bwd_dkv_scratch_bytes(int64_t S, int Hkv, int64_t self_tiles);
+size_t moba_bwd_dkv_scratch_bytes(int64_t S, int Hkv, int64_t kv_tiles);
 int moba_bwd_dq_key_split(int64_t S, int H, int K, int B, int64_t hist_bound, int64_t self_tiles);
 int moba_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out, const float* lse,
              const int32_t* sel, const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest,
              const int32_t* fchunk_tok, const int32_t* chunk_tok, const int32_t* self_tile_prefix,
-             const int32_t* tile_seg, const int32_t* self_tile_chunk, const int32_t* chunk_fid, float* delta,
-             void* part_dq, void* dq, void* dk, void* dv, int64_t S, int H, int Hkv, int D, int K, int F, int N, int B,
-             int64_t hist_bound, int64_t self_tiles, int dq_key_split, const int64_t* strides, int32_t* queues,
-             void* dkv_scratch, int64_t dkv_scratch_bytes, float softmax_scale, int dtype, void* stream);
+             const int32_t* tile_seg, const int32_t* self_tile_chunk, const int32_t* chunk_fid,
+             const int32_t* kv_chunk_tok, const int32_t* kv_tile_prefix, const int32_t* kv_tile_chunk,
+             const int32_t* chunk_self_end, float* delta, void* part_dq, void* dq, void* dk, void* dv, int64_t S, int H,
+             int Hkv, int D, int K, int F, int N, int B, int64_t hist_bound, int64_t self_tiles, int64_t kv_tiles,
+             int dq_key_split, const int64_t* strides, int32_t* queues, void* dkv_scratch, int64_t dkv_scratch_bytes,
+             float softmax_scale, int dtype, void* stream);
 
 /* Decode: one query token per sequence against the key/value cache.  Replaces the
  * flash_attn_func call of the adapter's decode branch, moba/wrapper.py:76-82 (full attention

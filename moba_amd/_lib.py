@@ -21,8 +21,8 @@ _lib = None
 _SIGNATURES = {
     "moba_version": (c_int, []),
     "moba_strerror": (c_char_p, [c_int]),
-    "moba_plan": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p]),
-    "moba_plan_fill": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p]),
+    "moba_plan": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
+    "moba_plan_fill": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
     "moba_plan_sizes": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p]),
     "moba_chunk_mean_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "moba_chunk_mean": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_strides,
@@ -31,10 +31,11 @@ _SIGNATURES = {
     "moba_chunk_mean_static": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_strides,
                                        c_int, c_void_p]),
     "moba_gate_topk": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                               c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_strides, c_int, c_void_p]),
+                               c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_strides, c_int,
+                               c_void_p]),
     "moba_topk_from_scores": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_void_p]),
     "moba_build_lists": (c_int, [c_void_p] * 10 + [c_int64] + [c_int] * 7 + [c_int64, c_int, c_int, c_void_p, c_void_p,
-                                                                             c_int64, c_void_p]),
+                                                                             c_int64, c_int, c_void_p]),
     "moba_tile_tables": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int64, c_void_p]),
     "moba_fwd_tile_rows": (c_int, []),
     "moba_bwd_tile_rows": (c_int, []),
@@ -43,12 +44,13 @@ _SIGNATURES = {
                                                    c_void_p]),
     "moba_fwd_merge": (c_int, [c_void_p] * 5 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "moba_fwd_key_split": (c_int, [c_int64, c_int, c_int, c_int, c_int64, c_int64]),
+    "moba_fwd_is_queued": (c_int, [c_int64, c_int64, c_int]),
     "moba_fwd": (c_int, [c_void_p] * 16 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_int64,
                                           c_int, c_strides, c_void_p, c_void_p, c_float, c_int, c_void_p]),
     "moba_bwd_dkv_scratch_bytes": (ctypes.c_size_t, [c_int64, c_int, c_int64]),
     "moba_bwd_dq_key_split": (c_int, [c_int64, c_int, c_int, c_int, c_int64, c_int64]),
-    "moba_bwd": (c_int, [c_void_p] * 21 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_int64,
-                                          c_int, c_strides, c_void_p, c_void_p, c_int64, c_float, c_int, c_void_p]),
+    "moba_bwd": (c_int, [c_void_p] * 25 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_int64,
+                                          c_int64, c_int, c_strides, c_void_p, c_void_p, c_int64, c_float, c_int, c_void_p]),
     "moba_decode_splits": (c_int, [c_int, c_int, c_int]),
     "moba_decode": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_int64] * 4 + [c_float, c_int, c_void_p]),
 }
@@ -58,12 +60,13 @@ OPTIONAL = set()
 class PlanStruct(ctypes.Structure):
     """moba_plan_t of include/moba_hip.h."""
     _fields_ = ([("S", c_int64)] + [(n, ctypes.c_int32) for n in ("nseq", "chunk", "topk", "N", "F", "K", "P", "cmax", "fallback",
-                                                               "fwd_tile_rows", "bwd_tile_rows")]
+                                                               "fwd_tile_rows", "bwd_tile_rows", "dense_local", "NA")]
                 + [("pairs_per_head", c_int64), ("fwd_self_tiles", c_int64), ("bwd_self_tiles", c_int64),
-                   ("flops_per_head_per_dim", ctypes.c_double)]
-                + [("off_" + n, c_int64) for n in ("cu_seqlens", "chunk_tok", "fwd_self_tile_prefix", "fwd_self_tile_chunk",
-                                                   "self_tile_prefix", "self_tile_chunk", "seq_fbase", "fchunk_tok", "chunk_fb",
-                                                   "chunk_local", "pair_off", "chunk_fid")]
+                   ("kv_tiles", c_int64), ("flops_per_head_per_dim", ctypes.c_double)]
+                + [("off_" + n, c_int64) for n in ("cu_seqlens", "chunk_tok", "achunk_tok", "fwd_self_tile_prefix",
+                                                   "fwd_self_tile_chunk", "self_tile_prefix", "self_tile_chunk",
+                                                   "kv_tile_prefix", "kv_tile_chunk", "chunk_self_end", "seq_fbase",
+                                                   "fchunk_tok", "chunk_fb", "chunk_local", "pair_off", "chunk_fid")]
                 + [("table_ints", c_int64)])
 
 
@@ -72,7 +75,7 @@ class SizesStruct(ctypes.Structure):
     _fields_ = [(n, c_int64) for n in ("kbar_elems", "chunk_mean_workspace_bytes", "sel_ints", "cnt_ints", "seg_off_ints",
                                        "seg_dest_ints", "fwd_hist_bound", "bwd_hist_bound", "part_rows", "redo_ints",
                                        "lse_floats", "delta_floats")]
-ABI_VERSION = 111  # MOBA_ABI_VERSION of include/moba_hip.h, the signatures above
+ABI_VERSION = 112  # MOBA_ABI_VERSION of include/moba_hip.h, the signatures above
 DTYPE_BF16, DTYPE_F16 = 0, 1
 
 

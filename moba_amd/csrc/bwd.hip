@@ -48,6 +48,14 @@ struct BwdParams {
   typename E::elem* dk;
   typename E::elem* dv;
   const int* chunk_fid;  // [N] filtered id of a chunk, -1 for the last chunk of a sequence
+  // The key tiles of the dK/dV kernel: TM keys of one chunk and key/value head.  The rows that attend them
+  // causally run from the tile's first key to chunk_self_end (the end of the chunk, or of the dense prefix the
+  // chunk belongs to); the rows beyond come from the chunk's gather list.
+  const int* kv_chunk_tok;    // [N+1] first token of every chunk
+  const int* kv_tile_prefix;  // [N+1] prefix sum of ceil(chunk length / TM)
+  const int* kv_tile_chunk;   // [kv_tile_prefix[N]] chunk of every such tile
+  const int* chunk_self_end;  // [N]
+  int kv_total;               // kv_tile_prefix[N] * Hkv
   TileTables t;
   float scale_log2;
   float scale;
@@ -64,21 +72,23 @@ struct BwdParams {
   int queues_log2;
 };
 
-// which 128-key tile of which key/value head: the forward's self-tile enumeration over Hkv heads
+// which 128-key tile of which key/value head: the forward's self-tile enumeration over the chunks and Hkv heads
 struct KvTile {
   int c, hkv, key0, c0, len;  // chunk, key/value head, first key inside the chunk, first token and length of the chunk
+  int self_len;               // the rows that attend the chunk's keys causally end this far behind c0 (>= len)
 };
 template <class E>
 __device__ __forceinline__ KvTile decode_kv_tile(const BwdParams<E>& p, int st) {
   const int Hkv = p.t.Hkv;
   KvTile t;
-  t.c = p.t.self_tile_chunk[st / Hkv];
-  const int rem = st - p.t.self_tile_prefix[t.c] * Hkv;
-  const int nt = p.t.self_tile_prefix[t.c + 1] - p.t.self_tile_prefix[t.c];
+  t.c = p.kv_tile_chunk[st / Hkv];
+  const int rem = st - p.kv_tile_prefix[t.c] * Hkv;
+  const int nt = p.kv_tile_prefix[t.c + 1] - p.kv_tile_prefix[t.c];
   t.hkv = rem / nt;
   t.key0 = (rem - t.hkv * nt) * TM;
-  t.c0 = p.t.chunk_tok[t.c];
-  t.len = p.t.chunk_tok[t.c + 1] - t.c0;
+  t.c0 = p.kv_chunk_tok[t.c];
+  t.len = p.kv_chunk_tok[t.c + 1] - t.c0;
+  t.self_len = p.chunk_self_end[t.c] - t.c0;
   return t;
 }
 
@@ -493,7 +503,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
   const int drawn = __builtin_amdgcn_readfirstlane(*reinterpret_cast<const int*>(smem + kDkvIdSlot));
   const int64_t id = (((int64_t)(drawn / kXcdBlock) << ql) + queue) * kXcdBlock + (drawn % kXcdBlock);
   const int split = p.dkv_split;
-  if (id >= (int64_t)(p.t.self_total / rep) * split) {
+  if (id >= (int64_t)p.kv_total * split) {
     queue = (queue + 1) & qmask;
     if (++empty_queues > qmask) break;
     continue;
@@ -507,8 +517,8 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv_kernel(const BwdParams<E> p) {
   const int mykey = key0 + wave * 32 + n;        // position inside the chunk
   const bool key_valid = mykey < len;
 
-  // ---- the rows that attend these keys: causal rows of the chunk, then the gather list ----
-  const int self_rows = len - key0;              // chunk positions key0 .. len-1
+  // ---- the rows that attend these keys: the causal rows (of the chunk, or of its dense prefix), then the gather list ----
+  const int self_rows = kt.self_len - key0;      // chunk positions key0 .. self_len-1
   const int nself = (self_rows + TQ - 1) / TQ;
   const int fid = (p.chunk_fid && K1 > 1) ? p.chunk_fid[c] : -1;
   // the query heads of this key/value head are walked one after the other; per head:
@@ -884,8 +894,9 @@ using namespace moba;
 
 template <class E>
 static int launch_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out, const float* lse,
-                      const int32_t* sel, const int32_t* chunk_fid, float* delta, void* part_dq, void* dq, void* dk,
-                      void* dv, const TileTables& t, int64_t S, int H, int D, int K, float softmax_scale, int64_t grid_q,
+                      const int32_t* sel, const int32_t* chunk_fid, const int32_t* kv_chunk_tok,
+                      const int32_t* kv_tile_prefix, const int32_t* kv_tile_chunk, const int32_t* chunk_self_end,
+                      int kv_total, float* delta, void* part_dq, void* dq, void* dk, void* dv, const TileTables& t, int64_t S, int H, int D, int K, float softmax_scale, int64_t grid_q,
                       int64_t grid_kv, int* queues, float* part_dkv, int dkv_split, hipStream_t st) {
   LaunchCheck launch_check;
   typedef typename E::elem elem;
@@ -893,6 +904,8 @@ static int launch_bwd(const void* dout, const void* q, const void* k, const void
   p.q = (const elem*)q; p.k = (const elem*)k; p.v = (const elem*)v; p.dout = (const elem*)dout;
   p.lse = lse; p.delta = delta; p.lse2 = delta + S * H; p.part_dq = (elem*)part_dq; p.dk = (elem*)dk; p.dv = (elem*)dv;
   p.chunk_fid = chunk_fid;
+  p.kv_chunk_tok = kv_chunk_tok; p.kv_tile_prefix = kv_tile_prefix; p.kv_tile_chunk = kv_tile_chunk;
+  p.chunk_self_end = chunk_self_end; p.kv_total = kv_total;
   p.queues = queues;
   p.part_dkv = part_dkv;
   p.dkv_split = dkv_split;
@@ -925,7 +938,7 @@ static int launch_bwd(const void* dout, const void* q, const void* k, const void
   if (batched) hipLaunchKernelGGL((bwd_dkv_kernel<E, true>), dim3((unsigned)grid_kv), dim3(256), kBwdDkvLds, st, p);
   else hipLaunchKernelGGL((bwd_dkv_kernel<E, false>), dim3((unsigned)grid_kv), dim3(256), kBwdDkvLds, st, p);
   if (dkv_split > 1)
-    hipLaunchKernelGGL(bwd_dkv_reduce_kernel<E>, dim3((unsigned)(t.self_total / t.rep) * 16), dim3(256), 0, st, p);
+    hipLaunchKernelGGL(bwd_dkv_reduce_kernel<E>, dim3((unsigned)p.kv_total * 16), dim3(256), 0, st, p);
   return launch_check.result();
 }
 
@@ -942,9 +955,9 @@ static int dkv_split_for(int64_t S, int64_t tiles) {
   return (int)(r < 1 ? 1 : (r > 4 ? 4 : r));
 }
 
-extern "C" size_t moba_bwd_dkv_scratch_bytes(int64_t S, int Hkv, int64_t self_tiles) {
-  if (S <= 0 || Hkv <= 0 || self_tiles <= 0) return 0;
-  const int64_t tiles = self_tiles * Hkv;
+extern "C" size_t moba_bwd_dkv_scratch_bytes(int64_t S, int Hkv, int64_t kv_tiles) {
+  if (S <= 0 || Hkv <= 0 || kv_tiles <= 0) return 0;
+  const int64_t tiles = kv_tiles * Hkv;
   const int split = dkv_split_for(S, tiles);
   return split > 1 ? (size_t)tiles * split * (2 * TM * kHeadDim) * sizeof(float) : 0;
 }
@@ -967,18 +980,20 @@ extern "C" int moba_bwd(const void* dout, const void* q, const void* k, const vo
                         const float* lse, const int32_t* sel, const int32_t* seg_off, const int32_t* tile_off,
                         const int32_t* seg_dest, const int32_t* fchunk_tok, const int32_t* chunk_tok,
                         const int32_t* self_tile_prefix, const int32_t* tile_seg, const int32_t* self_tile_chunk,
-                        const int32_t* chunk_fid, float* delta, void* part_dq,
+                        const int32_t* chunk_fid, const int32_t* kv_chunk_tok, const int32_t* kv_tile_prefix,
+                        const int32_t* kv_tile_chunk, const int32_t* chunk_self_end, float* delta, void* part_dq,
                         void* dq, void* dk, void* dv, int64_t S, int H, int Hkv, int D, int K, int F, int N, int B,
-                        int64_t hist_bound, int64_t self_tiles, int dq_key_split, const int64_t* strides,
+                        int64_t hist_bound, int64_t self_tiles, int64_t kv_tiles, int dq_key_split, const int64_t* strides,
                         int32_t* queues, void* dkv_scratch, int64_t dkv_scratch_bytes, float softmax_scale, int dtype,
                         void* stream) {
   if (!dout || !q || !k || !v || !out || !lse || !chunk_tok || !self_tile_prefix || !self_tile_chunk || !delta ||
-      !part_dq || !dq || !dk || !dv || !queues)
+      !part_dq || !dq || !dk || !dv || !queues || !kv_chunk_tok || !kv_tile_prefix || !kv_tile_chunk || !chunk_self_end)
     return MOBA_ERR_ARG;
   if (K > 0 && (!sel || !seg_off || !tile_off || !seg_dest || !fchunk_tok || !chunk_fid || !tile_seg))
     return MOBA_ERR_ARG;
   if (D != kHeadDim || (dtype != MOBA_DTYPE_BF16 && dtype != MOBA_DTYPE_F16)) return MOBA_ERR_UNSUPPORTED;
-  if (S <= 0 || H <= 0 || K < 0 || F < 0 || N <= 0 || B <= 0 || hist_bound < 0 || self_tiles <= 0) return MOBA_ERR_ARG;
+  if (S <= 0 || H <= 0 || K < 0 || F < 0 || N <= 0 || B <= 0 || hist_bound < 0 || self_tiles <= 0 || kv_tiles <= 0)
+    return MOBA_ERR_ARG;
   if (Hkv <= 0 || H % Hkv != 0) return MOBA_ERR_ARG;
   const void* ptrs[] = {dout, q, k, v, out, part_dq, dq, dk, dv};
   for (const void* x : ptrs)
@@ -1007,16 +1022,18 @@ extern "C" int moba_bwd(const void* dout, const void* q, const void* k, const vo
   while ((1 << t.key_split_log2) < dq_key_split) ++t.key_split_log2;
   t.part_stride = (int)(S * H * (K + 1));
   // the key tiles are cut into parts only if the caller brought the scratch for their sums
-  const int64_t kv_tiles = self_tiles * Hkv;
-  int dkv_split = dkv_split_for(S, kv_tiles);
+  const int64_t kv_total = kv_tiles * Hkv;
+  int dkv_split = dkv_split_for(S, kv_total);
   if (dkv_split > 1 && (!dkv_scratch || ((uintptr_t)dkv_scratch & 15) ||
-                        dkv_scratch_bytes < (int64_t)(kv_tiles * dkv_split * (2 * TM * kHeadDim) * sizeof(float))))
+                        dkv_scratch_bytes < (int64_t)(kv_total * dkv_split * (2 * TM * kHeadDim) * sizeof(float))))
     dkv_split = 1;
-  if (kv_tiles * dkv_split >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
+  if (kv_total * dkv_split >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
   hipStream_t st = (hipStream_t)stream;
   return dtype == MOBA_DTYPE_F16
-             ? launch_bwd<F16>(dout, q, k, v, out, lse, sel, chunk_fid, delta, part_dq, dq, dk, dv, t, S, H, D, K,
+             ? launch_bwd<F16>(dout, q, k, v, out, lse, sel, chunk_fid, kv_chunk_tok, kv_tile_prefix, kv_tile_chunk,
+                               chunk_self_end, (int)kv_total, delta, part_dq, dq, dk, dv, t, S, H, D, K,
                                softmax_scale, grid_q, grid_kv, queues, (float*)dkv_scratch, dkv_split, st)
-             : launch_bwd<Bf16>(dout, q, k, v, out, lse, sel, chunk_fid, delta, part_dq, dq, dk, dv, t, S, H, D, K,
+             : launch_bwd<Bf16>(dout, q, k, v, out, lse, sel, chunk_fid, kv_chunk_tok, kv_tile_prefix, kv_tile_chunk,
+                                chunk_self_end, (int)kv_total, delta, part_dq, dq, dk, dv, t, S, H, D, K,
                                 softmax_scale, grid_q, grid_kv, queues, (float*)dkv_scratch, dkv_split, st);
 }

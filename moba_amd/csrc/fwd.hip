@@ -787,6 +787,15 @@ static int64_t fwd_grid(int64_t total, int cus) {
   }
   return grid;
 }
+// Whether moba_fwd_partials would run a problem of this many tiles with resident workgroups that draw their tiles
+// from the queues (1) or with one workgroup per tile (0).  A caller that may plan a batch with or without dense
+// prefixes asks this for the plan with them: their long causal tiles pay only in the first form.
+extern "C" int moba_fwd_is_queued(int64_t hist_bound, int64_t self_tiles, int H) {
+  const int cus = resident_compute_units();
+  if (cus <= 0 || hist_bound < 0 || self_tiles < 0 || H <= 0) return 0;
+  return fwd_grid(hist_bound + self_tiles * H, cus) > 0 ? 1 : 0;
+}
+
 // Into how many parts moba_fwd_partials should cut the keys of every history tile: 1 unless the problem is so
 // small that whole tiles leave compute units idle at the end (a tile of 256 rows x 2048 keys takes 65 us, and
 // workgroups start in the order of their ids, not where the work is); then the largest power of two that

@@ -6,7 +6,9 @@
 // filtered-chunk ids are [fb, fb + c) with fb the first filtered id of the
 // sequence.  The K best are kept; ties go to the lower chunk id; a -inf or NaN
 // score is never picked.  Output sel[s, h, 0..K) holds filtered-chunk ids in
-// descending score order, -1 padded.
+// descending score order, -1 padded.  With dense_local = d > 0 the tokens of the
+// chunks 0..d of every sequence (which would pick every earlier chunk) get no picks
+// at all: the attention kernels serve them through one causal pass over the prefix.
 //
 // One wave handles 64 consecutive tokens of one head: the score tile
 // (32 chunks x 64 tokens) is two 32x32x16 MFMA accumulators, staged through LDS
@@ -56,7 +58,7 @@ __global__ __launch_bounds__(256) void gate_topk_kernel(
     const typename E::elem* __restrict__ q, const typename E::elem* __restrict__ kbar, const int* __restrict__ cu_seqlens,
     const int* __restrict__ seq_fbase, int* __restrict__ sel, float* __restrict__ scores_out,
     int S, int H, int Hkv, int nseq, int F, int B, int K, int64_t q_tok_stride, int64_t q_head_stride,
-    int batch_rows, int64_t q_batch_stride, const int* __restrict__ pair_off, int* __restrict__ cnt) {
+    int batch_rows, int64_t q_batch_stride, const int* __restrict__ pair_off, int* __restrict__ cnt, int dense_local) {
   MOBA_ELEM_TYPES(E)
   __shared__ float sc[4][64][33];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -73,6 +75,8 @@ __global__ __launch_bounds__(256) void gate_topk_kernel(
     const int b = find_seq(cu_seqlens, nseq, s);
     fb = seq_fbase[b];
     c = (s - cu_seqlens[b]) / B;
+    // a token of a dense prefix attends all its earlier chunks through the causal self path: no picks, no counts
+    if (c <= dense_local) c = 0;
   }
   // union of the candidate ranges of the 64 tokens (identical for the 4 waves)
   int flo = c > 0 ? fb : 0x7fffffff;
@@ -225,13 +229,14 @@ using namespace moba;
 
 extern "C" int moba_gate_topk(const void* q, const void* kbar, const int32_t* cu_seqlens, const int32_t* seq_fbase,
                               int32_t* sel, float* scores_out, const int32_t* pair_off, int32_t* cnt, int64_t S, int H,
-                              int Hkv, int D, int nseq, int F, int B, int K, const int64_t* strides, int dtype,
-                              void* stream) {
+                              int Hkv, int D, int nseq, int F, int B, int K, int dense_local, const int64_t* strides,
+                              int dtype, void* stream) {
   LaunchCheck launch_check;
   if (!q || !kbar || !cu_seqlens || !seq_fbase || !sel || (cnt && !pair_off)) return MOBA_ERR_ARG;
   if (Hkv <= 0 || H % Hkv != 0) return MOBA_ERR_ARG;
   if (dtype != MOBA_DTYPE_BF16 && dtype != MOBA_DTYPE_F16) return MOBA_ERR_UNSUPPORTED;
   if (S <= 0 || S > 0x7fffffff - 64 || H <= 0 || nseq <= 0 || F <= 0 || B <= 0 || K <= 0) return MOBA_ERR_ARG;
+  if (dense_local < 0 || dense_local > K) return MOBA_ERR_ARG;
   if (D != kHeadDim) return MOBA_ERR_UNSUPPORTED;
   if (((uintptr_t)q & 15) || ((uintptr_t)kbar & 15)) return MOBA_ERR_ARG;
   // strides (elements): {q token, q head, ., ., rows per batch entry, q batch, .}; null = packed [S, H, 128]
@@ -246,11 +251,11 @@ extern "C" int moba_gate_topk(const void* q, const void* kbar, const int32_t* cu
   if (dtype == MOBA_DTYPE_F16)                                                                                 \
     hipLaunchKernelGGL((gate_topk_kernel<F16, KM>), grid, dim3(256), 0, st, (const f16*)q, (const f16*)kbar,   \
                        cu_seqlens, seq_fbase, sel, scores_out, (int)S, H, Hkv, nseq, F, B, K, qts, qhs, qbr, qbs, \
-                       pair_off, cnt);                                                                         \
+                       pair_off, cnt, dense_local);                                                            \
   else                                                                                                         \
     hipLaunchKernelGGL((gate_topk_kernel<Bf16, KM>), grid, dim3(256), 0, st, (const bf16*)q, (const bf16*)kbar, \
                        cu_seqlens, seq_fbase, sel, scores_out, (int)S, H, Hkv, nseq, F, B, K, qts, qhs, qbr, qbs, \
-                       pair_off, cnt)
+                       pair_off, cnt, dense_local)
   MOBA_DISPATCH_K(K, CALL)
 #undef CALL
   return launch_check.result();

@@ -29,12 +29,17 @@ __device__ __forceinline__ int cnt_index(const int* __restrict__ pair_off, int f
 template <int NT>  // threads per workgroup
 __global__ __launch_bounds__(NT) void lists_count_kernel(
     const int* __restrict__ sel, const int* __restrict__ chunk_tok, const int* __restrict__ chunk_fb,
-    const int* __restrict__ chunk_local, const int* __restrict__ pair_off, int* __restrict__ cnt, int H, int K) {
+    const int* __restrict__ chunk_local, const int* __restrict__ pair_off, int* __restrict__ cnt, int H, int K,
+    int dense_local) {
   extern __shared__ int lds[];
   const int cq = blockIdx.x, h = blockIdx.y;
   const int c = chunk_local[cq];
   if (c == 0) return;
   const int fb = chunk_fb[cq];
+  if (c <= dense_local) {  // a chunk of a dense prefix: its tokens have no list entries, its counts are zero
+    for (int i = threadIdx.x; i < c; i += NT) cnt[cnt_index(pair_off, fb + i, h, H, c - i - 1)] = 0;
+    return;
+  }
   const int t0 = chunk_tok[cq], t1 = chunk_tok[cq + 1];
   for (int i = threadIdx.x; i < c; i += NT) lds[i] = 0;
   __syncthreads();
@@ -64,9 +69,10 @@ template <int KC, int NW, class BaseFn>
 __device__ __forceinline__ void lists_fill_body(
     const int* __restrict__ sel, const int* __restrict__ chunk_tok, const int* __restrict__ chunk_fb,
     const int* __restrict__ chunk_local, const int* __restrict__ pair_off, BaseFn base_of,
-    int* __restrict__ seg_dest, int H, int K, int* lds) {
+    int* __restrict__ seg_dest, int H, int K, int dense_local, int* lds) {
   const int cq = blockIdx.x, h = blockIdx.y;
-  const int c = chunk_local[cq];
+  const int c_real = chunk_local[cq];
+  const int c = c_real > dense_local ? c_real : 0;  // (no list entries from a chunk of a dense prefix)
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   int* pos = lds;                                             // [NW][c] running list position per wave
   unsigned* bits = reinterpret_cast<unsigned*>(lds + NW * c);  // [NW][c][2] lanes of the batch that picked i
@@ -174,9 +180,10 @@ template <int KC>
 __global__ __launch_bounds__(256) void lists_fill_kernel(
     const int* __restrict__ sel, const int* __restrict__ chunk_tok, const int* __restrict__ chunk_fb,
     const int* __restrict__ chunk_local, const int* __restrict__ pair_off, const int* __restrict__ base,
-    int* __restrict__ seg_dest, int H, int K) {
+    int* __restrict__ seg_dest, int H, int K, int dense_local) {
   extern __shared__ int lds[];
-  lists_fill_body<KC, 4>(sel, chunk_tok, chunk_fb, chunk_local, pair_off, [&] { return base; }, seg_dest, H, K, lds);
+  lists_fill_body<KC, 4>(sel, chunk_tok, chunk_fb, chunk_local, pair_off, [&] { return base; }, seg_dest, H, K,
+                         dense_local, lds);
 }
 
 // exclusive prefix sum of a[0..n) in place, total stored at a[n]; one workgroup.
@@ -356,7 +363,7 @@ __global__ __launch_bounds__(1024) void lists_fill_tail_kernel(
     const int* __restrict__ chunk_local, const int* __restrict__ pair_off, const int* __restrict__ cnt,
     int* __restrict__ seg_dest, int* __restrict__ seg_off, int* __restrict__ tile_off, int* __restrict__ tile_seg,
     int N, int H, int K, int F, int PH, int tile_rows, int bound, int tile_rows_b, int* __restrict__ tile_off_b,
-    int* __restrict__ tile_seg_b, int bound_b) {
+    int* __restrict__ tile_seg_b, int bound_b, int dense_local) {
   __shared__ int sbase[kFusedMaxCounts + 1];
   // the tail's tile starts, or the fill's positions and lane masks: 16 waves x 3 ints per candidate chunk
   __shared__ int off[kFusedMaxCand * 48 > kTailMaxSegments + 1 ? kFusedMaxCand * 48 : kTailMaxSegments + 1];
@@ -402,7 +409,8 @@ __global__ __launch_bounds__(1024) void lists_fill_tail_kernel(
       lists_tail_body(base, pair_off, seg_off, tile_off_b, tile_seg_b, F, H, tile_rows_b, bound_b, off, wsum);
     }
   } else
-    lists_fill_body<KC, 16>(sel, chunk_tok, chunk_fb, chunk_local, pair_off, scanned_counts, seg_dest, H, K, off);
+    lists_fill_body<KC, 16>(sel, chunk_tok, chunk_fb, chunk_local, pair_off, scanned_counts, seg_dest, H, K,
+                            dense_local, off);
 }
 
 }  // namespace moba
@@ -430,7 +438,7 @@ extern "C" int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, co
                                 int32_t* seg_off, int32_t* tile_off, int32_t* seg_dest, int32_t* tile_seg,
                                 int64_t S, int H, int K, int N, int F, int P, int cmax, int tile_rows,
                                 int64_t hist_bound, int counted, int tile_rows_b, int32_t* tile_off_b,
-                                int32_t* tile_seg_b, int64_t hist_bound_b, void* stream) {
+                                int32_t* tile_seg_b, int64_t hist_bound_b, int dense_local, void* stream) {
   LaunchCheck launch_check;
   if (!sel || !chunk_tok || !chunk_fb || !chunk_local || !pair_off || !cnt || !seg_off || !tile_off || !seg_dest ||
       !tile_seg)
@@ -439,6 +447,7 @@ extern "C" int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, co
   if (tile_off_b && (!tile_seg_b || tile_rows_b <= 0 || hist_bound_b <= 0 || hist_bound_b >= 0x7fffffffLL))
     return MOBA_ERR_ARG;
   if (S <= 0 || H <= 0 || K <= 0 || N <= 0 || F <= 0 || P <= 0 || cmax <= 0 || tile_rows <= 0) return MOBA_ERR_ARG;
+  if (dense_local < 0 || dense_local > K) return MOBA_ERR_ARG;
   if ((int64_t)S * H * (K + 1) >= 0x7fffffffLL || (int64_t)P * H >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
   if (H > 65535 || (size_t)cmax * 48 > 160 * 1024) return MOBA_ERR_LIMIT;
   hipStream_t st = (hipStream_t)stream;
@@ -448,11 +457,12 @@ extern "C" int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, co
       (!tile_off_b || hist_bound_b <= kTailMaxTiles)) {
     if (!counted)
       hipLaunchKernelGGL(lists_count_kernel<1024>, grid, dim3(1024), (size_t)cmax * 4, st, sel, chunk_tok, chunk_fb,
-                         chunk_local, pair_off, cnt, H, K);
+                         chunk_local, pair_off, cnt, H, K, dense_local);
 #define MOBA_FILL_TAIL(KC)                                                                                       \
   hipLaunchKernelGGL(lists_fill_tail_kernel<KC>, dim3(N + 1, H), dim3(1024), 0, st, sel, chunk_tok, chunk_fb,    \
                      chunk_local, pair_off, (const int*)cnt, seg_dest, seg_off, tile_off, tile_seg, N, H, K, F,  \
-                     P * H, tile_rows, (int)hist_bound, tile_rows_b, tile_off_b, tile_seg_b, (int)hist_bound_b)
+                     P * H, tile_rows, (int)hist_bound, tile_rows_b, tile_off_b, tile_seg_b, (int)hist_bound_b,     \
+                     dense_local)
     if (K <= 4) MOBA_FILL_TAIL(4);
     else MOBA_FILL_TAIL(16);
 #undef MOBA_FILL_TAIL
@@ -460,7 +470,7 @@ extern "C" int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, co
   }
   if (!counted)
     hipLaunchKernelGGL(lists_count_kernel<256>, grid, dim3(256), (size_t)cmax * 4, st, sel, chunk_tok, chunk_fb,
-                       chunk_local, pair_off, cnt, H, K);
+                       chunk_local, pair_off, cnt, H, K, dense_local);
   hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(1024), 0, st, cnt, P * H);
   // more than 64 KiB of dynamic LDS has to be asked for explicitly
 #define MOBA_FILL(KC)                                                                                          \
@@ -470,7 +480,7 @@ extern "C" int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, co
                             (int)((size_t)cmax * 48)) != hipSuccess)                                           \
       return MOBA_ERR_LAUNCH;                                                                                  \
     hipLaunchKernelGGL(lists_fill_kernel<KC>, grid, dim3(256), (size_t)cmax * 48, st, sel, chunk_tok, chunk_fb, \
-                       chunk_local, pair_off, (const int*)cnt, seg_dest, H, K);                                \
+                       chunk_local, pair_off, (const int*)cnt, seg_dest, H, K, dense_local);                   \
   }
   if (K <= 4) MOBA_FILL(4)
   else if (K <= 16) MOBA_FILL(16)

@@ -19,16 +19,20 @@ struct moba_plan_t {
   int32_t cmax;             // most chunks in a sequence minus one
   int32_t fallback;         // 1: topk - 1 <= 0 or no filtered chunk -- full causal attention, K = 0
   int32_t fwd_tile_rows, bwd_tile_rows;
-  int64_t pairs_per_head;   // selected (token, chunk) pairs per head: M = pairs_per_head * H
-  int64_t fwd_self_tiles, bwd_self_tiles;  // row tiles of the self part, per head
+  int32_t dense_local;      // chunks 0..dense_local of every sequence form one attention chunk (0: every chunk its own)
+  int32_t NA;               // attention chunks
+  int64_t pairs_per_head;   // list entries per head: M = pairs_per_head * H
+  int64_t fwd_self_tiles, bwd_self_tiles;  // row tiles of the attention chunks, per head
+  int64_t kv_tiles;         // key tiles (bwd_tile_rows keys) of the chunks, per key/value head
   double flops_per_head_per_dim;           // forward flops = this * H * head_dim
   // offsets (in int32 elements) of the tables inside the array moba_plan_fill writes, -1 = absent
-  int64_t off_cu_seqlens, off_chunk_tok, off_fwd_self_tile_prefix, off_fwd_self_tile_chunk, off_self_tile_prefix,
-      off_self_tile_chunk, off_seq_fbase, off_fchunk_tok, off_chunk_fb, off_chunk_local, off_pair_off, off_chunk_fid;
+  int64_t off_cu_seqlens, off_chunk_tok, off_achunk_tok, off_fwd_self_tile_prefix, off_fwd_self_tile_chunk,
+      off_self_tile_prefix, off_self_tile_chunk, off_kv_tile_prefix, off_kv_tile_chunk, off_chunk_self_end,
+      off_seq_fbase, off_fchunk_tok, off_chunk_fb, off_chunk_local, off_pair_off, off_chunk_fid;
   int64_t table_ints;       // length of that array
 };
 
-static int plan_core(const int32_t* cu, int nseq, int chunk, int topk, moba_plan_t* pl, int32_t* tab) {
+static int plan_core(const int32_t* cu, int nseq, int chunk, int topk, int dense, moba_plan_t* pl, int32_t* tab) {
   if (!cu || !pl || nseq <= 0 || chunk <= 0 || topk <= 0) return MOBA_ERR_ARG;
   if (cu[0] != 0) return MOBA_ERR_ARG;
   for (int b = 0; b < nseq; ++b)
@@ -50,33 +54,48 @@ static int plan_core(const int32_t* cu, int nseq, int chunk, int topk, moba_plan
   if (nchunks >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
   p.N = (int32_t)nchunks; p.F = (int32_t)F; p.cmax = cmax;
   p.K = p.fallback ? 0 : (int32_t)std::min<int64_t>(k_eff, cmax);
+  const int d = dense ? p.K : 0;
+  p.dense_local = d;
 
   // first pass over the chunks: tile counts, pair counts, flops
-  int64_t ftiles = 0, btiles = 0, pairs = 0, pairs_self = 0, P = 0;
+  int64_t ftiles = 0, btiles = 0, ktiles = 0, pairs = 0, pairs_all = 0, pairs_self = 0, P = 0, NA = 0;
+  auto add_achunk = [&](int64_t alen) {
+    ftiles += (alen + kFwdTileRows - 1) / kFwdTileRows;
+    btiles += (alen + TM - 1) / TM;
+    ++NA;
+  };
   for (int b = 0; b < nseq; ++b) {
     const int64_t len = (int64_t)cu[b + 1] - cu[b];
     const int64_t n = p.fallback ? 1 : (len + chunk - 1) / chunk;
+    int64_t alen = 0;  // length of the attention chunk being put together
     for (int64_t c = 0; c < n; ++c) {
       const int64_t clen = p.fallback ? len : std::min<int64_t>(chunk, len - c * chunk);
-      ftiles += (clen + kFwdTileRows - 1) / kFwdTileRows;
-      btiles += (clen + TM - 1) / TM;
+      if (c > d) { add_achunk(alen); alen = 0; }
+      alen += clen;
+      ktiles += (clen + TM - 1) / TM;
       pairs_self += clen * (clen + 1) / 2;
-      pairs += clen * std::min<int64_t>(p.K, c);
+      pairs_all += clen * std::min<int64_t>(p.K, c);
+      if (c > d) pairs += clen * std::min<int64_t>(p.K, c);
       if (!p.fallback && c < n - 1) P += n - 1 - c;
     }
+    add_achunk(alen);
   }
-  if (P >= 0x7fffffffLL || ftiles >= 0x7fffffffLL || btiles >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
-  p.fwd_self_tiles = ftiles; p.bwd_self_tiles = btiles; p.pairs_per_head = pairs; p.P = (int32_t)P;
-  p.flops_per_head_per_dim = 4.0 * ((double)pairs_self + (double)pairs * chunk);
+  if (P >= 0x7fffffffLL || ftiles >= 0x7fffffffLL || btiles >= 0x7fffffffLL || ktiles >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
+  p.fwd_self_tiles = ftiles; p.bwd_self_tiles = btiles; p.kv_tiles = ktiles; p.pairs_per_head = pairs; p.P = (int32_t)P;
+  p.NA = (int32_t)NA;
+  p.flops_per_head_per_dim = 4.0 * ((double)pairs_self + (double)pairs_all * chunk);
 
   int64_t off = 0;
   auto take = [&](int64_t n) { const int64_t o = off; off += n; return o; };
-  p.off_cu_seqlens = take(nseq + 1);
   p.off_chunk_tok = take(p.N + 1);
-  p.off_fwd_self_tile_prefix = take(p.N + 1);
+  p.off_achunk_tok = take(NA + 1);
+  p.off_fwd_self_tile_prefix = take(NA + 1);
   p.off_fwd_self_tile_chunk = take(ftiles);
-  p.off_self_tile_prefix = take(p.N + 1);
+  p.off_self_tile_prefix = take(NA + 1);
   p.off_self_tile_chunk = take(btiles);
+  p.off_kv_tile_prefix = take(p.N + 1);
+  p.off_kv_tile_chunk = take(ktiles);
+  p.off_chunk_self_end = take(p.N);
   if (p.fallback) {
     p.off_seq_fbase = p.off_fchunk_tok = p.off_chunk_fb = p.off_chunk_local = p.off_pair_off = p.off_chunk_fid = -1;
   } else {
@@ -87,6 +106,7 @@ static int plan_core(const int32_t* cu, int nseq, int chunk, int topk, moba_plan
     p.off_pair_off = take(p.F + 1);
     p.off_chunk_fid = take(p.N);
   }
+  p.off_cu_seqlens = take(nseq + 1);
   p.table_ints = off;
   *pl = p;
   if (!tab) return MOBA_OK;
@@ -94,23 +114,41 @@ static int plan_core(const int32_t* cu, int nseq, int chunk, int topk, moba_plan
   // second pass: the tables
   std::memcpy(tab + p.off_cu_seqlens, cu, sizeof(int32_t) * (nseq + 1));
   int32_t* chunk_tok = tab + p.off_chunk_tok;
+  int32_t* achunk_tok = tab + p.off_achunk_tok;
   int32_t* fpre = tab + p.off_fwd_self_tile_prefix;
   int32_t* fch = tab + p.off_fwd_self_tile_chunk;
   int32_t* bpre = tab + p.off_self_tile_prefix;
   int32_t* bch = tab + p.off_self_tile_chunk;
-  int32_t c_all = 0, f_all = 0, pair_all = 0;
-  int64_t ft = 0, bt = 0;
+  int32_t* kpre = tab + p.off_kv_tile_prefix;
+  int32_t* kch = tab + p.off_kv_tile_chunk;
+  int32_t* self_end = tab + p.off_chunk_self_end;
+  int32_t c_all = 0, f_all = 0, pair_all = 0, a_all = 0;
+  int64_t ft = 0, bt = 0, kt = 0;
+  auto close_achunk = [&](int32_t tok0, int64_t alen, int32_t first_chunk, int32_t end_chunk) {
+    achunk_tok[a_all] = tok0;
+    fpre[a_all] = (int32_t)ft; bpre[a_all] = (int32_t)bt;
+    for (int64_t i = 0; i < (alen + kFwdTileRows - 1) / kFwdTileRows; ++i) fch[ft++] = a_all;
+    for (int64_t i = 0; i < (alen + TM - 1) / TM; ++i) bch[bt++] = a_all;
+    for (int32_t cc = first_chunk; cc < end_chunk; ++cc) self_end[cc] = (int32_t)(tok0 + alen);
+    ++a_all;
+  };
   for (int b = 0; b < nseq; ++b) {
     const int64_t len = (int64_t)cu[b + 1] - cu[b];
     const int64_t n = p.fallback ? 1 : (len + chunk - 1) / chunk;
     if (!p.fallback) tab[p.off_seq_fbase + b] = f_all;
     const int32_t fb = f_all;
+    int64_t alen = 0;
+    int32_t a_tok0 = cu[b], a_first = c_all;
     for (int64_t c = 0; c < n; ++c, ++c_all) {
       const int64_t clen = p.fallback ? len : std::min<int64_t>(chunk, len - c * chunk);
       chunk_tok[c_all] = (int32_t)(cu[b] + c * chunk);
-      fpre[c_all] = (int32_t)ft; bpre[c_all] = (int32_t)bt;
-      for (int64_t i = 0; i < (clen + kFwdTileRows - 1) / kFwdTileRows; ++i) fch[ft++] = c_all;
-      for (int64_t i = 0; i < (clen + TM - 1) / TM; ++i) bch[bt++] = c_all;
+      if (c > d) {
+        close_achunk(a_tok0, alen, a_first, c_all);
+        a_tok0 = chunk_tok[c_all]; a_first = c_all; alen = 0;
+      }
+      alen += clen;
+      kpre[c_all] = (int32_t)kt;
+      for (int64_t i = 0; i < (clen + TM - 1) / TM; ++i) kch[kt++] = c_all;
       if (p.fallback) continue;
       tab[p.off_chunk_fb + c_all] = fb;
       tab[p.off_chunk_local + c_all] = (int32_t)c;
@@ -124,9 +162,12 @@ static int plan_core(const int32_t* cu, int nseq, int chunk, int topk, moba_plan
         tab[p.off_chunk_fid + c_all] = -1;
       }
     }
+    close_achunk(a_tok0, alen, a_first, c_all);
   }
   chunk_tok[c_all] = cu[nseq];
-  fpre[c_all] = (int32_t)ft; bpre[c_all] = (int32_t)bt;
+  achunk_tok[a_all] = cu[nseq];
+  fpre[a_all] = (int32_t)ft; bpre[a_all] = (int32_t)bt;
+  kpre[c_all] = (int32_t)kt;
   if (!p.fallback) {
     tab[p.off_seq_fbase + nseq] = f_all;
     tab[p.off_pair_off + f_all] = pair_all;
@@ -134,14 +175,14 @@ static int plan_core(const int32_t* cu, int nseq, int chunk, int topk, moba_plan
   return MOBA_OK;
 }
 
-extern "C" int moba_plan(const int32_t* cu_seqlens_host, int nseq, int chunk, int topk, moba_plan_t* plan) {
-  return plan_core(cu_seqlens_host, nseq, chunk, topk, plan, nullptr);
+extern "C" int moba_plan(const int32_t* cu_seqlens_host, int nseq, int chunk, int topk, int dense, moba_plan_t* plan) {
+  return plan_core(cu_seqlens_host, nseq, chunk, topk, dense, plan, nullptr);
 }
 
-extern "C" int moba_plan_fill(const int32_t* cu_seqlens_host, int nseq, int chunk, int topk, moba_plan_t* plan,
-                              int32_t* tables_host) {
+extern "C" int moba_plan_fill(const int32_t* cu_seqlens_host, int nseq, int chunk, int topk, int dense,
+                              moba_plan_t* plan, int32_t* tables_host) {
   if (!tables_host) return MOBA_ERR_ARG;
-  return plan_core(cu_seqlens_host, nseq, chunk, topk, plan, tables_host);
+  return plan_core(cu_seqlens_host, nseq, chunk, topk, dense, plan, tables_host);
 }
 
 // Sizes, for H query heads, of every device buffer a forward (and backward) call takes besides q, k, v and the

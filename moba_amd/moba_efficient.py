@@ -26,6 +26,13 @@ HEAD_DIM = 128
 # MOBA_FIXED_REFERENCE=0 keeps the forward kernel on its running-maximum softmax for every problem (the
 # fixed-reference form, with its redo list, is otherwise used where the C ABI's `redo` argument says)
 FIXED_REFERENCE = os.environ.get("MOBA_FIXED_REFERENCE", "1") != "0"
+# Dense prefixes (see MobaPlan.dense_local): None = where they pay (problems large enough for the kernels whose
+# workgroups stay resident), True / False (MOBA_DENSE_PREFIX=1 / 0) = always / never.
+DENSE_PREFIX = {"0": False, "1": True}.get(os.environ.get("MOBA_DENSE_PREFIX", ""))
+# diagnostics: with KEEP_SCRATCH set, a forward call leaves views of its scratch in last_scratch ("redo": the
+# list of tiles the fixed-reference softmax handed to the kernel that tracks the maximum, count first; or None)
+KEEP_SCRATCH = False
+last_scratch = {}
 
 
 def _ptr(t: Optional[torch.Tensor]):
@@ -151,7 +158,8 @@ def chunk_mean(k: torch.Tensor, plan: MobaPlan, clear: Optional[torch.Tensor] = 
 
 def gate_topk(q: torch.Tensor, kbar: torch.Tensor, plan: MobaPlan, return_scores: bool = False,
               cnt: Optional[torch.Tensor] = None):
-    """sel [S, H, K] int32: selected filtered-chunk ids per (token, head), -1 padded.
+    """sel [S, H, K] int32: selected filtered-chunk ids per (token, head), -1 padded (with a plan that has dense
+    prefixes their tokens get no picks: the lists this selection feeds do not hold them).
     kbar may have fewer heads than q (grouped-query attention).  `cnt` (list_buffers()[0], zeroed): receives
     the counts build_lists starts from."""
     lib = _lib.load()
@@ -165,8 +173,8 @@ def gate_topk(q: torch.Tensor, kbar: torch.Tensor, plan: MobaPlan, return_scores
         scores = torch.full((S, H, plan.F), float("-inf"), dtype=torch.float32, device=q.device)
     _lib.check(lib.moba_gate_topk(_ptr(q), _ptr(kbar), _ptr(plan.tables["cu_seqlens"]), _ptr(plan.tables["seq_fbase"]),
                                   _ptr(sel), _ptr(scores), _ptr(plan.tables["pair_off"]), _ptr(cnt), S, H, Hkv, D,
-                                  plan.nseq, plan.F, plan.chunk_size, plan.K, _strides(q, None), _dtype_code(q),
-                                  _stream(q.device)), "moba_gate_topk")
+                                  plan.nseq, plan.F, plan.chunk_size, plan.K, plan.dense_local, _strides(q, None),
+                                  _dtype_code(q), _stream(q.device)), "moba_gate_topk")
     return (sel, scores) if return_scores else sel
 
 
@@ -214,7 +222,8 @@ def build_lists(sel: torch.Tensor, plan: MobaPlan, tile_rows: int = FWD_TILE_ROW
     _lib.check(lib.moba_build_lists(_ptr(sel), _ptr(t["chunk_tok"]), _ptr(t["chunk_fb"]), _ptr(t["chunk_local"]),
                                     _ptr(t["pair_off"]), _ptr(cnt), _ptr(seg_off), _ptr(tile_off), _ptr(seg_dest),
                                     _ptr(tile_seg), S, H, K, plan.N, plan.F, plan.P, plan.cmax, tile_rows, bound,
-                                    1 if counted else 0, *second_args, _stream(dev)), "moba_build_lists")
+                                    1 if counted else 0, *second_args, plan.dense_local, _stream(dev)),
+               "moba_build_lists")
     return (seg_off, tile_off, seg_dest, tile_seg) + second
 
 
@@ -363,13 +372,13 @@ def _forward(q, k, v, plan: MobaPlan, timer: Optional[StageTimer] = None, scale:
                                            strides, code, cntp, g.list_sizes[0], stream), "moba_chunk_mean")
         with span("gate_topk"):
             _lib.check(lib.moba_gate_topk(qp, kbarp, tp["cu_seqlens"], tp["seq_fbase"], selp, null, tp["pair_off"],
-                                          cntp, S, H, Hkv, D, plan.nseq, plan.F, plan.chunk_size, K, strides, code,
-                                          stream), "moba_gate_topk")
+                                          cntp, S, H, Hkv, D, plan.nseq, plan.F, plan.chunk_size, K, plan.dense_local,
+                                          strides, code, stream), "moba_gate_topk")
         with span("build_lists"):
             _lib.check(lib.moba_build_lists(selp, tp["chunk_tok"], tp["chunk_fb"], tp["chunk_local"], tp["pair_off"],
                                             cntp, seg_offp, tile_offp, seg_destp, tile_segp, S, H, K, plan.N, plan.F,
-                                            plan.P, plan.cmax, FWD_TILE_ROWS, g.bound, 1, *bwd_args, stream),
-                       "moba_build_lists")
+                                            plan.P, plan.cmax, FWD_TILE_ROWS, g.bound, 1, *bwd_args, plan.dense_local,
+                                            stream), "moba_build_lists")
     out = torch.empty((S, H, D), dtype=q.dtype, device=dev)
     lse = torch.empty((S, H), dtype=torch.float32, device=dev)
     ws2 = torch.empty(g.ws_bytes, dtype=torch.uint8, device=dev)
@@ -378,10 +387,13 @@ def _forward(q, k, v, plan: MobaPlan, timer: Optional[StageTimer] = None, scale:
     part_lsep = ctypes.c_void_p(base + g.part_o_bytes)
     queuesp = ctypes.c_void_p(base + g.part_o_bytes + g.rows * 4)
     redop = ctypes.c_void_p(base + g.part_o_bytes + g.rows * 4 + 32) if FIXED_REFERENCE else null
+    if KEEP_SCRATCH:
+        at = g.part_o_bytes + g.rows * 4 + 32
+        last_scratch["redo"] = ws2[at:at + 4 * (g.scratch_ints - 8)].view(torch.int32) if FIXED_REFERENCE else None
     with span("fwd_partials"):
         _lib.check(lib.moba_fwd_partials(qp, kp, vp, part_op, part_lsep, seg_offp, tile_offp, seg_destp,
-                                         tp.get("fchunk_tok", null), tp["chunk_tok"], tp["fwd_self_tile_prefix"],
-                                         tile_segp, tp["fwd_self_tile_chunk"], S, H, Hkv, D, K, plan.F, plan.N,
+                                         tp.get("fchunk_tok", null), tp["achunk_tok"], tp["fwd_self_tile_prefix"],
+                                         tile_segp, tp["fwd_self_tile_chunk"], S, H, Hkv, D, K, plan.F, plan.NA,
                                          plan.chunk_size, g.bound, plan.fwd_self_tiles, g.split, strides, queuesp,
                                          redop, scale, code, stream), "moba_fwd_partials")
     with span("fwd_merge"):
@@ -407,7 +419,7 @@ def _backward(dout, q, k, v, out, lse, sel, seg_off, seg_dest, plan: MobaPlan, s
     b = g.bwd.get(Hkv)
     if b is None:
         bound = plan.hist_tile_bound(H, TILE_ROWS)
-        kv_bytes = int(lib.moba_bwd_dkv_scratch_bytes(S, Hkv, plan.self_tiles))
+        kv_bytes = int(lib.moba_bwd_dkv_scratch_bytes(S, Hkv, plan.kv_tiles))
         # small problems: the keys of every history tile of the dQ kernel in `split` parts with slots of their own
         split = 1 if plan.fallback else int(lib.moba_bwd_dq_key_split(S, H, K, plan.chunk_size, bound, plan.self_tiles))
         sizes = [split * S * H * (K + 1) * D * q.element_size(), 2 * S * H * 4, 64,
@@ -431,10 +443,11 @@ def _backward(dout, q, k, v, out, lse, sel, seg_off, seg_dest, plan: MobaPlan, s
     dk = torch.empty((S, Hkv, D), dtype=k.dtype, device=dev)
     dv = torch.empty((S, Hkv, D), dtype=v.dtype, device=dev)
     _lib.check(lib.moba_bwd(_ptr(dout), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _ptr(sel), _ptr(seg_off),
-                            tile_offp, _ptr(seg_dest), tp.get("fchunk_tok", null), tp["chunk_tok"],
+                            tile_offp, _ptr(seg_dest), tp.get("fchunk_tok", null), tp["achunk_tok"],
                             tp["self_tile_prefix"], tile_segp, tp["self_tile_chunk"], tp.get("chunk_fid", null),
-                            deltap, part_dqp, _ptr(dq), _ptr(dk), _ptr(dv), S, H, Hkv, D, K, plan.F, plan.N,
-                            plan.chunk_size, bound, plan.self_tiles, split, _strides(q, k), queuesp,
+                            tp["chunk_tok"], tp["kv_tile_prefix"], tp["kv_tile_chunk"], tp["chunk_self_end"],
+                            deltap, part_dqp, _ptr(dq), _ptr(dk), _ptr(dv), S, H, Hkv, D, K, plan.F, plan.NA,
+                            plan.chunk_size, bound, plan.self_tiles, plan.kv_tiles, split, _strides(q, k), queuesp,
                             kvp if kv_bytes else null, kv_bytes, scale, _dtype_code(q), stream), "moba_bwd")
     return dq, dk, dv
 
@@ -468,8 +481,31 @@ class _MobaAttention(torch.autograd.Function):
         return dq, dk, dv, None, None, None
 
 
+def _choose_plan(plan: MobaPlan, H: int) -> MobaPlan:
+    """The plan the kernels run: the batch's own, or its form with dense prefixes (MobaPlan.dense_local) where that
+    pays -- when the forward kernel would still keep its workgroups resident, i.e. for problems of many tiles; on
+    a problem of a few hundred tiles the long causal tiles of a dense prefix would run alone at the end."""
+    if plan.fallback or plan.dense_local:
+        return plan
+    key = ("dense", H, DENSE_PREFIX)
+    choice = plan.memo.get(key)
+    if choice is None:
+        choice = plan
+        if DENSE_PREFIX is not False:
+            dense = plan.with_dense_prefix()
+            if dense.pairs_per_head == 0:
+                # every token lies in a dense prefix: plain causal attention, no gate and no lists at all
+                dense = make_plan(plan.cu, plan.chunk_size, 1, device=plan.device)
+            if DENSE_PREFIX or _lib.load().moba_fwd_is_queued(dense.hist_tile_bound(H, FWD_TILE_ROWS),
+                                                               dense.fwd_self_tiles, H):
+                choice = dense
+        plan.memo[key] = choice
+    return choice
+
+
 def _attend(q, k, v, plan, timer=None, scale=0.0):
     """(out, lse): through autograd when a gradient may be asked for, straight to the kernels otherwise."""
+    plan = _choose_plan(plan, _dims(q)[1])
     if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad):
         return _MobaAttention.apply(q, k, v, plan, timer, scale)
     return _forward(q, k, v, plan, timer, scale)[:2]

@@ -35,20 +35,34 @@ class MobaPlan:
     fallback: bool      # k_eff <= 0: full causal attention (moba/moba_efficient.py:318-321)
     P: int              # (filtered chunk, later chunk of the same sequence) pairs
     cmax: int           # max chunks per sequence minus one
-    pairs_per_head: int  # selected (token, chunk) pairs per head  (M / H)
-    self_tiles: int     # row tiles of the self part, per head (TILE_ROWS rows each; tables self_tile_*)
+    pairs_per_head: int  # list entries per head (M / H): selected (token, chunk) pairs of the tokens beyond the dense prefixes
+    self_tiles: int     # row tiles of the attention chunks, per head (TILE_ROWS rows each; tables self_tile_*)
     fwd_self_tiles: int  # the same in tiles of FWD_TILE_ROWS rows (tables fwd_self_tile_*)
     flops_per_head: float
+    # Dense prefixes.  A token in chunk c <= K of its sequence selects every earlier chunk, so what it attends is
+    # the plain causal prefix.  With dense_local = d (0 <= d <= K) the chunks 0..d of every sequence form one
+    # attention chunk whose rows run through the causal self path alone: no gate, no list entries and one partial
+    # result for them.  d = 0 is the reference's own decomposition (every chunk its own attention chunk).
+    dense_local: int = 0
+    NA: int = 0         # attention chunks (tables achunk_tok, self_tile_*, fwd_self_tile_*)
+    kv_tiles: int = 0   # key tiles of TILE_ROWS keys of the chunks, per key/value head (tables kv_tile_*)
     tables: Dict[str, torch.Tensor] = field(default_factory=dict)
     host: Dict[str, np.ndarray] = field(default_factory=dict)
     memo: Dict[tuple, object] = field(default_factory=dict)  # what callers derive once per plan (sizes, pointers)
+    device: object = None
 
     def hist_tile_bound(self, H: int, rows: int = TILE_ROWS) -> int:
         """Upper bound on the number of history tiles of `rows` rows (every segment may end in a partial tile)."""
         return (self.pairs_per_head * H) // rows + self.F * H
 
+    def with_dense_prefix(self) -> "MobaPlan":
+        """The plan of the same batch with the first K + 1 chunks of every sequence as one attention chunk."""
+        if self.fallback or self.dense_local == self.K:
+            return self
+        return _build(np.asarray(self.cu, dtype=np.int64), self.chunk_size, self.moba_topk, self.device, dense=True)
 
-def _host_tables(cu: np.ndarray, B: int, topk: int):
+
+def _host_tables(cu: np.ndarray, B: int, topk: int, dense: bool = False):
     lens = np.diff(cu)
     nseq = lens.size
     n_chunks = (lens + B - 1) // B
@@ -60,6 +74,9 @@ def _host_tables(cu: np.ndarray, B: int, topk: int):
         n_chunks = np.ones_like(n_chunks)
         chunk_tok = cu.copy()
         chunk_len = lens
+        seq_of_chunk = np.arange(nseq)
+        local = np.zeros(nseq, dtype=np.int64)
+        K = d = 0
     else:
         seq_of_chunk = np.repeat(np.arange(nseq), n_chunks)
         cbase = np.concatenate([[0], np.cumsum(n_chunks)])[:-1]
@@ -67,15 +84,30 @@ def _host_tables(cu: np.ndarray, B: int, topk: int):
         chunk_start = cu[seq_of_chunk] + local * B
         chunk_len = np.minimum(B, cu[seq_of_chunk + 1] - chunk_start)
         chunk_tok = np.concatenate([chunk_start, [cu[-1]]])
+        cmax = int(n_chunks.max() - 1)
+        K = min(k_eff, cmax)
+        d = K if dense else 0
     N = int(n_chunks.sum())
-    tiles = (chunk_len + TILE_ROWS - 1) // TILE_ROWS
-    ftiles = (chunk_len + FWD_TILE_ROWS - 1) // FWD_TILE_ROWS
-    out = dict(chunk_tok=chunk_tok, self_tile_prefix=np.concatenate([[0], np.cumsum(tiles)]),
-               self_tile_chunk=np.repeat(np.arange(N), tiles),
+    # attention chunks: chunks 0..d of a sequence together, every later chunk alone
+    starts_a = (local == 0) | (local > d)
+    achunk_tok = np.concatenate([chunk_tok[:-1][starts_a], [cu[-1]]])
+    achunk_len = np.diff(achunk_tok)
+    NA = achunk_len.size
+    achunk_of = np.cumsum(starts_a) - 1                      # attention chunk of every chunk
+    tiles = (achunk_len + TILE_ROWS - 1) // TILE_ROWS
+    ftiles = (achunk_len + FWD_TILE_ROWS - 1) // FWD_TILE_ROWS
+    ktiles = (chunk_len + TILE_ROWS - 1) // TILE_ROWS
+    out = dict(chunk_tok=chunk_tok, achunk_tok=achunk_tok,
                fwd_self_tile_prefix=np.concatenate([[0], np.cumsum(ftiles)]),
-               fwd_self_tile_chunk=np.repeat(np.arange(N), ftiles))
+               fwd_self_tile_chunk=np.repeat(np.arange(NA), ftiles),
+               self_tile_prefix=np.concatenate([[0], np.cumsum(tiles)]),
+               self_tile_chunk=np.repeat(np.arange(NA), tiles),
+               kv_tile_prefix=np.concatenate([[0], np.cumsum(ktiles)]),
+               kv_tile_chunk=np.repeat(np.arange(N), ktiles),
+               chunk_self_end=achunk_tok[achunk_of + 1])     # where the causal rows of a chunk's keys end
     info = dict(nseq=nseq, N=N, F=0 if fallback else F, k_eff=k_eff, fallback=fallback, K=0, P=0, cmax=0,
-                pairs_per_head=0, self_tiles=int(tiles.sum()), fwd_self_tiles=int(ftiles.sum()))
+                pairs_per_head=0, self_tiles=int(tiles.sum()), fwd_self_tiles=int(ftiles.sum()), NA=NA, dense_local=d,
+                kv_tiles=int(ktiles.sum()))
     pairs_self = int((chunk_len.astype(np.int64) * (chunk_len + 1) // 2).sum())
     if not fallback:
         seq_fbase = np.concatenate([[0], np.cumsum(n_chunks - 1)])
@@ -84,15 +116,14 @@ def _host_tables(cu: np.ndarray, B: int, topk: int):
         fchunk_tok = chunk_start[fidx]
         nq = (n_chunks[seq_of_chunk] - 1 - local)[fidx]          # later chunks of the same sequence
         pair_off = np.concatenate([[0], np.cumsum(nq)])
-        cmax = int(n_chunks.max() - 1)
-        K = min(k_eff, cmax)
-        pairs = int((chunk_len.astype(np.int64) * np.minimum(K, local)).sum())
+        pairs_all = int((chunk_len.astype(np.int64) * np.minimum(K, local)).sum())
+        pairs = int((chunk_len.astype(np.int64) * np.where(local > d, np.minimum(K, local), 0)).sum())
         chunk_fid = np.full(N, -1, dtype=np.int64)
         chunk_fid[fidx] = np.arange(F)
         out.update(seq_fbase=seq_fbase, fchunk_tok=fchunk_tok, chunk_fb=seq_fbase[seq_of_chunk], chunk_local=local,
                    pair_off=pair_off, chunk_fid=chunk_fid)
         info.update(K=K, P=int(nq.sum()), cmax=cmax, pairs_per_head=pairs)
-        flops = 4.0 * (pairs_self + pairs * B)
+        flops = 4.0 * (pairs_self + pairs_all * B)
     else:
         flops = 4.0 * pairs_self
     info["flops_per_head_per_d"] = flops
@@ -117,7 +148,7 @@ def _remember(cache, key, value):
         cache.popitem(last=False)
 
 
-def _build(cu: np.ndarray, chunk_size: int, moba_topk: int, device) -> MobaPlan:
+def _build(cu: np.ndarray, chunk_size: int, moba_topk: int, device, dense: bool = False) -> MobaPlan:
     if cu.ndim != 1 or cu.size < 2:
         raise ValueError("cu_seqlens must be a 1-D tensor with at least two entries")
     if cu[0] != 0 or (np.diff(cu) <= 0).any():
@@ -125,17 +156,19 @@ def _build(cu: np.ndarray, chunk_size: int, moba_topk: int, device) -> MobaPlan:
     if chunk_size <= 0 or moba_topk <= 0:
         raise ValueError("moba_chunk_size and moba_topk must be positive")
     on_device = device is not None and torch.device(device).type != "cpu"
-    vkey = (cu.tobytes(), int(chunk_size), int(moba_topk), str(device) if on_device else None)
+    vkey = (cu.tobytes(), int(chunk_size), int(moba_topk), str(device) if on_device else None, bool(dense))
     hit = _BY_VALUE.get(vkey)
     if hit is not None:
         _BY_VALUE.move_to_end(vkey)
         return hit
-    host, info = _host_tables(cu, int(chunk_size), int(moba_topk))
+    host, info = _host_tables(cu, int(chunk_size), int(moba_topk), dense)
     host["cu_seqlens"] = cu  # the kernels read the plan's own copy, never the caller's tensor
     plan = MobaPlan(cu=cu.tolist(), chunk_size=int(chunk_size), moba_topk=int(moba_topk), S=int(cu[-1]),
                     nseq=info["nseq"], N=info["N"], F=info["F"], k_eff=info["k_eff"], K=info["K"],
                     fallback=info["fallback"], P=info["P"], cmax=info["cmax"], pairs_per_head=info["pairs_per_head"],
-                    self_tiles=info["self_tiles"], fwd_self_tiles=info["fwd_self_tiles"], flops_per_head=info["flops_per_head_per_d"], host=host)
+                    self_tiles=info["self_tiles"], fwd_self_tiles=info["fwd_self_tiles"],
+                    flops_per_head=info["flops_per_head_per_d"], dense_local=info["dense_local"], NA=info["NA"],
+                    kv_tiles=info["kv_tiles"], host=host, device=device if on_device else None)
     if on_device:
         names = list(host)
         flat = np.concatenate([host[n_].astype(np.int32) for n_ in names])

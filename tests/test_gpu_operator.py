@@ -20,7 +20,38 @@ MAX_ABS, MEAN_ABS = 2e-2, 2e-3
 REF_MAX_ABS, REF_MEAN_ABS = 4e-2, 4e-4
 
 
-def run_case(batch, seqlen, heads, B, topk, seed=0, check_grad=True, dtype=torch.bfloat16, ref_bounds=True):
+class dense_prefix:
+    """The operator's choice between a batch's plain plan and the one with dense prefixes, for the calls inside:
+    True / False force it, None leaves it to the operator (dense prefixes for large problems only)."""
+
+    def __init__(self, choice):
+        self.choice = choice
+
+    def __enter__(self):
+        from moba_amd import moba_efficient as E
+        self.saved = E.DENSE_PREFIX
+        E.DENSE_PREFIX = self.choice
+
+    def __exit__(self, *exc):
+        from moba_amd import moba_efficient as E
+        E.DENSE_PREFIX = self.saved
+        return False
+
+
+def check_selection(sel, want, gate, tol=1e-4):
+    """The kernel's selection against the oracle's: equal as sets except where the fp32 scores nearly tie."""
+    got = torch.sort(torch.where(sel < 0, torch.full_like(sel, 1 << 30), sel), dim=-1).values
+    got = torch.where(got == 1 << 30, torch.full_like(got, -1), got)
+    diff_rows = (got != want).any(dim=-1)
+    for s_, h_ in diff_rows.nonzero().tolist():
+        a = set(got[s_, h_].tolist()) - {-1}
+        b = set(want[s_, h_].tolist()) - {-1}
+        gap = max(abs(float(gate[s_, h_, x]) - float(gate[s_, h_, y])) for x in a ^ b for y in a ^ b)
+        assert gap < tol, (s_, h_, a, b, gap)
+    assert diff_rows.float().mean() < 1e-3
+
+
+def run_case(batch, seqlen, heads, B, topk, seed=0, check_grad=True, dtype=torch.bfloat16, ref_bounds=True, dense=None):
     from moba_amd import moba_efficient as E
     from moba_amd.plan import make_plan
 
@@ -28,28 +59,17 @@ def run_case(batch, seqlen, heads, B, topk, seed=0, check_grad=True, dtype=torch
     dev = torch.device("cuda")
     cu_t = torch.tensor(cu, dtype=torch.int32, device=dev)
     qg, kg, vg = (x.to(dev).requires_grad_(True) for x in (q, k, v))
-    out = E.moba_attn_varlen(qg, kg, vg, cu_t, mx, moba_chunk_size=B, moba_topk=topk)
-    if check_grad:
-        torch.autograd.backward(out, do.to(dev))
+    with dense_prefix(dense):
+        out = E.moba_attn_varlen(qg, kg, vg, cu_t, mx, moba_chunk_size=B, moba_topk=topk)
+        if check_grad:
+            torch.autograd.backward(out, do.to(dev))
     plan = make_plan(cu_t, B, topk)
     sel = None
     if not plan.fallback:
         sel = E.gate_topk(qg.detach(), E.chunk_mean(kg.detach(), plan), plan).cpu()
         # the kernel's selection must agree with the oracle's except at numerical near-ties
-        kbar = O.chunk_mean(k, cu, B)
-        gate = O.gate_scores(q, kbar, cu, B)
-        want = O.select_topk(gate, plan.K)
-        got = torch.sort(torch.where(sel < 0, torch.full_like(sel, 1 << 30), sel), dim=-1).values
-        got = torch.where(got == 1 << 30, torch.full_like(got, -1), got)
-        diff_rows = (got != want).any(dim=-1)
-        if diff_rows.any():
-            # every disagreement must be a near-tie of the fp32 scores
-            for s_, h_ in diff_rows.nonzero().tolist():
-                a = set(got[s_, h_].tolist()) - {-1}
-                b = set(want[s_, h_].tolist()) - {-1}
-                gap = max(abs(float(gate[s_, h_, x]) - float(gate[s_, h_, y])) for x in a ^ b for y in a ^ b)
-                assert gap < 1e-4, (s_, h_, a, b, gap)
-        assert diff_rows.float().mean() < 1e-3
+        gate = O.gate_scores(q, O.chunk_mean(k, cu, B), cu, B)
+        check_selection(sel, O.select_topk(gate, plan.K), gate)
     qc, kc, vc = (x.clone().requires_grad_(True) for x in (q, k, v))
     ref = O.moba_attn_varlen_oracle(qc, kc, vc, cu, mx, B, topk, sel=sel)
     err = (out.detach().cpu().float() - ref.detach()).abs()
@@ -79,13 +99,15 @@ def run_case(batch, seqlen, heads, B, topk, seed=0, check_grad=True, dtype=torch
 GRID = list(itertools.product([1, 4, 7], [1, 2, 4, 8], [512, 1024, 2048], [128, 256, 1024], [2, 3, 4]))
 
 
+@pytest.mark.parametrize("dense", [None, True])
 @pytest.mark.parametrize("chunk", range(12))
-def test_reference_grid(chunk):
-    """The reference's 324 cases (batch x heads x seqlen x chunk x topk), 27 per test."""
+def test_reference_grid(chunk, dense):
+    """The reference's 324 cases (batch x heads x seqlen x chunk x topk), 27 per test; as the operator plans them
+    (problems this small: the reference's own decomposition) and with dense prefixes forced."""
     cases = GRID[chunk * 27:(chunk + 1) * 27]
     for batch, heads, seqlen, B, topk in cases:
-        print("case", batch, heads, seqlen, B, topk, flush=True)
-        run_case(batch, seqlen, heads, B, topk)
+        print("case", batch, heads, seqlen, B, topk, dense, flush=True)
+        run_case(batch, seqlen, heads, B, topk, dense=dense)
 
 
 @pytest.mark.parametrize("batch,seqlen,heads,B,topk", [
@@ -100,6 +122,7 @@ def test_reference_grid(chunk):
 ])
 def test_edge_shapes(batch, seqlen, heads, B, topk):
     run_case(batch, seqlen, heads, B, topk, seed=7)
+    run_case(batch, seqlen, heads, B, topk, seed=7, dense=True)
 
 
 @pytest.mark.parametrize("batch,seqlen,heads,B,topk", [
@@ -113,6 +136,7 @@ def test_edge_shapes(batch, seqlen, heads, B, topk):
 def test_float16(batch, seqlen, heads, B, topk):
     """fp16 inputs (the dtype of the reference's example script), same bounds as bf16."""
     run_case(batch, seqlen, heads, B, topk, seed=11, dtype=torch.float16)
+    run_case(batch, seqlen, heads, B, topk, seed=11, dtype=torch.float16, dense=True)
 
 
 @pytest.mark.parametrize("batch,seqlen,heads,kv_heads,B,topk,dtype", [
@@ -159,7 +183,8 @@ def test_grouped_query(batch, seqlen, heads, kv_heads, B, topk, dtype):
     (1, 2048, 4, 2, 128, 1, torch.bfloat16),     # fallback: full causal attention
     (1, 8192, 2, 1, 1024, 3, torch.bfloat16),    # few tiles: the forward cuts the history tiles' keys into parts
 ])
-def test_grouped_query_vs_oracle(batch, seqlen, heads, kv_heads, B, topk, dtype):
+@pytest.mark.parametrize("dense", [None, True])
+def test_grouped_query_vs_oracle(batch, seqlen, heads, kv_heads, B, topk, dtype, dense):
     """The grouped-query operator against the oracle run on key/value heads expanded with repeat_interleave
     (the reference's semantics, moba/wrapper.py:59-61): out and dq as they are, dk and dv against the
     oracle's gradients summed over the query heads of each group."""
@@ -171,18 +196,17 @@ def test_grouped_query_vs_oracle(batch, seqlen, heads, kv_heads, B, topk, dtype)
     _, k, v, _, _, _ = make_case(batch, seqlen, kv_heads, seed=6, dtype=dtype)
     cu_t = torch.tensor(cu, dtype=torch.int32, device="cuda")
     qg, kg, vg = (x.cuda().requires_grad_(True) for x in (q, k, v))
-    out = moba_attn_varlen_gqa(qg, kg, vg, cu_t, mx, B, topk)
-    out.backward(do.cuda())
+    with dense_prefix(dense):
+        out = moba_attn_varlen_gqa(qg, kg, vg, cu_t, mx, B, topk)
+        out.backward(do.cuda())
     plan = make_plan(cu_t, B, topk)
     sel = None
     if not plan.fallback:
         sel = E.gate_topk(qg.detach(), E.chunk_mean(kg.detach(), plan), plan).cpu()
         # the selection itself: the oracle's on the expanded heads, up to near-ties of the fp32 scores
         kx = torch.repeat_interleave(k, rep, dim=1)
-        want = O.select_topk(O.gate_scores(q, O.chunk_mean(kx, cu, B), cu, B), plan.K)
-        got = torch.sort(torch.where(sel < 0, torch.full_like(sel, 1 << 30), sel), dim=-1).values
-        got = torch.where(got == 1 << 30, torch.full_like(got, -1), got)
-        assert (got != want).any(dim=-1).float().mean() < 1e-3
+        gate = O.gate_scores(q, O.chunk_mean(kx, cu, B), cu, B)
+        check_selection(sel, O.select_topk(gate, plan.K), gate)
     qc = q.clone().requires_grad_(True)
     kc, vc = (x.clone().requires_grad_(True) for x in (k, v))
     ref = O.moba_attn_varlen_oracle(qc, torch.repeat_interleave(kc, rep, dim=1), torch.repeat_interleave(vc, rep, dim=1),
@@ -221,8 +245,9 @@ def test_random_shapes(seed):
         B = int(rng.integers(8, 300))
         topk = int(rng.integers(1, 9))
         dtype = torch.float16 if rng.integers(0, 2) else torch.bfloat16
-        print("random case", batch, seqlen, heads, B, topk, dtype, flush=True)
-        run_case(batch, seqlen, heads, B, topk, seed=int(rng.integers(0, 1000)), dtype=dtype, ref_bounds=False)
+        dense = bool(rng.integers(0, 2))
+        print("random case", batch, seqlen, heads, B, topk, dtype, dense, flush=True)
+        run_case(batch, seqlen, heads, B, topk, seed=int(rng.integers(0, 1000)), dtype=dtype, ref_bounds=False, dense=dense)
 
 
 def test_peaked_softmax_and_exact_gate_ties():
@@ -459,10 +484,8 @@ def test_narrow_heads_are_padded(head_dim, dtype):
         err = (got.detach().cpu().float() - want.detach().float()).abs()
         assert err.max() < MAX_ABS and err.mean() < MEAN_ABS, (name, err.max().item(), err.mean().item())
     # and the selection itself is the oracle's on the narrow tensors, up to near-ties of the fp32 scores
-    want = O.select_topk(O.gate_scores(q, O.chunk_mean(k, cu, 128), cu, 128), plan.K)
-    got = torch.sort(torch.where(sel < 0, torch.full_like(sel, 1 << 30), sel), dim=-1).values
-    got = torch.where(got == 1 << 30, torch.full_like(got, -1), got)
-    assert (got != want).any(dim=-1).float().mean() < 1e-3
+    gate = O.gate_scores(q, O.chunk_mean(k, cu, 128), cu, 128)
+    check_selection(sel, O.select_topk(gate, plan.K), gate)
 
 
 def test_heads_wider_than_128_are_refused():

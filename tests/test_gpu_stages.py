@@ -11,9 +11,15 @@ from oracle import moba_oracle as O
 pytestmark = pytest.mark.gpu
 
 
-def _plan(cu, B, topk):
+def _plan(cu, B, topk, dense=False):
     from moba_amd.plan import make_plan
-    return make_plan(torch.tensor(cu, dtype=torch.int32, device="cuda"), B, topk)
+    plan = make_plan(torch.tensor(cu, dtype=torch.int32, device="cuda"), B, topk)
+    return plan.with_dense_prefix() if dense else plan
+
+
+def _token_chunk_local(cu, B):
+    """index, inside its sequence, of the chunk of every token"""
+    return torch.cat([torch.arange(b - a) // B for a, b in zip(cu[:-1], cu[1:])])
 
 
 def _note(*a):
@@ -108,17 +114,25 @@ def test_topk_from_injected_scores_bit_exact(K):
 
 # ------------------------------------------------------------------ gather lists
 # (the last case: more candidate chunks than one pass of the gate's LDS histogram holds)
+@pytest.mark.parametrize("dense", [False, True])
 @pytest.mark.parametrize("counted", [False, True])
 @pytest.mark.parametrize("batch,seqlen,heads,B,topk", [(1, 2048, 2, 128, 3), (5, 3000, 3, 100, 4), (2, 9000, 1, 64, 12),
                                                        (3, 5000, 5, 192, 2), (1, 140817, 1, 64, 2)])
-def test_gather_lists(batch, seqlen, heads, B, topk, counted):
+def test_gather_lists(batch, seqlen, heads, B, topk, counted, dense):
     """The lists from the counting pass of moba_build_lists, and from the counts the gate leaves as a by-product
-    in an array that the chunk mean cleared."""
+    in an array that the chunk mean cleared.  With dense prefixes the tokens of the first K + 1 chunks of every
+    sequence have no picks and no list entries; every other token's picks are what they are without."""
     from moba_amd import moba_efficient as E
-    _note("lists", batch, seqlen, heads, B, topk, counted)
+    _note("lists", batch, seqlen, heads, B, topk, counted, dense)
     q, k, v, _, cu, _ = make_case(batch, seqlen, heads, seed=4)
-    plan = _plan(cu, B, topk)
+    plan = _plan(cu, B, topk, dense)
     kbar = O.chunk_mean(k, cu, B)
+    if dense:
+        plain = E.gate_topk(q.cuda(), kbar.cuda(), _plan(cu, B, topk)).cpu()
+        in_prefix = (_token_chunk_local(cu, B) <= plan.K)[:, None, None].expand_as(plain)
+        want_sel = torch.where(in_prefix, torch.full_like(plain, -1), plain)
+        assert plan.dense_local == plan.K > 0 and bool(in_prefix.any())
+        assert torch.equal(E.gate_topk(q.cuda(), kbar.cuda(), plan).cpu(), want_sel)
     if counted:
         buffers = E.list_buffers(plan, heads, torch.device("cuda"))
         for b in buffers:
@@ -136,7 +150,9 @@ def test_gather_lists(batch, seqlen, heads, B, topk, counted):
     sel = sel.cpu()
     counts, offs, rows, slots = O.gather_lists(sel, plan.F)
     H, K1 = heads, plan.K + 1
-    assert offs[-1] == plan.pairs_per_head * H == O.expected_pair_count(cu, B, plan.K, H)
+    assert offs[-1] == plan.pairs_per_head * H
+    if not dense:
+        assert offs[-1] == O.expected_pair_count(cu, B, plan.K, H)
     assert np.array_equal(seg_off, offs)
     heads_of = np.repeat(np.arange(plan.F * H) % H, counts)
     want_dest = (rows * H + heads_of) * K1 + 1 + slots
@@ -225,17 +241,19 @@ def test_merge_of_random_partials(K, dtype, parts):
 
 
 # ------------------------------------------------------------------ the one-call attention entry point
+@pytest.mark.parametrize("dense", [False, True])
 @pytest.mark.parametrize("batch,seqlen,heads,B,topk,dtype", [(3, 3000, 3, 100, 3, torch.bfloat16),
                                                               (2, 4096, 2, 256, 4, torch.float16),
                                                               (1, 2048, 2, 128, 1, torch.bfloat16)])
-def test_moba_fwd_entry_point(batch, seqlen, heads, B, topk, dtype):
+def test_moba_fwd_entry_point(batch, seqlen, heads, B, topk, dtype, dense):
     """moba_fwd (partial attentions + merge behind one call): bit for bit what moba_fwd_partials followed by
-    moba_fwd_merge give, and within the tolerances of the oracle run on the same selection."""
+    moba_fwd_merge give, and within the tolerances of the oracle run on the same selection (with dense prefixes:
+    on the selection of the plain plan, whose attended sets are the same)."""
     from moba_amd import _lib
     from moba_amd import moba_efficient as E
-    _note("moba_fwd", batch, seqlen, heads, B, topk, dtype)
+    _note("moba_fwd", batch, seqlen, heads, B, topk, dtype, dense)
     q, k, v, _, cu, mx = make_case(batch, seqlen, heads, seed=9, dtype=dtype)
-    plan = _plan(cu, B, topk)
+    plan = _plan(cu, B, topk, dense)
     qg, kg, vg = q.cuda(), k.cuda(), v.cuda()
     want_out, want_lse, sel, seg_off, tile_off, seg_dest, tile_seg = E._forward(qg, kg, vg, plan)
     lib = _lib.load()
@@ -250,12 +268,14 @@ def test_moba_fwd_entry_point(batch, seqlen, heads, B, topk, dtype):
     queues = torch.empty(8, dtype=torch.int32, device=dev)
     p = E._ptr
     _lib.check(lib.moba_fwd(p(qg), p(kg), p(vg), p(part_o), p(part_lse), p(sel), p(seg_off), p(tile_off), p(seg_dest),
-                            p(t.get("fchunk_tok")), p(t["chunk_tok"]), p(t["fwd_self_tile_prefix"]), p(tile_seg),
-                            p(t["fwd_self_tile_chunk"]), p(out), p(lse), S, H, H, D, K, plan.F, plan.N, plan.chunk_size,
+                            p(t.get("fchunk_tok")), p(t["achunk_tok"]), p(t["fwd_self_tile_prefix"]), p(tile_seg),
+                            p(t["fwd_self_tile_chunk"]), p(out), p(lse), S, H, H, D, K, plan.F, plan.NA, plan.chunk_size,
                             bound, plan.fwd_self_tiles, split, None, p(queues), None, 0.0, E._dtype_code(qg),
                             E._stream(dev)), "moba_fwd")
     torch.cuda.synchronize()
     assert torch.equal(out, want_out) and torch.equal(lse, want_lse)
+    if dense and sel is not None:
+        sel = E.gate_topk(qg, E.chunk_mean(kg, plan), _plan(cu, B, topk))
     ref, ref_lse, _ = O.moba_attn_varlen_oracle(q, k, v, cu, mx, B, topk, sel=None if sel is None else sel.cpu(),
                                                 return_aux=True)
     err = (out.cpu().float() - ref).abs()
@@ -282,8 +302,8 @@ def _attention_stage(q, k, v, plan, aux, with_redo, key_split=1):
     redo = torch.full((1 + tiles,), -7, dtype=torch.int32, device=dev) if with_redo else None
     p = E._ptr
     _lib.check(lib.moba_fwd(p(q), p(k), p(v), p(part_o), p(part_lse), p(sel), p(seg_off), p(tile_off), p(seg_dest),
-                            p(t.get("fchunk_tok")), p(t["chunk_tok"]), p(t["fwd_self_tile_prefix"]), p(tile_seg),
-                            p(t["fwd_self_tile_chunk"]), p(out), p(lse), S, H, H, D, K, plan.F, plan.N, plan.chunk_size,
+                            p(t.get("fchunk_tok")), p(t["achunk_tok"]), p(t["fwd_self_tile_prefix"]), p(tile_seg),
+                            p(t["fwd_self_tile_chunk"]), p(out), p(lse), S, H, H, D, K, plan.F, plan.NA, plan.chunk_size,
                             plan.hist_tile_bound(H, 256), plan.fwd_self_tiles, key_split, None, p(queues), p(redo), 0.0,
                             E._dtype_code(q), E._stream(dev)), "moba_fwd")
     torch.cuda.synchronize()
@@ -339,8 +359,9 @@ def test_history_keys_cut_into_parts(seqlens, heads, B, topk, dtype):
             _attention_stage(qg, kg, vg, plan, aux, False, bad)
 
 
+@pytest.mark.parametrize("dense", [False, True])
 @pytest.mark.parametrize("spread", [1.0, 8.0])
-def test_fixed_reference_softmax_and_redo_list(spread):
+def test_fixed_reference_softmax_and_redo_list(spread, dense):
     """A problem large enough for the resident-workgroup forward kernel (bf16): with a redo list the kernel takes
     each tile's softmax relative to a fixed per-row reference.  On N(0,1) data no tile leaves its range; with q
     and k scaled by 8 (logits of +-64 nats around zero, near one-hot rows) many do and are computed again by the
@@ -349,13 +370,15 @@ def test_fixed_reference_softmax_and_redo_list(spread):
     from moba_amd import moba_efficient as E
     from test_gpu_large import _row_oracle
     S, H, B, topk = 32768, 8, 1024, 3
-    _note("fixed reference", S, H, B, topk, spread)
+    _note("fixed reference", S, H, B, topk, spread, dense)
     g = torch.Generator(device="cuda").manual_seed(17)
     q, k, v = (torch.randn((S, H, 128), generator=g, device="cuda", dtype=torch.float32) for _ in range(3))
     q, k, v = (q * spread).to(torch.bfloat16), (k * spread).to(torch.bfloat16), v.to(torch.bfloat16)
-    plan = _plan([0, S], B, topk)
+    plan = _plan([0, S], B, topk, dense)
     sel = E.gate_topk(q, E.chunk_mean(k, plan), plan)
     aux = (sel,) + tuple(E.build_lists(sel, plan))
+    if dense:   # (the rows' attended sets, for the row oracle below: the plain plan's selection)
+        sel = E.gate_topk(q, E.chunk_mean(k, plan), _plan([0, S], B, topk))
     out_f, lse_f, n_redo = _attention_stage(q, k, v, plan, aux, True)
     out_m, lse_m, _ = _attention_stage(q, k, v, plan, aux, False)
     _note("  tiles computed again:", n_redo)

@@ -35,7 +35,7 @@ def test_plan_tables_match_oracle(seed):
     assert plan.P == int(sum(n * (n - 1) // 2 for n in m["n_chunks"]))
     assert plan.flops_per_head * 128 == pytest.approx(O.attention_flops(cu, B, topk, 1, 128))
     lens = np.diff(m["cu_chunk"])
-    assert plan.self_tiles == int(((lens + TILE_ROWS - 1) // TILE_ROWS).sum())
+    assert plan.self_tiles == plan.kv_tiles == int(((lens + TILE_ROWS - 1) // TILE_ROWS).sum())
     # every per-head self tile names its chunk: prefix[c] <= t < prefix[c+1]
     stc, pre = plan.host["self_tile_chunk"], plan.host["self_tile_prefix"]
     assert stc.size == plan.self_tiles
@@ -48,11 +48,69 @@ def test_plan_tables_match_oracle(seed):
     assert all(pre[c] <= t < pre[c + 1] for t, c in enumerate(stc.tolist()))
 
 
+def brute_force_dense(cu, B, K, d):
+    """Token-by-token restatement of the dense-prefix decomposition: attention chunk of every token, number of
+    list entries, and for every chunk where the causal rows of its keys end."""
+    achunk_starts, entries, self_end = [], 0, []
+    for a, b in zip(cu[:-1], cu[1:]):
+        n = -(-(b - a) // B)
+        prefix_end = min(b, a + (d + 1) * B)
+        achunk_starts.append(a)
+        for c in range(n):
+            lo, hi = a + c * B, min(b, a + (c + 1) * B)
+            if c > d:
+                achunk_starts.append(lo)
+                entries += (hi - lo) * min(K, c)
+                self_end.append(hi)
+            else:
+                self_end.append(prefix_end)
+    return achunk_starts + [cu[-1]], entries, self_end
+
+
+@pytest.mark.parametrize("seed", range(20))
+def test_dense_prefix_tables(seed):
+    """The plan with dense prefixes: chunks 0..K of every sequence form one attention chunk, their tokens have no
+    list entries, everything about the gate's chunks stays as it is."""
+    rng = np.random.default_rng(500 + seed)
+    cu = rand_cu(rng, int(rng.integers(1, 6)), 1, 600)
+    B = int(rng.integers(1, 80))
+    topk = int(rng.integers(2, 7))
+    plan = make_plan(cu, B, topk)
+    if plan.fallback:
+        assert plan.with_dense_prefix() is plan
+        return
+    assert plan.dense_local == 0 and plan.NA == plan.N and plan.kv_tiles == plan.self_tiles
+    assert np.array_equal(plan.host["achunk_tok"], plan.host["chunk_tok"])
+    assert np.array_equal(plan.host["chunk_self_end"], plan.host["chunk_tok"][1:])
+    assert np.array_equal(plan.host["kv_tile_prefix"], plan.host["self_tile_prefix"])
+    dense = plan.with_dense_prefix()
+    assert dense.dense_local == plan.K and dense.with_dense_prefix() is dense and plan.with_dense_prefix() is dense
+    for name in ("chunk_tok", "seq_fbase", "fchunk_tok", "chunk_fb", "chunk_local", "pair_off", "chunk_fid",
+                 "kv_tile_prefix", "kv_tile_chunk", "cu_seqlens"):
+        assert np.array_equal(dense.host[name], plan.host[name]), name
+    assert (dense.N, dense.F, dense.K, dense.P, dense.cmax, dense.kv_tiles) == \
+        (plan.N, plan.F, plan.K, plan.P, plan.cmax, plan.kv_tiles)
+    assert dense.flops_per_head == plan.flops_per_head
+    achunk, entries, self_end = brute_force_dense(cu, B, plan.K, plan.K)
+    assert dense.host["achunk_tok"].tolist() == achunk and dense.NA == len(achunk) - 1
+    assert dense.pairs_per_head == entries
+    assert dense.host["chunk_self_end"].tolist() == self_end
+    alen = np.diff(dense.host["achunk_tok"])
+    for rows, pre, chunk, count in ((TILE_ROWS, "self_tile_prefix", "self_tile_chunk", dense.self_tiles),
+                                    (FWD_TILE_ROWS, "fwd_self_tile_prefix", "fwd_self_tile_chunk", dense.fwd_self_tiles)):
+        assert count == int(((alen + rows - 1) // rows).sum()) == dense.host[chunk].size
+        assert np.array_equal(np.diff(dense.host[pre]), (alen + rows - 1) // rows)
+        assert all(dense.host[pre][c] <= t < dense.host[pre][c + 1] for t, c in enumerate(dense.host[chunk].tolist()))
+
+
 def test_plan_headline_config_sizes():
     plan = make_plan([0, 131072], 4096, 12)
     assert (plan.N, plan.F, plan.K, plan.P) == (32, 31, 11, 496)
     assert plan.pairs_per_head * 32 == 37486592
     assert plan.flops_per_head * 128 * 32 == pytest.approx(8.301e13, rel=1e-3)
+    dense = plan.with_dense_prefix()
+    assert (dense.NA, dense.dense_local) == (21, 11) and dense.host["achunk_tok"][:3].tolist() == [0, 49152, 53248]
+    assert dense.pairs_per_head == 20 * 4096 * 11 and dense.fwd_self_tiles == plan.fwd_self_tiles
 
 
 def test_plan_rejects_bad_input():
@@ -109,16 +167,20 @@ def test_c_planner_equals_python_planner(seed):
     if seed == 0:
         cu, B, topk = [0, 131072], 4096, 12
     plan = make_plan(cu, B, topk)
+    dense = seed % 2
+    if dense:
+        plan = plan.with_dense_prefix()
     cu_arr = (ctypes.c_int32 * len(cu))(*cu)
     ps, ps2 = _lib.PlanStruct(), _lib.PlanStruct()
-    assert lib.moba_plan(cu_arr, len(cu) - 1, B, topk, ctypes.byref(ps)) == 0
+    assert lib.moba_plan(cu_arr, len(cu) - 1, B, topk, dense, ctypes.byref(ps)) == 0
     tab = (ctypes.c_int32 * max(1, ps.table_ints))()
-    assert lib.moba_plan_fill(cu_arr, len(cu) - 1, B, topk, ctypes.byref(ps2), tab) == 0
+    assert lib.moba_plan_fill(cu_arr, len(cu) - 1, B, topk, dense, ctypes.byref(ps2), tab) == 0
     assert bytes(ps) == bytes(ps2)
     tab = np.frombuffer(tab, dtype=np.int32)
     assert (ps.S, ps.nseq, ps.N, ps.F, ps.K, ps.P, ps.cmax, bool(ps.fallback)) == \
         (plan.S, plan.nseq, plan.N, plan.F, plan.K, plan.P, plan.cmax, plan.fallback)
     assert (ps.pairs_per_head, ps.fwd_self_tiles, ps.bwd_self_tiles) == (plan.pairs_per_head, plan.fwd_self_tiles, plan.self_tiles)
+    assert (ps.dense_local, ps.NA, ps.kv_tiles) == (plan.dense_local, plan.NA, plan.kv_tiles)
     assert (ps.fwd_tile_rows, ps.bwd_tile_rows) == (FWD_TILE_ROWS, TILE_ROWS)
     assert ps.flops_per_head_per_dim == plan.flops_per_head
     seen = 0
@@ -146,6 +208,6 @@ def test_c_planner_rejects_bad_input():
     ps = _lib.PlanStruct()
     for cu in ([0, 5, 5, 9], [1, 5], [0, 4, 3]):
         arr = (ctypes.c_int32 * len(cu))(*cu)
-        assert lib.moba_plan(arr, len(cu) - 1, 4, 3, ctypes.byref(ps)) == -1
+        assert lib.moba_plan(arr, len(cu) - 1, 4, 3, 0, ctypes.byref(ps)) == -1
     arr = (ctypes.c_int32 * 2)(0, 8)
-    assert lib.moba_plan(arr, 1, 0, 3, ctypes.byref(ps)) == -1 and lib.moba_plan(arr, 1, 4, 0, ctypes.byref(ps)) == -1
+    assert lib.moba_plan(arr, 1, 0, 3, 0, ctypes.byref(ps)) == -1 and lib.moba_plan(arr, 1, 4, 0, 1, ctypes.byref(ps)) == -1
