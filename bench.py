@@ -29,9 +29,10 @@ sys.path.insert(0, ROOT)
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of moba_fwd_kernel from rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled by a copy
-# kernel of known size (profiles/moba_fwd_128k_hbm_traffic.txt); measured for the headline workload only
-FWD_KERNEL_TRAFFIC_BYTES = {"cfg4_L131072_h32_c4096_k12": 51.3e9}
+# HBM bytes per launch of moba_fwd_kernel come from rocprofv3 FETCH_SIZE / WRITE_SIZE, scaled by a copy kernel of
+# known size: a counter run of its own, whose summary (for the headline workload only) is this file; the figure
+# is read from its line "traffic_bytes_per_launch = <number>"
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "moba_fwd_128k_hbm_traffic.txt")
 
 WORKLOADS = {
     # name: (seq lens or None, heads, kv_heads, chunk, topk, normalise, backward)
@@ -40,6 +41,8 @@ WORKLOADS = {
     "cfg3_varlen8_h32_c2048_k3": (None, 32, 32, 2048, 3, False, True),
     "cfg4_L131072_h32_c4096_k12": ([131072], 32, 8, 4096, 12, True, False),
     "cfg5_L1048576_h32_c4096_k12": ([1048576], 32, 8, 4096, 12, False, False),
+    # the default shape of the reference's speed script (tests/test_moba_speedup.py:84)
+    "speedscript_L32768_h1_c512_k3": ([32768], 1, 1, 512, 3, False, True),
 }
 DEFAULT = "cfg4_L131072_h32_c4096_k12"
 
@@ -122,13 +125,60 @@ def bench_decode(dev, skv, heads, kv_heads=8, iters=50):
                          "frac": gbs / HBM_PEAK_GBS}}
 
 
-def quick_measure(name, dev, steps, warmup, backward):
+def traffic_from_profile(workload):
+    """HBM bytes per launch of the dominant kernel, as the committed counter profile states them (None if it does
+    not cover this workload)."""
+    if workload != DEFAULT or not os.path.exists(TRAFFIC_PROFILE):
+        return None
+    for line in open(TRAFFIC_PROFILE):
+        if line.strip().startswith("traffic_bytes_per_launch"):
+            return float(line.split("=")[1].split()[0])
+    return None
+
+
+def mfma_ceiling(dev, iters=40000):
+    """What the chip's matrix pipes sustain when they do nothing else, on this box, now: a register-resident loop
+    of v_mfma_f32_32x32x16_bf16 on every compute unit (eight waves each, as the forward kernel runs), once on
+    constant operands and once on random bf16 N(0,1) operands.  The clock the chip holds at its power limit depends
+    on how much the multipliers' inputs toggle, so the second figure, not the published peak, is the ceiling of any
+    kernel that multiplies real data."""
+    import ctypes
+    from moba_amd import _lib
+    lib = _lib.load()
+    sink = torch.zeros(1, dtype=torch.float32, device=dev)
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    flops = cus * 8 * iters * 16 * 32768.0
+    stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    out = {"kernel": "mfma_probe_kernel", "workgroups": cus, "waves_per_workgroup": 8, "unit": "TFLOP/s",
+           "peak": MFMA_BF16_PEAK_TFLOPS}
+    g = torch.Generator(device=dev).manual_seed(3)
+    for name, data in (("constant_operands", torch.ones(8192, device=dev, dtype=torch.bfloat16)),
+                       ("random_bf16_operands", torch.randn(8192, generator=g, device=dev).to(torch.bfloat16))):
+        best = None
+        for _ in range(4):   # (about 10 ms each: long enough for the clock to settle at the power limit)
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            _lib.check(lib.moba_mfma_probe(ctypes.c_void_p(data.data_ptr()), ctypes.c_void_p(sink.data_ptr()), iters, 0,
+                                           stream), "moba_mfma_probe")
+            b.record()
+            torch.cuda.synchronize()
+            ms = a.elapsed_time(b)
+            best = ms if best is None else min(best, ms)
+        out[name] = flops / (best * 1e-3) / 1e12
+    out["random_frac_of_peak"] = out["random_bf16_operands"] / MFMA_BF16_PEAK_TFLOPS
+    return out
+
+
+def quick_measure(name, dev, steps, warmup, backward, dtype=torch.bfloat16, topk=None):
     """Forward (and forward + backward) time of one of the other workloads, a few steps each: wall clock around
-    the steps, bracketed by synchronisations, like the headline figure."""
+    the steps, bracketed by synchronisations, like the headline figure.  topk overrides the workload's
+    (topk = 1: full causal attention through the same operator)."""
     from moba_amd import moba_efficient as E
     from moba_amd.plan import make_plan
 
-    q, k, v, cu, max_seqlen, B, topk = make_inputs(name, dev)
+    q, k, v, cu, max_seqlen, B, topk0 = make_inputs(name, dev)
+    topk = topk0 if topk is None else topk
+    q, k, v = (x.to(dtype) for x in (q, k, v))
     S, H, D = q.shape
     cu_t = torch.tensor(cu, dtype=torch.int32, device=dev)
     flops = make_plan(cu_t, B, topk).flops_per_head * D * H
@@ -149,7 +199,7 @@ def quick_measure(name, dev, steps, warmup, backward):
            "fwd_ms": fwd_ms, "fwd_tflops": flops / (fwd_ms * 1e-3) / 1e12}
     if backward:
         g = torch.Generator(device=dev).manual_seed(1)
-        do = torch.randn(q.shape, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+        do = torch.randn(q.shape, generator=g, device=dev, dtype=torch.float32).to(dtype)
         qg, kg, vg = (x.requires_grad_(True) for x in (q, k, v))
 
         def both():
@@ -175,6 +225,7 @@ def main():
                          "8 KV heads) next to PyTorch SDPA")
     ap.add_argument("--no-other-configs", action="store_true",
                     help="with the default workload: do not also time the other BASELINE configurations")
+    ap.add_argument("--no-ceiling", action="store_true", help="do not run the matrix-pipe ceiling probe")
     ap.add_argument("--gqa", action="store_true",
                     help="keep the key/value heads unexpanded (grouped-query operator) instead of the reference "
                          "wrapper's repeat_kv; not the headline configuration")
@@ -265,8 +316,14 @@ def main():
         "device_ms_per_step": {"median": step_ms[len(step_ms) // 2], "min": step_ms[0]},
         "roofline": {"kernel": "moba_fwd_kernel", "bound": "mfma", "achieved": achieved,
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
-                     "traffic": FWD_KERNEL_TRAFFIC_BYTES.get(args.workload)},
+                     "traffic": traffic_from_profile(args.workload),
+                     "traffic_source": "profiles/moba_fwd_128k_hbm_traffic.txt (rocprofv3 counter runs of this "
+                                       "workload; not measured in this run)"},
     }
+    if not args.no_ceiling:
+        # the same box, the same minute: what the matrix pipes sustain with nothing else to do
+        result["mfma_ceiling"] = mfma_ceiling(dev)
+        result["roofline"]["frac_of_random_operand_ceiling"] = achieved / result["mfma_ceiling"]["random_bf16_operands"]
     if fwd_bwd_ms is not None:
         # algorithmic backward work is 2.5x the forward's
         result["fwd_bwd"] = {"ms_per_step": fwd_bwd_ms, "tflops": 3.5 * flops / (fwd_bwd_ms * 1e-3) / 1e12,
@@ -284,8 +341,23 @@ def main():
         torch.cuda.empty_cache()
         result["other_configs"] = {}
         for name, steps, warmup in (("cfg1_L4096_h4_c512_k3", 200, 20), ("cfg2_L32768_h1_c2048_k3", 200, 20),
+                                    ("speedscript_L32768_h1_c512_k3", 200, 20),
                                     ("cfg3_varlen8_h32_c2048_k3", 3, 1), ("cfg5_L1048576_h32_c4096_k12", 2, 1)):
             result["other_configs"][name] = quick_measure(name, dev, steps, warmup, backward=True)
+            torch.cuda.empty_cache()
+        # the headline shape in fp16 (the dtype of the reference's example, examples/llama.py:26)
+        result["other_configs"]["cfg4_fp16"] = quick_measure(DEFAULT, dev, 5, 2, backward=False, dtype=torch.float16)
+        torch.cuda.empty_cache()
+        # Full causal attention through the same operator (moba_topk = 1) beside MoBA: the ratio the reference's
+        # report plots (full FlashAttention / MoBA forward time: 1.19x at 128K, 6.5x at 1M tokens, on its hardware)
+        result["full_attention"] = {}
+        for name, steps, warmup, published in (("cfg2_L32768_h1_c2048_k3", 50, 5, None), (DEFAULT, 3, 1, 1.19),
+                                               ("cfg5_L1048576_h32_c4096_k12", 1, 1, 6.5)):
+            full = quick_measure(name, dev, steps, warmup, backward=False, topk=1)
+            moba_ms = dt * 1e3 if name == DEFAULT else result["other_configs"][name]["fwd_ms"]
+            result["full_attention"][name] = {"full_fwd_ms": full["fwd_ms"], "full_fwd_tflops": full["fwd_tflops"],
+                                              "moba_fwd_ms": moba_ms, "full_over_moba": full["fwd_ms"] / moba_ms,
+                                              "report_full_over_moba": published}
             torch.cuda.empty_cache()
         q, k, v, cu, max_seqlen, B, topk = make_inputs(args.workload, dev, args.gqa)   # for the CPU baseline's sample
     if not args.no_cpu_baseline:

@@ -300,6 +300,14 @@ int moba_decode(const void* q, const void* k, const void* v, void* out, float* p
                 int Hkv, int Skv, int D, int64_t q_stride_b, int64_t q_stride_h, int64_t kv_stride_b,
                 int64_t kv_stride_h, float scale, int dtype, void* stream);
 
+/* Measurement aid, no counterpart in the reference: what the matrix pipes sustain when they do nothing else.
+ * Launches `workgroups` workgroups (0: one per compute unit) of eight waves, two per SIMD as in the forward kernel;
+ * every wave issues iters * 16 v_mfma_f32_32x32x16_bf16 on sixteen operand registers it loads once from
+ * `operands` (16 KiB of bf16 on the device: constant or random data, the caller's choice) -- no LDS, no memory
+ * traffic, no vector work.  Flops = workgroups * 8 * iters * 16 * 32768; the caller times the launch on
+ * `stream`.  sink: one float on the device (never written in practice). */
+int moba_mfma_probe(const void* operands, float* sink, int iters, int workgroups, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -51,6 +51,7 @@ _SIGNATURES = {
     "moba_bwd_dq_key_split": (c_int, [c_int64, c_int, c_int, c_int, c_int64, c_int64]),
     "moba_bwd": (c_int, [c_void_p] * 25 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_int64,
                                           c_int64, c_int, c_strides, c_void_p, c_void_p, c_int64, c_float, c_int, c_void_p]),
+    "moba_mfma_probe": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "moba_decode_splits": (c_int, [c_int, c_int, c_int]),
     "moba_decode": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_int64] * 4 + [c_float, c_int, c_void_p]),
 }

@@ -14,7 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(CSRC, "build")
 LIB = os.path.join(HERE, "libmoba_hip.so")
-SOURCES = ["chunk_mean.hip", "gate_topk.hip", "lists.hip", "fwd.hip", "bwd.hip", "decode.hip", "plan.hip", "capi.hip"]
+SOURCES = ["chunk_mean.hip", "gate_topk.hip", "lists.hip", "fwd.hip", "bwd.hip", "decode.hip", "plan.hip", "probe.hip", "capi.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
