@@ -55,7 +55,7 @@ extern "C" {
 
 enum { MOBA_DTYPE_BF16 = 0, MOBA_DTYPE_F16 = 1 };
 
-#define MOBA_ABI_VERSION 112 /* the signatures below; moba_version() returns the number the library was built with */
+#define MOBA_ABI_VERSION 113 /* the signatures below; moba_version() returns the number the library was built with */
 int moba_version(void);
 const char* moba_strerror(int code);
 
@@ -78,7 +78,8 @@ const char* moba_strerror(int code);
  * Tables: cu_seqlens, chunk_tok [N+1], achunk_tok [NA+1] (first token of every attention chunk: the chunk_tok
  * argument of moba_fwd* and moba_bwd), fwd_self_tile_prefix [NA+1] / fwd_self_tile_chunk (the self_tile_* arguments of
  * moba_fwd*), self_tile_prefix [NA+1] / self_tile_chunk (those of moba_bwd), kv_tile_prefix [N+1] / kv_tile_chunk
- * and chunk_self_end [N] (moba_bwd), seq_fbase [nseq+1], fchunk_tok [F], chunk_fb [N], chunk_local [N], pair_off [F+1],
+ * and chunk_self_end [N] (moba_bwd), achunk_direct [NA] (the chunk_direct argument of moba_fwd*), mrg_start [nseq] and
+ * mrg_prefix [nseq+1] (moba_fwd_merge), seq_fbase [nseq+1], fchunk_tok [F], chunk_fb [N], chunk_local [N], pair_off [F+1],
  * chunk_fid [N].
  * moba_plan_sizes gives, for H query and Hkv key/value heads, the size of every scratch buffer of the calls below. */
 typedef struct moba_plan_t {
@@ -92,10 +93,11 @@ typedef struct moba_plan_t {
   int64_t pairs_per_head;                  /* M = pairs_per_head * H */
   int64_t fwd_self_tiles, bwd_self_tiles;  /* the self_tiles arguments of moba_fwd* and of moba_bwd */
   int64_t kv_tiles;                        /* the kv_tiles argument of moba_bwd */
+  int64_t merge_tokens;                    /* the merge_tokens argument of moba_fwd_merge */
   double flops_per_head_per_dim;           /* forward flops = this * H * D */
   int64_t off_cu_seqlens, off_chunk_tok, off_achunk_tok, off_fwd_self_tile_prefix, off_fwd_self_tile_chunk,
       off_self_tile_prefix, off_self_tile_chunk, off_kv_tile_prefix, off_kv_tile_chunk, off_chunk_self_end,
-      off_seq_fbase, off_fchunk_tok, off_chunk_fb, off_chunk_local, off_pair_off, off_chunk_fid;
+      off_achunk_direct, off_mrg_start, off_mrg_prefix, off_seq_fbase, off_fchunk_tok, off_chunk_fb, off_chunk_local, off_pair_off, off_chunk_fid;
   int64_t table_ints;
 } moba_plan_t;
 typedef struct moba_sizes_t {
@@ -214,6 +216,13 @@ int moba_tile_tables(const int32_t* seg_off, int32_t* tile_off, int32_t* tile_se
  *   tile_off, tile_seg: from moba_build_lists or moba_tile_tables with tile_rows = moba_fwd_tile_rows()
  *              (may be NULL when K = 0)
  *   out [S,H,D] elem, lse [S,H] fp32 (natural log)
+ *   chunk_direct [N] int32 or NULL: 1 for an attention chunk whose rows have no history slots (the first one of
+ *              every sequence: the plan's achunk_direct).  moba_fwd_partials writes the result of such a chunk's
+ *              rows straight into out and lse (there is nothing to merge it with) instead of into slot 0, and
+ *              moba_fwd_merge is told to leave those rows alone: mrg_start [nranges] / mrg_prefix [nranges+1] name the
+ *              token ranges it walks (range b: tokens mrg_start[b] + i, i < mrg_prefix[b+1] - mrg_prefix[b]) and
+ *              merge_tokens = mrg_prefix[nranges] their number (0: no launch at all, e.g. with K = 0).  NULL, NULL,
+ *              NULL, 0 and merge_tokens = S: every row goes through its slot and the merge.
  *   hist_bound: upper bound on the number of history tiles, e.g. M / moba_fwd_tile_rows() + F*H
  *   self_tiles: self_tile_prefix[N]
  *   queues [8] int32 scratch: the tile counters of the forward kernel, whose workgroups (one per CU) stay
@@ -233,12 +242,13 @@ int moba_bwd_tile_rows(void);
 int moba_fwd_partials(const void* q, const void* k, const void* v, void* part_o, float* part_lse,
                       const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest,
                       const int32_t* fchunk_tok, const int32_t* chunk_tok, const int32_t* self_tile_prefix,
-                      const int32_t* tile_seg, const int32_t* self_tile_chunk, int64_t S, int H, int Hkv, int D, int K,
-                      int F, int N, int B, int64_t hist_bound, int64_t self_tiles, int key_split,
-                      const int64_t* strides, int32_t* queues, int32_t* redo, float softmax_scale, int dtype,
-                      void* stream);
+                      const int32_t* tile_seg, const int32_t* self_tile_chunk, const int32_t* chunk_direct, void* out,
+                      float* lse, int64_t S, int H, int Hkv, int D, int K, int F, int N, int B, int64_t hist_bound,
+                      int64_t self_tiles, int key_split, const int64_t* strides, int32_t* queues, int32_t* redo,
+                      float softmax_scale, int dtype, void* stream);
 int moba_fwd_merge(const void* part_o, const float* part_lse, const int32_t* sel, void* out, float* lse, int64_t S,
-                   int H, int D, int K, int key_split, int dtype, void* stream);
+                   int H, int D, int K, int key_split, const int32_t* mrg_start, const int32_t* mrg_prefix, int nranges,
+                   int64_t merge_tokens, int dtype, void* stream);
 int moba_fwd_key_split(int64_t S, int H, int K, int B, int64_t hist_bound, int64_t self_tiles);
 /* 1 if moba_fwd_partials would run a problem of hist_bound + self_tiles * H tiles with resident workgroups drawing
  * from the tile queues, 0 if with one workgroup per tile (no counterpart in the reference). */
@@ -246,9 +256,10 @@ int moba_fwd_is_queued(int64_t hist_bound, int64_t self_tiles, int H);
 int moba_fwd(const void* q, const void* k, const void* v, void* part_o, float* part_lse, const int32_t* sel,
              const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest, const int32_t* fchunk_tok,
              const int32_t* chunk_tok, const int32_t* self_tile_prefix, const int32_t* tile_seg,
-             const int32_t* self_tile_chunk, void* out, float* lse, int64_t S, int H, int Hkv, int D, int K, int F,
-             int N, int B, int64_t hist_bound, int64_t self_tiles, int key_split, const int64_t* strides,
-             int32_t* queues, int32_t* redo, float softmax_scale, int dtype, void* stream);
+             const int32_t* self_tile_chunk, const int32_t* chunk_direct, const int32_t* mrg_start,
+             const int32_t* mrg_prefix, int nranges, int64_t merge_tokens, void* out, float* lse, int64_t S, int H,
+             int Hkv, int D, int K, int F, int N, int B, int64_t hist_bound, int64_t self_tiles, int key_split,
+             const int64_t* strides, int32_t* queues, int32_t* redo, float softmax_scale, int dtype, void* stream);
 
 /* Backward.  Replaces MixedAttention.backward, moba/moba_efficient.py:185-267, and the
  * autograd scatter of its gathered gradients.  Deterministic (no floating-point atomics).

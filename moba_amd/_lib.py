@@ -39,13 +39,15 @@ _SIGNATURES = {
     "moba_tile_tables": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int64, c_void_p]),
     "moba_fwd_tile_rows": (c_int, []),
     "moba_bwd_tile_rows": (c_int, []),
-    "moba_fwd_partials": (c_int, [c_void_p] * 13 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int64,
+    "moba_fwd_partials": (c_int, [c_void_p] * 16 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int64,
                                                    c_int64, c_int, c_strides, c_void_p, c_void_p, c_float, c_int,
                                                    c_void_p]),
-    "moba_fwd_merge": (c_int, [c_void_p] * 5 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "moba_fwd_merge": (c_int, [c_void_p] * 5 + [c_int64, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_int64,
+                                               c_int, c_void_p]),
     "moba_fwd_key_split": (c_int, [c_int64, c_int, c_int, c_int, c_int64, c_int64]),
     "moba_fwd_is_queued": (c_int, [c_int64, c_int64, c_int]),
-    "moba_fwd": (c_int, [c_void_p] * 16 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_int64,
+    "moba_fwd": (c_int, [c_void_p] * 17 + [c_int, c_int64, c_void_p, c_void_p,
+                                          c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_int64,
                                           c_int, c_strides, c_void_p, c_void_p, c_float, c_int, c_void_p]),
     "moba_bwd_dkv_scratch_bytes": (ctypes.c_size_t, [c_int64, c_int, c_int64]),
     "moba_bwd_dq_key_split": (c_int, [c_int64, c_int, c_int, c_int, c_int64, c_int64]),
@@ -63,10 +65,11 @@ class PlanStruct(ctypes.Structure):
     _fields_ = ([("S", c_int64)] + [(n, ctypes.c_int32) for n in ("nseq", "chunk", "topk", "N", "F", "K", "P", "cmax", "fallback",
                                                                "fwd_tile_rows", "bwd_tile_rows", "dense_local", "NA")]
                 + [("pairs_per_head", c_int64), ("fwd_self_tiles", c_int64), ("bwd_self_tiles", c_int64),
-                   ("kv_tiles", c_int64), ("flops_per_head_per_dim", ctypes.c_double)]
+                   ("kv_tiles", c_int64), ("merge_tokens", c_int64), ("flops_per_head_per_dim", ctypes.c_double)]
                 + [("off_" + n, c_int64) for n in ("cu_seqlens", "chunk_tok", "achunk_tok", "fwd_self_tile_prefix",
                                                    "fwd_self_tile_chunk", "self_tile_prefix", "self_tile_chunk",
-                                                   "kv_tile_prefix", "kv_tile_chunk", "chunk_self_end", "seq_fbase",
+                                                   "kv_tile_prefix", "kv_tile_chunk", "chunk_self_end", "achunk_direct",
+                                                   "mrg_start", "mrg_prefix", "seq_fbase",
                                                    "fchunk_tok", "chunk_fb", "chunk_local", "pair_off", "chunk_fid")]
                 + [("table_ints", c_int64)])
 
@@ -76,7 +79,7 @@ class SizesStruct(ctypes.Structure):
     _fields_ = [(n, c_int64) for n in ("kbar_elems", "chunk_mean_workspace_bytes", "sel_ints", "cnt_ints", "seg_off_ints",
                                        "seg_dest_ints", "fwd_hist_bound", "bwd_hist_bound", "part_rows", "redo_ints",
                                        "lse_floats", "delta_floats")]
-ABI_VERSION = 112  # MOBA_ABI_VERSION of include/moba_hip.h, the signatures above
+ABI_VERSION = 113  # MOBA_ABI_VERSION of include/moba_hip.h, the signatures above
 DTYPE_BF16, DTYPE_F16 = 0, 1
 
 

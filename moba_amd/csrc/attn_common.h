@@ -26,6 +26,10 @@ struct TileTables {
   const int* self_tile_prefix;  // [N+1] prefix sum of row tiles per chunk
   const int* tile_seg;          // [hist_bound] segment (f*H + h) of every history tile, -1 past the last one
   const int* self_tile_chunk;   // [self_tile_prefix[N]] chunk of every per-head self tile
+  // [N] or null: 1 for a chunk whose rows have no history slots at all (the first attention chunk of a sequence).
+  // The forward kernel writes the result of such a chunk's self tiles straight into the operator's outputs: there
+  // is nothing to merge it with.  Null (the backward): every tile writes its slot row.
+  const int* chunk_direct;
   int S, H, K1, F, N, B;
   int Hkv, rep;                 // key/value heads and query heads per key/value head (H = Hkv * rep)
   int hist_bound;               // logical tile ids below it are history tiles
@@ -64,6 +68,7 @@ __device__ __forceinline__ int64_t kv_tok_bytes(const TileTables& t, int tok) {
 constexpr int kStrideEntries = 7;
 inline bool set_layout(TileTables& t, const int64_t* strides) {
   t.batch_rows = 0; t.q_batch_b = 0; t.kv_batch_b = 0;
+  t.chunk_direct = nullptr;
   t.key_split_log2 = 0; t.part_stride = 0; t.xcd_block_log2 = 6; t.self_first = 0;
   if (!strides) {
     t.q_tok_b = (int64_t)t.H * kHeadDim * 2; t.q_head_b = kHeadDim * 2;
@@ -96,6 +101,7 @@ struct Tile {
   int wave_min_limit, wave_max_limit;  // over the wave's 32 rows
   int rot;        // history tiles may visit their key tiles in any order: start offset
   int base;       // history tile: index of row 0 in seg_dest; self tile: -(row 0 inside the chunk) - 1
+  int direct;     // self tile of a chunk without history slots: dest is the output row token*H + h
 };
 
 // the tile counters of a kernel whose resident workgroups draw their tiles from per-XCD queues start at zero
@@ -135,9 +141,10 @@ __device__ __forceinline__ int decode_tile_code(const TileTables& p, int logical
 struct TileHeadEntries {
   int a, b, c, d;  // history tile: tile_off[seg], seg_off[seg], seg_off[seg+1], fchunk_tok[f];
                    // self tile: self_tile_prefix[c], self_tile_prefix[c+1], chunk_tok[c], chunk_tok[c+1]
+  int e;           // self tile: chunk_direct[c] (0 without that table)
 };
 __device__ __forceinline__ TileHeadEntries tile_head_entries(const TileTables& p, int logical, int code) {
-  TileHeadEntries e = {0, 0, 0, 0};
+  TileHeadEntries e = {0, 0, 0, 0, 0};
   if (code < 0) return e;
   if (logical < p.hist_bound) {
     e.a = table_load(p.tile_off + code);
@@ -149,6 +156,7 @@ __device__ __forceinline__ TileHeadEntries tile_head_entries(const TileTables& p
     e.b = table_load(p.self_tile_prefix + code + 1);
     e.c = table_load(p.chunk_tok + code);
     e.d = table_load(p.chunk_tok + code + 1);
+    if (p.chunk_direct) e.e = table_load(p.chunk_direct + code);
   }
   return e;
 }
@@ -158,6 +166,7 @@ __device__ __forceinline__ bool decode_tile_head(const TileTables& p, int logica
   t.id = logical;
   t.row_count = 0;
   t.base = -1;
+  t.direct = 0;
   if (code < 0) return false;
   if (logical < p.hist_bound) {
     const int seg = code;
@@ -183,6 +192,7 @@ __device__ __forceinline__ bool decode_tile_head(const TileTables& p, int logica
   t.kv_tok0 = c0;
   t.nkeys = min(len, tin * tm + tm);
   t.rot = 0;
+  t.direct = e.e;
   return true;
 }
 __device__ __forceinline__ bool decode_tile_head(const TileTables& p, int logical, int code, Tile& t, int tm = TM) {
@@ -207,7 +217,7 @@ __device__ __forceinline__ void decode_tile_rows(const TileTables& p, int wave, 
   } else {
     const int r0 = -1 - t.base;
     t.tok = t.kv_tok0 + r0 + min(r, t.row_count - 1);
-    t.dest = (t.tok * H + t.h) * p.K1;
+    t.dest = t.direct ? t.tok * H + t.h : (t.tok * H + t.h) * p.K1;
     t.limit = r0 + min(r, t.row_count - 1);
     t.wave_min_limit = r0 + min(wave * 32, t.row_count - 1);
     t.wave_max_limit = r0 + min(wave * 32 + 31, t.row_count - 1);

@@ -40,6 +40,8 @@ struct FwdParams {
   const typename E::elem* v;
   typename E::elem* part_o;  // [S*H*K1, D]
   float* part_lse;  // [S*H*K1], log2 domain
+  typename E::elem* out;     // [S*H, D]: where the tiles of chunks without history slots (TileTables::chunk_direct) write
+  float* lse;                // [S*H], natural log
   TileTables t;
   float scale_log2;  // D^-0.5 * log2(e)
   int* queues;       // [8] tile counters, one per XCD, zero when the kernel starts
@@ -99,11 +101,11 @@ __global__ __launch_bounds__(512, 2) void moba_fwd_kernel(const FwdParams<E> p) 
   const int r = wave * 32 + n;
   Tile t, t1;              // the tile being computed; the next one (its row entries on their way to LDS)
   int id1 = -1, code1 = kTileUnused;   // id and first lookup of the next tile
-  TileHeadEntries head1 = {0, 0, 0, 0};  // its small-table entries
+  TileHeadEntries head1 = {0, 0, 0, 0, 0};  // its small-table entries
   int id2 = -1, code2 = kTileUnused;   // id and first lookup of the tile after next
   int id3 = -1;                        // id of the tile after that, as drawn
   int queue = blockIdx.x & 7, empty_queues = 0;
-  t.row_count = 0; t.nkeys = 0; t.base = -1; t1 = t;   // row_count 0: not a tile; nkeys < 0: no tiles left
+  t.row_count = 0; t.nkeys = 0; t.base = -1; t.direct = 0; t1 = t;   // row_count 0: not a tile; nkeys < 0: no tiles left
   int h = 0, nkeys = 0, kv_tok0 = 0, hkv = 0;
   int min_limit = 0;       // smallest row limit of the wave's 32 rows
   bool row_valid = false;
@@ -239,7 +241,7 @@ __global__ __launch_bounds__(512, 2) void moba_fwd_kernel(const FwdParams<E> p) 
   // other word.  The word of pass i is rewritten in pass i + 2, behind the barrier of pass i + 1.
   int id_word = 0;
   int dest_done = 0, rows_done = 0, id_done = 0;
-  bool valid_done = false;
+  bool valid_done = false, direct_done = false;  // (direct: the tile's rows go straight to the outputs)
   int list_pos = blockIdx.x;  // kTilesListed: position in the list of the next tile
   int key_part = 0;           // kTilePerGroup: which part of a history tile's keys this workgroup takes
   if constexpr (kFixedRef) {
@@ -265,7 +267,13 @@ __global__ __launch_bounds__(512, 2) void moba_fwd_kernel(const FwdParams<E> p) 
     char* stage = smem + (wave_u < 4 ? 2 * kTileBytes + wave_u * 4096 : kFwdVBase + 2 * kTileBytes + (wave_u - 4) * 4096);
     char* wrow = stage + en * 128 + 8 * ehh;
     const int wsw = (en >> 1) & 7;  // rows 128 bytes apart: the 16-byte column is swizzled by the row pair
-    if (valid_done && ehh == 0) pn.part_lse[dest_done] = m_run + fast_log2(l_tot);
+    // a tile of a chunk without history slots writes the operator's outputs (natural-log LSE), any other its slot row
+    elem* const o_base = direct_done ? pn.out : pn.part_o;
+    if (valid_done && ehh == 0) {
+      const float l2 = m_run + fast_log2(l_tot);
+      if (direct_done) pn.lse[dest_done] = l2 * 0.6931471805599453f;
+      else pn.part_lse[dest_done] = l2;
+    }
     const int c16 = ln & 7;
     int dest[4];
 #pragma unroll
@@ -287,7 +295,7 @@ __global__ __launch_bounds__(512, 2) void moba_fwd_kernel(const FwdParams<E> p) 
       for (int i = 0; i < 4; ++i) {
         const int row = 8 * i + (ln >> 3);
         const u32x4 x = *reinterpret_cast<const u32x4*>(stage + row * 128 + ((c16 ^ ((row >> 1) & 7)) << 4));
-        if (row < rows_done) *reinterpret_cast<u32x4*>(pn.part_o + (int64_t)dest[i] * kHeadDim + 64 * half + c16 * 8) = x;
+        if (row < rows_done) *reinterpret_cast<u32x4*>(o_base + (int64_t)dest[i] * kHeadDim + 64 * half + c16 * 8) = x;
       }
     }
   };
@@ -481,6 +489,7 @@ __global__ __launch_bounds__(512, 2) void moba_fwd_kernel(const FwdParams<E> p) 
     continue;
   }
   dest_done = t.dest;
+  direct_done = t.direct != 0;
   id_done = t.id;
   valid_done = row_valid;
   rows_done = t.row_count - wave_u * 32;  // rows of this wave that exist
@@ -691,15 +700,25 @@ __global__ __launch_bounds__(512, 2) void moba_fwd_kernel(const FwdParams<E> p) 
 
 // Combine the K1 slots of each (token, head): slot 0 is the self part, slot 1+j the
 // j-th selected history chunk (present iff sel[row, j] >= 0).  16 lanes per row.
+// With token ranges (mrg_start / mrg_prefix [nranges(+1)]: range b holds the tokens mrg_start[b] + i for
+// i < mrg_prefix[b+1] - mrg_prefix[b]) only the rows of those tokens are merged, `rows` counting them: the others
+// were written by the attention kernel itself.  Null: every row of [0, rows).
 template <class E>
 __global__ __launch_bounds__(256) void moba_merge_kernel(const typename E::elem* __restrict__ part_o,
                                                          const float* __restrict__ part_lse,
                                                          const int* __restrict__ sel, typename E::elem* __restrict__ out,
-                                                         float* __restrict__ lse, int64_t rows, int K1, int parts) {
+                                                         float* __restrict__ lse, int64_t rows, int K1, int parts,
+                                                         int64_t all_rows, const int* __restrict__ mrg_start,
+                                                         const int* __restrict__ mrg_prefix, int nranges, int H) {
   MOBA_ELEM_TYPES(E)
   const int64_t row_raw = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
   const bool row_ok = row_raw < rows;
-  const int64_t row = row_ok ? row_raw : rows - 1;  // whole 16-lane groups stay active for the shuffles
+  int64_t row = row_ok ? row_raw : rows - 1;  // whole 16-lane groups stay active for the shuffles
+  if (mrg_start) {
+    const int t = (int)(row / H), h = (int)(row - (int64_t)t * H);
+    const int b = upper_row(mrg_prefix, nranges, t);
+    row = (int64_t)(mrg_start[b] + (t - mrg_prefix[b])) * H + h;
+  }
   const int c8 = threadIdx.x & 15;
   const int K = K1 - 1;
   const float* pl = part_lse + row * K1;
@@ -714,7 +733,7 @@ __global__ __launch_bounds__(256) void moba_merge_kernel(const typename E::elem*
   // The parts are slots like any other: slot v of the parts * K1 is slot v % K1 of part v / K1, at slot row
   // (v / K1) * rows * K1 + v % K1 of the row's first (an int: the buffers hold fewer than 2^31 slot rows).
   const int nvirt = parts * K1;
-  const int part_rows = (int)(rows * K1);
+  const int part_rows = (int)(all_rows * K1);
   float mx = -INFINITY;
   for (int v0 = 0; v0 < nvirt; v0 += 16) {
     const int v = v0 + c8;
@@ -813,13 +832,14 @@ extern "C" int moba_fwd_key_split(int64_t S, int H, int K, int B, int64_t hist_b
 }
 
 template <class E>
-static int launch_partials(const void* q, const void* k, const void* v, void* part_o, float* part_lse,
-                           const TileTables& t, int D, float softmax_scale, int64_t grid, int* queues, int* redo,
-                           hipStream_t st) {
+static int launch_partials(const void* q, const void* k, const void* v, void* part_o, float* part_lse, void* out,
+                           float* lse, const TileTables& t, int D, float softmax_scale, int64_t grid, int* queues,
+                           int* redo, hipStream_t st) {
   LaunchCheck launch_check;
   FwdParams<E> p;
   p.q = (const typename E::elem*)q; p.k = (const typename E::elem*)k; p.v = (const typename E::elem*)v;
   p.part_o = (typename E::elem*)part_o; p.part_lse = part_lse;
+  p.out = (typename E::elem*)out; p.lse = lse;
   p.t = t;
   p.scale_log2 = softmax_scale > 0.f ? (float)(1.4426950408889634 * (double)softmax_scale)
                                      : (float)(1.4426950408889634 / sqrt((double)D));
@@ -853,12 +873,14 @@ extern "C" int moba_fwd_partials(const void* q, const void* k, const void* v, vo
                                  const int32_t* seg_off, const int32_t* tile_off, const int32_t* seg_dest,
                                  const int32_t* fchunk_tok, const int32_t* chunk_tok,
                                  const int32_t* self_tile_prefix, const int32_t* tile_seg,
-                                 const int32_t* self_tile_chunk, int64_t S, int H, int Hkv, int D, int K, int F,
+                                 const int32_t* self_tile_chunk, const int32_t* chunk_direct, void* out, float* lse,
+                                 int64_t S, int H, int Hkv, int D, int K, int F,
                                  int N, int B, int64_t hist_bound, int64_t self_tiles, int key_split,
                                  const int64_t* strides, int32_t* queues, int32_t* redo, float softmax_scale,
                                  int dtype, void* stream) {
   if (!q || !k || !v || !part_o || !part_lse || !chunk_tok || !self_tile_prefix || !self_tile_chunk || !queues)
     return MOBA_ERR_ARG;
+  if (chunk_direct && (!out || !lse || ((uintptr_t)out & 15))) return MOBA_ERR_ARG;
   if (Hkv <= 0 || H % Hkv != 0) return MOBA_ERR_ARG;
   if (K > 0 && (!seg_off || !tile_off || !seg_dest || !fchunk_tok || !tile_seg)) return MOBA_ERR_ARG;
   if (D != kHeadDim || (dtype != MOBA_DTYPE_BF16 && dtype != MOBA_DTYPE_F16)) return MOBA_ERR_UNSUPPORTED;
@@ -893,28 +915,36 @@ extern "C" int moba_fwd_partials(const void* q, const void* k, const void* v, vo
   t.part_stride = (int)(S * H * (K + 1));
   t.xcd_block_log2 = fwd_xcd_block_log2(total);
   t.self_first = key_split > 1;
+  t.chunk_direct = chunk_direct;
   hipStream_t st = (hipStream_t)stream;
   return dtype == MOBA_DTYPE_F16
-             ? launch_partials<F16>(q, k, v, part_o, part_lse, t, D, softmax_scale, grid, queues, redo, st)
-             : launch_partials<Bf16>(q, k, v, part_o, part_lse, t, D, softmax_scale, grid, queues, redo, st);
+             ? launch_partials<F16>(q, k, v, part_o, part_lse, out, lse, t, D, softmax_scale, grid, queues, redo, st)
+             : launch_partials<Bf16>(q, k, v, part_o, part_lse, out, lse, t, D, softmax_scale, grid, queues, redo, st);
 }
 
+// mrg_start [nranges], mrg_prefix [nranges + 1], merge_tokens = mrg_prefix[nranges]: the tokens to merge, for a
+// caller whose attention call wrote the other tokens' rows itself (chunk_direct); null, null, 0, S: every token.
 extern "C" int moba_fwd_merge(const void* part_o, const float* part_lse, const int32_t* sel, void* out, float* lse,
-                              int64_t S, int H, int D, int K, int key_split, int dtype, void* stream) {
+                              int64_t S, int H, int D, int K, int key_split, const int32_t* mrg_start,
+                              const int32_t* mrg_prefix, int nranges, int64_t merge_tokens, int dtype, void* stream) {
   LaunchCheck launch_check;
   if (!part_o || !part_lse || !out || !lse || (K > 0 && !sel)) return MOBA_ERR_ARG;
   if (key_split < 1 || key_split > kMaxKeySplit) return MOBA_ERR_ARG;
   if (K == 0) key_split = 1;
   if (D != kHeadDim || (dtype != MOBA_DTYPE_BF16 && dtype != MOBA_DTYPE_F16)) return MOBA_ERR_UNSUPPORTED;
   if (S <= 0 || H <= 0 || K < 0 || ((uintptr_t)part_o & 15) || ((uintptr_t)out & 15)) return MOBA_ERR_ARG;
-  const int64_t rows = S * H;
+  if (mrg_start ? (!mrg_prefix || nranges <= 0 || merge_tokens < 0 || merge_tokens > S)
+                : (mrg_prefix || merge_tokens != S))
+    return MOBA_ERR_ARG;
+  if (merge_tokens == 0) return MOBA_OK;  // every row was written by the attention kernel
+  const int64_t rows = merge_tokens * H;
   const dim3 grid((unsigned)((rows + 15) / 16));
   if (dtype == MOBA_DTYPE_F16)
     hipLaunchKernelGGL(moba_merge_kernel<F16>, grid, dim3(256), 0, (hipStream_t)stream, (const f16*)part_o, part_lse,
-                       sel, (f16*)out, lse, rows, K + 1, key_split);
+                       sel, (f16*)out, lse, rows, K + 1, key_split, S * H, mrg_start, mrg_prefix, nranges, H);
   else
     hipLaunchKernelGGL(moba_merge_kernel<Bf16>, grid, dim3(256), 0, (hipStream_t)stream, (const bf16*)part_o,
-                       part_lse, sel, (bf16*)out, lse, rows, K + 1, key_split);
+                       part_lse, sel, (bf16*)out, lse, rows, K + 1, key_split, S * H, mrg_start, mrg_prefix, nranges, H);
   return launch_check.result();
 }
 
@@ -923,12 +953,17 @@ extern "C" int moba_fwd(const void* q, const void* k, const void* v, void* part_
                         const int32_t* sel, const int32_t* seg_off, const int32_t* tile_off,
                         const int32_t* seg_dest, const int32_t* fchunk_tok, const int32_t* chunk_tok,
                         const int32_t* self_tile_prefix, const int32_t* tile_seg, const int32_t* self_tile_chunk,
-                        void* out, float* lse, int64_t S, int H, int Hkv, int D, int K, int F, int N, int B,
-                        int64_t hist_bound, int64_t self_tiles, int key_split, const int64_t* strides,
+                        const int32_t* chunk_direct, const int32_t* mrg_start, const int32_t* mrg_prefix, int nranges,
+                        int64_t merge_tokens, void* out, float* lse, int64_t S, int H, int Hkv, int D, int K, int F,
+                        int N, int B, int64_t hist_bound, int64_t self_tiles, int key_split, const int64_t* strides,
                         int32_t* queues, int32_t* redo, float softmax_scale, int dtype, void* stream) {
+  if (!out || !lse) return MOBA_ERR_ARG;
+  // (direct rows and the merge's token ranges come together: either both or neither)
+  if ((chunk_direct != nullptr) != (mrg_start != nullptr)) return MOBA_ERR_ARG;
   int rc = moba_fwd_partials(q, k, v, part_o, part_lse, seg_off, tile_off, seg_dest, fchunk_tok, chunk_tok,
-                             self_tile_prefix, tile_seg, self_tile_chunk, S, H, Hkv, D, K, F, N, B, hist_bound,
-                             self_tiles, key_split, strides, queues, redo, softmax_scale, dtype, stream);
+                             self_tile_prefix, tile_seg, self_tile_chunk, chunk_direct, out, lse, S, H, Hkv, D, K, F, N,
+                             B, hist_bound, self_tiles, key_split, strides, queues, redo, softmax_scale, dtype, stream);
   if (rc != MOBA_OK) return rc;
-  return moba_fwd_merge(part_o, part_lse, sel, out, lse, S, H, D, K, key_split, dtype, stream);
+  return moba_fwd_merge(part_o, part_lse, sel, out, lse, S, H, D, K, key_split, mrg_start, mrg_prefix, nranges,
+                        merge_tokens, dtype, stream);
 }

@@ -24,11 +24,12 @@ struct moba_plan_t {
   int64_t pairs_per_head;   // list entries per head: M = pairs_per_head * H
   int64_t fwd_self_tiles, bwd_self_tiles;  // row tiles of the attention chunks, per head
   int64_t kv_tiles;         // key tiles (bwd_tile_rows keys) of the chunks, per key/value head
+  int64_t merge_tokens;     // tokens behind the first attention chunk of their sequence: the rows the merge walks
   double flops_per_head_per_dim;           // forward flops = this * H * head_dim
   // offsets (in int32 elements) of the tables inside the array moba_plan_fill writes, -1 = absent
   int64_t off_cu_seqlens, off_chunk_tok, off_achunk_tok, off_fwd_self_tile_prefix, off_fwd_self_tile_chunk,
       off_self_tile_prefix, off_self_tile_chunk, off_kv_tile_prefix, off_kv_tile_chunk, off_chunk_self_end,
-      off_seq_fbase, off_fchunk_tok, off_chunk_fb, off_chunk_local, off_pair_off, off_chunk_fid;
+      off_achunk_direct, off_mrg_start, off_mrg_prefix, off_seq_fbase, off_fchunk_tok, off_chunk_fb, off_chunk_local, off_pair_off, off_chunk_fid;
   int64_t table_ints;       // length of that array
 };
 
@@ -70,6 +71,7 @@ static int plan_core(const int32_t* cu, int nseq, int chunk, int topk, int dense
     int64_t alen = 0;  // length of the attention chunk being put together
     for (int64_t c = 0; c < n; ++c) {
       const int64_t clen = p.fallback ? len : std::min<int64_t>(chunk, len - c * chunk);
+      if (c == d + 1) p.merge_tokens += len - alen;  // (the tokens behind the sequence's first attention chunk)
       if (c > d) { add_achunk(alen); alen = 0; }
       alen += clen;
       ktiles += (clen + TM - 1) / TM;
@@ -96,6 +98,9 @@ static int plan_core(const int32_t* cu, int nseq, int chunk, int topk, int dense
   p.off_kv_tile_prefix = take(p.N + 1);
   p.off_kv_tile_chunk = take(ktiles);
   p.off_chunk_self_end = take(p.N);
+  p.off_achunk_direct = take(NA);
+  p.off_mrg_start = take(nseq);
+  p.off_mrg_prefix = take(nseq + 1);
   if (p.fallback) {
     p.off_seq_fbase = p.off_fchunk_tok = p.off_chunk_fb = p.off_chunk_local = p.off_pair_off = p.off_chunk_fid = -1;
   } else {
@@ -124,8 +129,15 @@ static int plan_core(const int32_t* cu, int nseq, int chunk, int topk, int dense
   int32_t* self_end = tab + p.off_chunk_self_end;
   int32_t c_all = 0, f_all = 0, pair_all = 0, a_all = 0;
   int64_t ft = 0, bt = 0, kt = 0;
-  auto close_achunk = [&](int32_t tok0, int64_t alen, int32_t first_chunk, int32_t end_chunk) {
+  int64_t merged = 0;
+  auto close_achunk = [&](int32_t tok0, int64_t alen, int32_t first_chunk, int32_t end_chunk, int b, bool first) {
     achunk_tok[a_all] = tok0;
+    tab[p.off_achunk_direct + a_all] = first ? 1 : 0;
+    if (first) {
+      tab[p.off_mrg_start + b] = (int32_t)(tok0 + alen);
+      tab[p.off_mrg_prefix + b] = (int32_t)merged;
+      merged += cu[b + 1] - (tok0 + alen);
+    }
     fpre[a_all] = (int32_t)ft; bpre[a_all] = (int32_t)bt;
     for (int64_t i = 0; i < (alen + kFwdTileRows - 1) / kFwdTileRows; ++i) fch[ft++] = a_all;
     for (int64_t i = 0; i < (alen + TM - 1) / TM; ++i) bch[bt++] = a_all;
@@ -143,7 +155,7 @@ static int plan_core(const int32_t* cu, int nseq, int chunk, int topk, int dense
       const int64_t clen = p.fallback ? len : std::min<int64_t>(chunk, len - c * chunk);
       chunk_tok[c_all] = (int32_t)(cu[b] + c * chunk);
       if (c > d) {
-        close_achunk(a_tok0, alen, a_first, c_all);
+        close_achunk(a_tok0, alen, a_first, c_all, b, c == d + 1);
         a_tok0 = chunk_tok[c_all]; a_first = c_all; alen = 0;
       }
       alen += clen;
@@ -162,8 +174,9 @@ static int plan_core(const int32_t* cu, int nseq, int chunk, int topk, int dense
         tab[p.off_chunk_fid + c_all] = -1;
       }
     }
-    close_achunk(a_tok0, alen, a_first, c_all);
+    close_achunk(a_tok0, alen, a_first, c_all, b, n <= (int64_t)d + 1);
   }
+  tab[p.off_mrg_prefix + nseq] = (int32_t)merged;
   chunk_tok[c_all] = cu[nseq];
   achunk_tok[a_all] = cu[nseq];
   fpre[a_all] = (int32_t)ft; bpre[a_all] = (int32_t)bt;

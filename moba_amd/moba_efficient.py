@@ -393,12 +393,15 @@ def _forward(q, k, v, plan: MobaPlan, timer: Optional[StageTimer] = None, scale:
     with span("fwd_partials"):
         _lib.check(lib.moba_fwd_partials(qp, kp, vp, part_op, part_lsep, seg_offp, tile_offp, seg_destp,
                                          tp.get("fchunk_tok", null), tp["achunk_tok"], tp["fwd_self_tile_prefix"],
-                                         tile_segp, tp["fwd_self_tile_chunk"], S, H, Hkv, D, K, plan.F, plan.NA,
+                                         tile_segp, tp["fwd_self_tile_chunk"], tp["achunk_direct"], _ptr(out),
+                                         _ptr(lse), S, H, Hkv, D, K, plan.F, plan.NA,
                                          plan.chunk_size, g.bound, plan.fwd_self_tiles, g.split, strides, queuesp,
                                          redop, scale, code, stream), "moba_fwd_partials")
-    with span("fwd_merge"):
-        _lib.check(lib.moba_fwd_merge(part_op, part_lsep, selp, _ptr(out), _ptr(lse), S, H, D, K, g.split, code,
-                                      stream), "moba_fwd_merge")
+    if plan.merge_tokens:   # (the rows of every sequence's first attention chunk are written by the kernel above)
+        with span("fwd_merge"):
+            _lib.check(lib.moba_fwd_merge(part_op, part_lsep, selp, _ptr(out), _ptr(lse), S, H, D, K, g.split,
+                                          tp["mrg_start"], tp["mrg_prefix"], plan.nseq, plan.merge_tokens, code,
+                                          stream), "moba_fwd_merge")
     return out, lse, sel, seg_off, tile_off, seg_dest, tile_seg
 
 

@@ -46,6 +46,9 @@ class MobaPlan:
     dense_local: int = 0
     NA: int = 0         # attention chunks (tables achunk_tok, self_tile_*, fwd_self_tile_*)
     kv_tiles: int = 0   # key tiles of TILE_ROWS keys of the chunks, per key/value head (tables kv_tile_*)
+    # The rows of a sequence's first attention chunk have no history slots: the forward kernel writes them straight
+    # to the output (table achunk_direct) and the merge walks the other tokens only (tables mrg_start, mrg_prefix).
+    merge_tokens: int = 0
     tables: Dict[str, torch.Tensor] = field(default_factory=dict)
     host: Dict[str, np.ndarray] = field(default_factory=dict)
     memo: Dict[tuple, object] = field(default_factory=dict)  # what callers derive once per plan (sizes, pointers)
@@ -104,10 +107,14 @@ def _host_tables(cu: np.ndarray, B: int, topk: int, dense: bool = False):
                self_tile_chunk=np.repeat(np.arange(NA), tiles),
                kv_tile_prefix=np.concatenate([[0], np.cumsum(ktiles)]),
                kv_tile_chunk=np.repeat(np.arange(N), ktiles),
-               chunk_self_end=achunk_tok[achunk_of + 1])     # where the causal rows of a chunk's keys end
+               chunk_self_end=achunk_tok[achunk_of + 1],     # where the causal rows of a chunk's keys end
+               achunk_direct=(local[starts_a] == 0).astype(np.int64))
+    # the tokens behind the first attention chunk of every sequence: ranges of the merge
+    first_end = achunk_tok[1:][local[starts_a] == 0]         # end of the first attention chunk of every sequence
+    out.update(mrg_start=first_end, mrg_prefix=np.concatenate([[0], np.cumsum(cu[1:] - first_end)]))
     info = dict(nseq=nseq, N=N, F=0 if fallback else F, k_eff=k_eff, fallback=fallback, K=0, P=0, cmax=0,
                 pairs_per_head=0, self_tiles=int(tiles.sum()), fwd_self_tiles=int(ftiles.sum()), NA=NA, dense_local=d,
-                kv_tiles=int(ktiles.sum()))
+                kv_tiles=int(ktiles.sum()), merge_tokens=int((cu[1:] - first_end).sum()))
     pairs_self = int((chunk_len.astype(np.int64) * (chunk_len + 1) // 2).sum())
     if not fallback:
         seq_fbase = np.concatenate([[0], np.cumsum(n_chunks - 1)])
@@ -168,7 +175,8 @@ def _build(cu: np.ndarray, chunk_size: int, moba_topk: int, device, dense: bool 
                     fallback=info["fallback"], P=info["P"], cmax=info["cmax"], pairs_per_head=info["pairs_per_head"],
                     self_tiles=info["self_tiles"], fwd_self_tiles=info["fwd_self_tiles"],
                     flops_per_head=info["flops_per_head_per_d"], dense_local=info["dense_local"], NA=info["NA"],
-                    kv_tiles=info["kv_tiles"], host=host, device=device if on_device else None)
+                    kv_tiles=info["kv_tiles"], merge_tokens=info["merge_tokens"], host=host,
+                    device=device if on_device else None)
     if on_device:
         names = list(host)
         flat = np.concatenate([host[n_].astype(np.int32) for n_ in names])

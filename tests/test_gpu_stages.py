@@ -230,7 +230,8 @@ def test_merge_of_random_partials(K, dtype, parts):
     p = lambda t: ctypes.c_void_p(t.data_ptr())
     code = _lib.DTYPE_F16 if dtype == torch.float16 else _lib.DTYPE_BF16
     _lib.check(lib.moba_fwd_merge(p(part_o_dev), p(part_lse_dev), p(sel.cuda()), p(out), p(lse), S, H, 128, K, parts,
-                                  code, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)), "moba_fwd_merge")
+                                  None, None, 0, S, code, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)),
+               "moba_fwd_merge")
     lses = lse_nat.clone()
     lses[absent] = float("-inf")
     # (the parts of a slot are slots like any other to the merge algebra)
@@ -269,9 +270,10 @@ def test_moba_fwd_entry_point(batch, seqlen, heads, B, topk, dtype, dense):
     p = E._ptr
     _lib.check(lib.moba_fwd(p(qg), p(kg), p(vg), p(part_o), p(part_lse), p(sel), p(seg_off), p(tile_off), p(seg_dest),
                             p(t.get("fchunk_tok")), p(t["achunk_tok"]), p(t["fwd_self_tile_prefix"]), p(tile_seg),
-                            p(t["fwd_self_tile_chunk"]), p(out), p(lse), S, H, H, D, K, plan.F, plan.NA, plan.chunk_size,
-                            bound, plan.fwd_self_tiles, split, None, p(queues), None, 0.0, E._dtype_code(qg),
-                            E._stream(dev)), "moba_fwd")
+                            p(t["fwd_self_tile_chunk"]), p(t["achunk_direct"]), p(t["mrg_start"]), p(t["mrg_prefix"]),
+                            plan.nseq, plan.merge_tokens, p(out), p(lse), S, H, H, D, K, plan.F, plan.NA,
+                            plan.chunk_size, bound, plan.fwd_self_tiles, split, None, p(queues), None, 0.0,
+                            E._dtype_code(qg), E._stream(dev)), "moba_fwd")
     torch.cuda.synchronize()
     assert torch.equal(out, want_out) and torch.equal(lse, want_lse)
     if dense and sel is not None:
@@ -284,8 +286,10 @@ def test_moba_fwd_entry_point(batch, seqlen, heads, B, topk, dtype, dense):
 
 
 # ------------------------------------------------------------------ fixed-reference softmax and its redo list
-def _attention_stage(q, k, v, plan, aux, with_redo, key_split=1):
-    """moba_fwd on prepared selection/lists; returns (out, lse, number of tiles sent to the redo list or None)."""
+def _attention_stage(q, k, v, plan, aux, with_redo, key_split=1, direct=True):
+    """moba_fwd on prepared selection/lists; returns (out, lse, number of tiles sent to the redo list or None).
+    direct: the rows without history slots go straight to the outputs (as the operator runs it), or every row
+    through its slot and the merge."""
     from moba_amd import _lib
     from moba_amd import moba_efficient as E
     lib = _lib.load()
@@ -303,9 +307,11 @@ def _attention_stage(q, k, v, plan, aux, with_redo, key_split=1):
     p = E._ptr
     _lib.check(lib.moba_fwd(p(q), p(k), p(v), p(part_o), p(part_lse), p(sel), p(seg_off), p(tile_off), p(seg_dest),
                             p(t.get("fchunk_tok")), p(t["achunk_tok"]), p(t["fwd_self_tile_prefix"]), p(tile_seg),
-                            p(t["fwd_self_tile_chunk"]), p(out), p(lse), S, H, H, D, K, plan.F, plan.NA, plan.chunk_size,
-                            plan.hist_tile_bound(H, 256), plan.fwd_self_tiles, key_split, None, p(queues), p(redo), 0.0,
-                            E._dtype_code(q), E._stream(dev)), "moba_fwd")
+                            p(t["fwd_self_tile_chunk"]), p(t["achunk_direct"]) if direct else None,
+                            p(t["mrg_start"]) if direct else None, p(t["mrg_prefix"]) if direct else None,
+                            plan.nseq if direct else 0, plan.merge_tokens if direct else S, p(out), p(lse), S, H, H, D, K,
+                            plan.F, plan.NA, plan.chunk_size, plan.hist_tile_bound(H, 256), plan.fwd_self_tiles, key_split,
+                            None, p(queues), p(redo), 0.0, E._dtype_code(q), E._stream(dev)), "moba_fwd")
     torch.cuda.synchronize()
     if redo is None:
         return out, lse, None
@@ -337,6 +343,9 @@ def test_history_keys_cut_into_parts(seqlens, heads, B, topk, dtype):
     sel = E.gate_topk(qg, E.chunk_mean(kg, plan), plan)
     aux = (sel,) + tuple(E.build_lists(sel, plan))
     out1, lse1, _ = _attention_stage(qg, kg, vg, plan, aux, False, 1)
+    # the rows without history slots written straight to the outputs, or through slot 0 and the merge: same bits
+    out0, lse0, _ = _attention_stage(qg, kg, vg, plan, aux, False, 1, direct=False)
+    assert torch.equal(out0, out1) and (lse0 - lse1).abs().max() < 1e-6
     ref, ref_lse, _ = O.moba_attn_varlen_oracle(q, k, v, cu, max(seqlens), B, topk, sel=sel.cpu(), return_aux=True)
     proposed = lib.moba_fwd_key_split(S, heads, plan.K, B, plan.hist_tile_bound(heads, 256), plan.fwd_self_tiles)
     _note("  proposed", proposed)

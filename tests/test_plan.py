@@ -95,6 +95,14 @@ def test_dense_prefix_tables(seed):
     assert dense.host["achunk_tok"].tolist() == achunk and dense.NA == len(achunk) - 1
     assert dense.pairs_per_head == entries
     assert dense.host["chunk_self_end"].tolist() == self_end
+    # the first attention chunk of every sequence has no history slots; the merge walks the tokens behind it
+    for pl, d in ((plan, 0), (dense, plan.K)):
+        first_end = [min(b_, a_ + (d + 1) * B) for a_, b_ in zip(cu[:-1], cu[1:])]
+        assert pl.host["mrg_start"].tolist() == first_end
+        assert np.array_equal(np.diff(pl.host["mrg_prefix"]), np.asarray(cu[1:]) - np.asarray(first_end))
+        assert pl.merge_tokens == int(pl.host["mrg_prefix"][-1]) and pl.host["mrg_prefix"][0] == 0
+        starts = set(cu[:-1])
+        assert pl.host["achunk_direct"].tolist() == [int(t in starts) for t in pl.host["achunk_tok"][:-1].tolist()]
     alen = np.diff(dense.host["achunk_tok"])
     for rows, pre, chunk, count in ((TILE_ROWS, "self_tile_prefix", "self_tile_chunk", dense.self_tiles),
                                     (FWD_TILE_ROWS, "fwd_self_tile_prefix", "fwd_self_tile_chunk", dense.fwd_self_tiles)):
