@@ -17,7 +17,7 @@
  * compute units' worth of workgroups; results do not depend on it.
  * Inputs are expected to be finite: the attention kernels are compiled without NaN handling, and with an
  * infinity or a NaN in q, k, v or dout the outputs are unspecified (no fault, no hang).  Scores of any finite
- * size are handled (the softmax subtracts a row reference before it exponentiates).
+ * size are handled (the softmax subtracts a row reference before it exponentiates; see `redo`).
  * Index limits, checked (code -4): S * H * (K + 1) < 2^31 (slot rows are 32-bit: 1M tokens x 64 heads x top-k 12
  * is beyond it, 1M x 32 x 12 is not), K <= 64, chunks per sequence <= 3413, tile counts < 2^31.  head_dim 128 (D below; narrower heads are padded with zeros by the
  * caller, see softmax_scale); q, k, v and everything derived from them are
@@ -228,12 +228,14 @@ int moba_tile_tables(const int32_t* seg_off, int32_t* tile_off, int32_t* tile_se
  *   queues [8] int32 scratch: the tile counters of the forward kernel, whose workgroups (one per CU) stay
  *              resident and draw tiles from one queue per XCD; the call zeroes them with a kernel of its own.
  *              Calls that overlap in time need their own eight counters each.
- *   redo   [1 + hist_bound + self_tiles * H] int32 scratch, or NULL.  With it, bf16 problems large enough for the
+ *   redo   [1 + hist_bound + self_tiles * H] int32 scratch, or NULL.  With it, problems large enough for the
  *              resident-workgroup kernel take each tile's softmax relative to one fixed reference per row (the row
- *              maximum of the tile's first 32 keys) instead of a running maximum; a tile in which a row's scores rise
- *              more than 96 powers of two above that reference is entered in this list and computed again by the
- *              kernel that tracks the maximum (redo[0] = number of such tiles after the call, normally 0).  The result
- *              is within rounding of the other path's either way.  NULL, fp16 and small problems: running maximum only.
+ *              maximum of the tile's first 32 keys) instead of a running maximum; a tile in which a row leaves the
+ *              range that is safe -- scores that rise more than 96 powers of two above that reference (bf16) or 16
+ *              (fp16: a probability beyond the type's range), or accumulators that leave fp32 (products with |v| of
+ *              2^31 and more) -- is entered in this list and computed again by the kernel that tracks the maximum
+ *              (redo[0] = number of such tiles after the call, normally 0).  The result is within rounding of the
+ *              other path's either way.  NULL and small problems: running maximum only.
  *   softmax_scale: the factor on q k^T; 0 (or less) stands for D^-0.5, the reference's only choice
  *              (moba/moba_efficient.py:86).  A caller whose heads are narrower than D pads them with zeros
  *              and passes its own head_dim^-0.5. */

@@ -50,8 +50,9 @@ struct FwdParams {
 
 constexpr float kRescaleThreshold = 8.f;  // log2 units: the running max may lag the true max by this much
 // Fixed-reference softmax: a row's sum of exponentials (relative to the row maximum of the tile's first key
-// block) at or beyond this, or not a number, sends the tile to the kernel that tracks the maximum.  Below it
-// every probability is a finite bf16 and the accumulators stay finite for |v| < 2^31.
+// block) at or beyond this, or not a number, sends the tile to the kernel that tracks the maximum; so does an
+// accumulator of the row that is not finite (a probability beyond the element type's range -- 2^16 for fp16 --
+// or products with large |v| that left fp32).
 constexpr float kFixedRefMaxSum = 0x1p96f;
 
 // how a workgroup comes by its tiles
@@ -74,18 +75,21 @@ enum : int {
 // kMode: resident workgroups that draw tiles from the queues (large problems), or one tile per workgroup,
 // the id from the workgroup id: with few tiles the queue protocol's start-up and wind-down (three passes
 // to fill the look-ahead, eight empty draws to know that nothing is left) would dominate.
-// kFixedRef (bf16, queued): the softmax of a tile is taken relative to one fixed reference per row, the row
+// kFixedRef (queued): the softmax of a tile is taken relative to one fixed reference per row, the row
 // maximum of the tile's first 32-key block, instead of a running maximum.  A bf16 probability has the
-// exponent range of fp32, so later scores may exceed the reference by almost 2^7 before anything overflows:
+// exponent range of fp32, so later scores may exceed the reference by almost 2^7 before anything overflows
+// (an fp16 probability: by 2^4 = 16 powers of two, still far more than scores of one row differ in practice):
 // the per-block row maximum, its exchange between the lane halves, the comparison with the running maximum
-// and the rescale branch all go (22 of 88 vector instructions per key block).  A row whose sum leaves the
-// safe range -- scores that rise by more than 96 powers of two within one tile -- marks its tile in
-// FwdParams::redo, and the kTilesListed kernel, which tracks the maximum, computes those tiles again.
+// and the rescale branch all go (22 of 88 vector instructions per key block).  A row that leaves the safe
+// range -- its sum of exponentials beyond 2^96, or an accumulator that is not finite because a probability
+// overflowed the element type -- marks its tile in FwdParams::redo, and the kTilesListed kernel, which tracks
+// the maximum, computes those tiles again.  (A probability below the element type's smallest number is lost
+// either way; relative to the first block's maximum fewer are than relative to the true one.)
 template <class E, int kMode, bool kFixedRef>
 __global__ __launch_bounds__(512, 2) void moba_fwd_kernel(const FwdParams<E> p) {
   MOBA_ELEM_TYPES(E)
   constexpr bool kQueued = kMode == kTilesQueued;
-  static_assert(!kFixedRef || (kQueued && std::is_same<E, Bf16>::value), "the fixed reference needs bf16's exponent range");
+  static_assert(!kFixedRef || kQueued, "the fixed reference comes with the queued tiles' redo list");
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int n = lane & 31, hh = lane >> 5;
@@ -260,8 +264,15 @@ __global__ __launch_bounds__(512, 2) void moba_fwd_kernel(const FwdParams<E> p) 
     const float l_tot = sum_xhalf(l_run);
     const float inv = 1.f / l_tot;
     if constexpr (kFixedRef) {
-      // compared as bit patterns: infinities, every NaN and negative values all read as "too large"
-      const bool bad = valid_done && __builtin_bit_cast(uint32_t, l_tot) >= __builtin_bit_cast(uint32_t, kFixedRefMaxSum);
+      // compared as bit patterns (the file is compiled without NaN semantics): infinities, every NaN and
+      // negative sums all read as "too large"; the largest magnitude among the row's accumulators likewise
+      uint32_t worst = 0;
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) worst = max(worst, __builtin_bit_cast(uint32_t, oacc[db][e]) & 0x7fffffffu);
+      const bool bad = valid_done && (__builtin_bit_cast(uint32_t, l_tot) >= __builtin_bit_cast(uint32_t, kFixedRefMaxSum) ||
+                                      worst >= 0x7f800000u);
       if (__any(bad) && ln == 0) *reinterpret_cast<volatile int*>(smem + kFwdRedoWord) = 1;
     }
     char* stage = smem + (wave_u < 4 ? 2 * kTileBytes + wave_u * 4096 : kFwdVBase + 2 * kTileBytes + (wave_u - 4) * 4096);
@@ -848,7 +859,7 @@ static int launch_partials(const void* q, const void* k, const void* v, void* pa
   static bool allowed[4][kMaxDevices];  // one set of arrays per element type
   if (grid > 0) {  // resident workgroups drawing from the queues
     hipLaunchKernelGGL(zero_queues_kernel, dim3(1), dim3(8), 0, st, queues, redo);  // a kernel, not a memset: graph safe
-    if constexpr (std::is_same<E, Bf16>::value) {
+    {
       if (redo) {
         // fixed-reference softmax, then the tiles it could not serve (normally none) with the tracked maximum
         if (!allow_dynamic_lds((const void*)moba_fwd_kernel<E, kTilesQueued, true>, kFwdLds, allowed[2]) ||

@@ -29,6 +29,8 @@ FIXED_REFERENCE = os.environ.get("MOBA_FIXED_REFERENCE", "1") != "0"
 # Dense prefixes (see MobaPlan.dense_local): None = where they pay (problems large enough for the kernels whose
 # workgroups stay resident), True / False (MOBA_DENSE_PREFIX=1 / 0) = always / never.
 DENSE_PREFIX = {"0": False, "1": True}.get(os.environ.get("MOBA_DENSE_PREFIX", ""))
+# MOBA_DIRECT_ROWS=0 (a diagnostic): every row goes through its slot and the merge, also the rows without history slots
+DIRECT_ROWS = os.environ.get("MOBA_DIRECT_ROWS", "1") != "0"
 # diagnostics: with KEEP_SCRATCH set, a forward call leaves views of its scratch in last_scratch ("redo": the
 # list of tiles the fixed-reference softmax handed to the kernel that tracks the maximum, count first; or None)
 KEEP_SCRATCH = False
@@ -393,11 +395,15 @@ def _forward(q, k, v, plan: MobaPlan, timer: Optional[StageTimer] = None, scale:
     with span("fwd_partials"):
         _lib.check(lib.moba_fwd_partials(qp, kp, vp, part_op, part_lsep, seg_offp, tile_offp, seg_destp,
                                          tp.get("fchunk_tok", null), tp["achunk_tok"], tp["fwd_self_tile_prefix"],
-                                         tile_segp, tp["fwd_self_tile_chunk"], tp["achunk_direct"], _ptr(out),
-                                         _ptr(lse), S, H, Hkv, D, K, plan.F, plan.NA,
+                                         tile_segp, tp["fwd_self_tile_chunk"], tp["achunk_direct"] if DIRECT_ROWS else null,
+                                         _ptr(out), _ptr(lse), S, H, Hkv, D, K, plan.F, plan.NA,
                                          plan.chunk_size, g.bound, plan.fwd_self_tiles, g.split, strides, queuesp,
                                          redop, scale, code, stream), "moba_fwd_partials")
-    if plan.merge_tokens:   # (the rows of every sequence's first attention chunk are written by the kernel above)
+    if not DIRECT_ROWS:
+        with span("fwd_merge"):
+            _lib.check(lib.moba_fwd_merge(part_op, part_lsep, selp, _ptr(out), _ptr(lse), S, H, D, K, g.split,
+                                          null, null, 0, S, code, stream), "moba_fwd_merge")
+    elif plan.merge_tokens:   # (the rows of every sequence's first attention chunk are written by the kernel above)
         with span("fwd_merge"):
             _lib.check(lib.moba_fwd_merge(part_op, part_lsep, selp, _ptr(out), _ptr(lse), S, H, D, K, g.split,
                                           tp["mrg_start"], tp["mrg_prefix"], plan.nseq, plan.merge_tokens, code,

@@ -406,3 +406,15 @@ def test_fixed_reference_softmax_and_redo_list(spread, dense):
     if spread == 1.0:  # the resident-workgroup kernel takes whole tiles only: key parts are refused, not ignored
         with pytest.raises(RuntimeError):
             _attention_stage(q, k, v, plan, aux, False, 2)
+    else:
+        # Values of large magnitude: probabilities of up to 2^96 times |v| of 2^40 leave fp32 in the accumulators of
+        # the fixed-reference kernel, where the kernel that tracks the maximum (probabilities up to 2^8) stays
+        # finite.  Such tiles must be found and computed again: the result is finite and the other path's.
+        big = (v.float() * 2.0 ** 40).to(torch.bfloat16)
+        out_b, lse_b, n_big = _attention_stage(q, k, big, plan, aux, True)
+        out_r, lse_r, _ = _attention_stage(q, k, big, plan, aux, False)
+        _note("  tiles computed again with |v| ~ 2^40:", n_big)
+        assert n_big >= n_redo and torch.isfinite(out_b.float()).all() and torch.isfinite(out_r.float()).all()
+        err = (out_b.float() - out_r.float()).abs() * 2.0 ** -40
+        assert err.max() < 2e-2 and err.mean() < 1e-4, (err.max().item(), err.mean().item())
+        assert torch.equal(lse_b, lse_f)
