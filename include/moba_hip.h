@@ -8,7 +8,9 @@
  * The library allocates nothing, frees nothing, and never synchronises the device:
  * every launch is enqueued on `stream`.  Return value: 0, or a negative code that
  * moba_strerror() explains.  A HIP error already pending on the calling thread is neither reported
- * nor cleared; an error raised by an entry point's own launches is reported (-3) and cleared.
+ * nor cleared; an error raised by an entry point's own launches is reported (-3) and cleared.  (With an error
+ * pending, a launch failure of the entry point's own that carries the same code cannot be told from it and is
+ * not reported: a caller that relies on the return value clears pending errors, hipGetLastError(), first.)
  * State the library keeps, all of it per device and filled on first use: the number of compute units,
  * which kernels have been allowed their dynamic LDS size, and the address of the array of
  * moba_chunk_mean_static.  First calls may come from several threads at once (the writes are idempotent,

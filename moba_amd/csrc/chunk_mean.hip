@@ -198,6 +198,7 @@ static int check_chunk_mean_args(const void* k, const int32_t* fchunk_tok, void*
   // strides (elements): {., ., k token, k head, rows per batch entry, ., k batch}; null = packed [S, H, D]
   kts = strides ? strides[2] : (int64_t)H * D;
   khs = strides ? strides[3] : D;
+  if (strides && (strides[4] < 0 || strides[4] > 0x7fffffffLL)) return MOBA_ERR_ARG;  // (before it is narrowed)
   kbr = strides ? (int)strides[4] : 0;
   kbs = strides ? strides[6] : 0;
   if (kts <= 0 || khs <= 0 || (kts & 7) || (khs & 7)) return MOBA_ERR_ARG;

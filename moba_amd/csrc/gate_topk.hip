@@ -241,6 +241,7 @@ extern "C" int moba_gate_topk(const void* q, const void* kbar, const int32_t* cu
   if (((uintptr_t)q & 15) || ((uintptr_t)kbar & 15)) return MOBA_ERR_ARG;
   // strides (elements): {q token, q head, ., ., rows per batch entry, q batch, .}; null = packed [S, H, 128]
   const int64_t qts = strides ? strides[0] : (int64_t)H * kHeadDim, qhs = strides ? strides[1] : kHeadDim;
+  if (strides && (strides[4] < 0 || strides[4] > 0x7fffffffLL)) return MOBA_ERR_ARG;  // (before it is narrowed)
   const int qbr = strides ? (int)strides[4] : 0;
   const int64_t qbs = strides ? strides[5] : 0;
   if (qts <= 0 || qhs <= 0 || (qts & 7) || (qhs & 7)) return MOBA_ERR_ARG;

@@ -27,7 +27,11 @@ def _cu_seqlens_for(batch: int, seq_len: int, device) -> torch.Tensor:
     if t is None:
         if len(_CU_SEQLENS) >= 16:
             _CU_SEQLENS.pop(next(iter(_CU_SEQLENS)))
-        t = torch.arange(0, (batch + 1) * seq_len, seq_len, dtype=torch.int32, device=device)
+        # Made outside inference mode even when the model runs inside it: an inference tensor has no version
+        # counter, the planner would not remember it by identity, and every layer would then read it back from
+        # the device (a blocking copy) to plan by value.  Nobody writes to this tensor.
+        with torch.inference_mode(False):
+            t = torch.arange(0, (batch + 1) * seq_len, seq_len, dtype=torch.int32, device=device)
         _CU_SEQLENS[key] = t
     return t
 

@@ -111,8 +111,9 @@ def test_moba_layer_hands_grouped_heads_to_an_impl_that_takes_them():
 
 
 def test_moba_layer_prefill_under_inference_mode():
-    """Under torch.inference_mode() the adapter's cu_seqlens is an inference tensor; an operator that plans
-    from host lengths (as the HIP operator does) must get through make_plan with it."""
+    """Under torch.inference_mode() the adapter still hands the operator an ordinary cu_seqlens tensor (made
+    outside the mode), so that the planner remembers it by identity and no layer reads it back from the device;
+    an inference tensor from another caller is planned by value (tests/test_plan.py)."""
     from moba_amd import MoBAConfig
     from moba_amd.plan import make_plan
     from moba_amd.wrapper import moba_layer
@@ -121,6 +122,7 @@ def test_moba_layer_prefill_under_inference_mode():
 
     def impl(q, k, v, cu_seqlens, max_seqlen, moba_chunk_size, moba_topk):
         seen["plan"] = make_plan(cu_seqlens, moba_chunk_size, moba_topk, device="cpu")
+        seen["again"] = make_plan(cu_seqlens, moba_chunk_size, moba_topk, device="cpu")
         seen["inference"] = cu_seqlens.is_inference()
         return q
 
@@ -133,7 +135,8 @@ def test_moba_layer_prefill_under_inference_mode():
     with torch.inference_mode():
         x = torch.randn(b, h, s, d)
         out, _ = moba_layer(impl, MoBAConfig(4, 3), Mod(), x, x, x, None)
-    assert seen["inference"] and seen["plan"].cu == [0, 7, 14] and out.shape == (b * s, h, d)
+    assert not seen["inference"] and seen["plan"].cu == [0, 7, 14] and out.shape == (b * s, h, d)
+    assert seen["again"] is seen["plan"]
 
 
 def test_full_attention_layers_switch():
