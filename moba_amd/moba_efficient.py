@@ -29,6 +29,11 @@ FIXED_REFERENCE = os.environ.get("MOBA_FIXED_REFERENCE", "1") != "0"
 # Dense prefixes (see MobaPlan.dense_local): None = where they pay (problems large enough for the kernels whose
 # workgroups stay resident), True / False (MOBA_DENSE_PREFIX=1 / 0) = always / never.
 DENSE_PREFIX = {"0": False, "1": True}.get(os.environ.get("MOBA_DENSE_PREFIX", ""))
+# The per-slot partial results of a call take S * H * (K + 1) rows of head_dim elements, and the kernels index those
+# rows with 32 bits.  A call whose partials would exceed this many bytes (MOBA_SCRATCH_GB, default 48), or 2^31
+# rows, goes through its query heads in groups (whole key/value head groups): heads are independent, the result
+# is the same bit for bit, and the scratch of one group is reused by the next.
+SCRATCH_LIMIT_BYTES = int(float(os.environ.get("MOBA_SCRATCH_GB", "48")) * 2 ** 30)
 # MOBA_DIRECT_ROWS=0 (a diagnostic): every row goes through its slot and the merge, also the rows without history slots
 DIRECT_ROWS = os.environ.get("MOBA_DIRECT_ROWS", "1") != "0"
 # diagnostics: with KEEP_SCRATCH set, a forward call leaves views of its scratch in last_scratch ("redo": the
@@ -512,10 +517,87 @@ def _choose_plan(plan: MobaPlan, H: int) -> MobaPlan:
     return choice
 
 
+def _head_groups(plan: MobaPlan, H: int, Hkv: int, D: int, esize: int):
+    """[(first query head, one past the last)]: the groups of heads a call works through, one group unless the
+    per-slot partials of all heads together are too many (SCRATCH_LIMIT_BYTES, 2^31 slot rows)."""
+    rep = H // Hkv
+    rows_per_head = plan.S * (plan.K + 1)
+    most = min((0x7fffffff - 1) // rows_per_head, SCRATCH_LIMIT_BYTES // (rows_per_head * (D * esize + 4)))
+    most = max(rep, most // rep * rep)           # whole key/value head groups, at least one
+    if most >= H:
+        return [(0, H)]
+    n = -(-H // most)                            # groups, as equal as whole key/value head groups allow
+    size = -(-(H // rep) // n) * rep
+    return [(h0, min(H, h0 + size)) for h0 in range(0, H, size)]
+
+
+def _forward_in_groups(q, k, v, plan, groups, timer, scale, keep):
+    """The forward group by group; `keep` receives what a backward needs of every group."""
+    S, H, D = _dims(q)
+    rep = H // _dims(k)[1]
+    out = torch.empty((S, H, D), dtype=q.dtype, device=q.device)
+    lse = torch.empty((S, H), dtype=torch.float32, device=q.device)
+    for h0, h1 in groups:
+        group_plan = _choose_plan(plan, h1 - h0)
+        tables = [] if keep is not None else None
+        res = _forward(q[:, h0:h1], k[:, h0 // rep:h1 // rep], v[:, h0 // rep:h1 // rep], group_plan, timer, scale,
+                       bwd_tables=tables)
+        out[:, h0:h1] = res[0]
+        lse[:, h0:h1] = res[1]
+        if keep is not None:
+            keep.append((group_plan, res[2], res[3], res[5], tables))
+        del res
+    return out, lse
+
+
+class _MobaAttentionInGroups(torch.autograd.Function):
+    """_MobaAttention for a call that works through its heads in groups (see SCRATCH_LIMIT_BYTES)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, plan, groups, timer=None, scale=0.0):
+        keep = []
+        out, lse = _forward_in_groups(q, k, v, plan, groups, timer, scale, keep)
+        ctx.groups, ctx.keep, ctx.scale = groups, keep, scale
+        ctx.save_for_backward(q, k, v, out, lse)
+        ctx.mark_non_differentiable(lse)
+        ctx.set_materialize_grads(False)
+        return out, lse
+
+    @staticmethod
+    def backward(ctx, dout, _dlse):
+        q, k, v, out, lse = ctx.saved_tensors
+        if dout is None:
+            return None, None, None, None, None, None, None
+        S, H, D = _dims(q)
+        Hkv = _dims(k)[1]
+        rep = H // Hkv
+        dout = dout.to(q.dtype)
+        dq = torch.empty((S, H, D), dtype=q.dtype, device=q.device)
+        dk = torch.empty((S, Hkv, D), dtype=k.dtype, device=q.device)
+        dv = torch.empty((S, Hkv, D), dtype=v.dtype, device=q.device)
+        for (h0, h1), (group_plan, sel, seg_off, seg_dest, tables) in zip(ctx.groups, ctx.keep):
+            g0, g1 = h0 // rep, h1 // rep
+            got = _backward(_aligned(dout[:, h0:h1]), q[:, h0:h1], k[:, g0:g1], v[:, g0:g1], out[:, h0:h1].contiguous(),
+                            lse[:, h0:h1].contiguous(), sel, seg_off, seg_dest, group_plan, ctx.scale, tables)
+            dq[:, h0:h1], dk[:, g0:g1], dv[:, g0:g1] = got
+            del got
+        if q.dim() == 4:
+            b, _, l, d = q.shape
+            dq, dk, dv = (g.view(b, l, -1, d).transpose(1, 2) for g in (dq, dk, dv))
+        return dq, dk, dv, None, None, None, None
+
+
 def _attend(q, k, v, plan, timer=None, scale=0.0):
     """(out, lse): through autograd when a gradient may be asked for, straight to the kernels otherwise."""
-    plan = _choose_plan(plan, _dims(q)[1])
-    if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad):
+    S, H, D = _dims(q)
+    groups = _head_groups(plan, H, _dims(k)[1], D, q.element_size())
+    grad = torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad)
+    if len(groups) > 1:
+        if grad:
+            return _MobaAttentionInGroups.apply(q, k, v, plan, groups, timer, scale)
+        return _forward_in_groups(q, k, v, plan, groups, timer, scale, None)
+    plan = _choose_plan(plan, H)
+    if grad:
         return _MobaAttention.apply(q, k, v, plan, timer, scale)
     return _forward(q, k, v, plan, timer, scale)[:2]
 

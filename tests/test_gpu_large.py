@@ -173,3 +173,42 @@ def test_chunk_mean_many_chunks():
     kbar = E.chunk_mean(k, plan)
     want = (k[:F * B].double().view(F, B, H, 128).sum(1) / B).float().to(torch.bfloat16)
     assert torch.equal(kbar, want)
+
+
+def test_a_million_tokens_of_64_heads():
+    """1M tokens x 64 query heads x top-k 12: 8.05e8 slot rows, 206 GB of per-slot partials in one piece.  The
+    operator works through the heads in groups that fit its scratch budget (the reference has no such limit,
+    moba/moba_efficient.py:270-297).  Forward, grouped-query heads (8 key/value heads), sampled rows against the
+    explicit softmax over the row's attended keys."""
+    from moba_amd import moba_efficient as E
+    from moba_amd.plan import make_plan
+    S, H, Hkv, B, topk = 1048576, 64, 8, 4096, 12
+    print("large case", S, H, B, topk, flush=True)
+    dev = torch.device("cuda")
+    g = torch.Generator(device=dev).manual_seed(5)
+    q = torch.randn((S, H, 128), generator=g, device=dev, dtype=torch.bfloat16)
+    k = torch.randn((S, Hkv, 128), generator=g, device=dev, dtype=torch.bfloat16)
+    v = torch.randn((S, Hkv, 128), generator=g, device=dev, dtype=torch.bfloat16)
+    cu_t = torch.tensor([0, S], dtype=torch.int32, device=dev)
+    plan = make_plan(cu_t, B, topk)
+    assert S * H * (plan.K + 1) * 256 > 200e9 > E.SCRATCH_LIMIT_BYTES
+    groups = E._head_groups(plan, H, Hkv, 128, 2)
+    assert len(groups) > 1 and all((b - a) % (H // Hkv) == 0 for a, b in groups)
+    with torch.no_grad():
+        out, lse = E.moba_attn_varlen_with_lse(q, k, v, cu_t, S, B, topk, gqa=True)
+    torch.cuda.synchronize()
+    rng = np.random.default_rng(3)
+    rep = H // Hkv
+    rows = sorted(set(rng.integers(0, S, size=6).tolist() + [0, S - 1, 12 * B, 12 * B - 1]))
+    for h in (0, 37, H - 1):
+        # the selection of this head's rows: the gate stage alone on a one-head view
+        qh = q[:, h:h + 1].contiguous()
+        kh = k[:, h // rep:h // rep + 1].contiguous()
+        vh = v[:, h // rep:h // rep + 1].contiguous()
+        sel_h = E.gate_topk(qh, E.chunk_mean(kh, plan), plan)
+        for s in rows:
+            ref, ref_lse = _row_oracle(qh, kh, vh, sel_h[s, 0].cpu(), s, 0, 0, B, 0)
+            err = (out[s, h].float().cpu() - ref).abs().max().item()
+            assert err < 2e-2 and err <= 3e-2 * ref.abs().max().item() + 1e-5, (s, h, err)
+            assert abs(lse[s, h].item() - ref_lse.item()) < 2e-3
+        del qh, kh, vh, sel_h

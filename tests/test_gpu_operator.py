@@ -631,3 +631,53 @@ def test_batched_layout_in_place(b, hq, hkv, s, B, topk, dtype):
     odd = buf[4:].view(query.shape)
     assert not E._addressable(odd)
     assert torch.equal(E.moba_attn_batched(odd, key.detach(), value.detach(), B, topk), want)
+
+
+@pytest.mark.parametrize("heads,kv_heads,batched", [(6, 6, False), (8, 2, False), (8, 4, True), (10, 5, False)])
+def test_heads_in_groups(heads, kv_heads, batched, monkeypatch):
+    """A call whose per-slot partials would not fit its scratch budget (or 2^31 slot rows) works through its heads in
+    groups of whole key/value head groups: same output, LSE and gradients bit for bit as in one piece -- the packed
+    operator, grouped-query heads, and the batched layout read in place."""
+    from moba_amd import moba_efficient as E
+    from moba_amd.plan import make_plan
+    from moba_amd.wrapper import hf_to_fa
+    b, s, B, topk = 3, 1400, 128, 3
+    g = torch.Generator().manual_seed(17)
+    query = torch.randn((b, heads, s, 128), generator=g).to(torch.bfloat16).cuda()
+    key = torch.randn((b, kv_heads, s, 128), generator=g).to(torch.bfloat16).cuda()
+    value = torch.randn((b, kv_heads, s, 128), generator=g).to(torch.bfloat16).cuda()
+    do = torch.randn((b * s, heads, 128), generator=g).to(torch.bfloat16).cuda()
+    cu = torch.arange(0, (b + 1) * s, s, dtype=torch.int32, device="cuda")
+
+    def run():
+        if batched:
+            q, k, v = (x.clone().requires_grad_(True) for x in (query, key, value))
+            out = E.moba_attn_batched(q, k, v, B, topk)
+        else:
+            q, k, v = (hf_to_fa(x).contiguous().requires_grad_(True) for x in (query, key, value))
+            out = E.moba_attn_varlen_gqa(q, k, v, cu, s, B, topk)
+        out.backward(do)
+        return out.detach(), q.grad, k.grad, v.grad
+
+    whole = run()
+    plan = make_plan(cu, B, topk)
+    rep = heads // kv_heads
+    per_head = plan.S * (plan.K + 1) * (128 * 2 + 4)
+    monkeypatch.setattr(E, "SCRATCH_LIMIT_BYTES", per_head * rep * 2 - 1)     # one key/value head group at a time
+    assert E._head_groups(plan, heads, kv_heads, 128, 2) == [(h, h + rep) for h in range(0, heads, rep)]
+    parts = run()
+    for a, b_ in zip(whole, parts):
+        assert a.shape == b_.shape and torch.equal(a, b_)
+    if kv_heads > 2:
+        monkeypatch.setattr(E, "SCRATCH_LIMIT_BYTES", per_head * rep * 3 - 1)     # two key/value heads at a time
+        groups = E._head_groups(plan, heads, kv_heads, 128, 2)
+        assert len(groups) == -(-kv_heads // 2) and groups[0] == (0, 2 * rep) and groups[-1][1] == heads
+        assert all(a % rep == 0 and 0 < b_ - a <= 2 * rep for a, b_ in groups)
+        for a, b_ in zip(whole, run()):
+            assert torch.equal(a, b_)
+    # the forward alone (no autograd)
+    monkeypatch.setattr(E, "SCRATCH_LIMIT_BYTES", per_head * rep * 2 - 1)
+    with torch.no_grad():
+        q, k, v = (hf_to_fa(x).contiguous() for x in (query, key, value))
+        out, lse = E.moba_attn_varlen_with_lse(q, k, v, cu, s, B, topk, gqa=True)
+    assert torch.equal(out, whole[0])
