@@ -58,7 +58,7 @@ extern "C" {
 
 enum { MOBA_DTYPE_BF16 = 0, MOBA_DTYPE_F16 = 1 };
 
-#define MOBA_ABI_VERSION 113 /* the signatures below; moba_version() returns the number the library was built with */
+#define MOBA_ABI_VERSION 114 /* the signatures below; moba_version() returns the number the library was built with */
 int moba_version(void);
 const char* moba_strerror(int code);
 
@@ -241,7 +241,14 @@ int moba_tile_tables(const int32_t* seg_off, int32_t* tile_off, int32_t* tile_se
  *              other path's either way.  NULL and small problems: running maximum only.
  *   softmax_scale: the factor on q k^T; 0 (or less) stands for D^-0.5, the reference's only choice
  *              (moba/moba_efficient.py:86).  A caller whose heads are narrower than D pads them with zeros
- *              and passes its own head_dim^-0.5. */
+ *              and passes its own head_dim^-0.5.
+ *   self_tile_skip, q_tok_shift (moba_fwd_partials only; 0, 0 otherwise): queries that are the tail of their
+ *              sequence -- new tokens against a key/value cache, the decode branch of moba/wrapper.py:76-82 with
+ *              more than one query token (flash_attn_func with a bottom-right aligned causal mask).  K = 0,
+ *              chunk_direct set: the first self_tile_skip row tiles of every chunk do not exist (self_tile_prefix
+ *              counts the others), and q, out and lse hold the rows from token q_tok_shift on
+ *              (q_tok_shift <= self_tile_skip * moba_fwd_tile_rows(); the rows between the two are computed from
+ *              whatever q holds there and land in out's rows of the same index: padding of the caller's). */
 int moba_fwd_tile_rows(void);
 int moba_bwd_tile_rows(void);
 int moba_fwd_partials(const void* q, const void* k, const void* v, void* part_o, float* part_lse,
@@ -250,7 +257,7 @@ int moba_fwd_partials(const void* q, const void* k, const void* v, void* part_o,
                       const int32_t* tile_seg, const int32_t* self_tile_chunk, const int32_t* chunk_direct, void* out,
                       float* lse, int64_t S, int H, int Hkv, int D, int K, int F, int N, int B, int64_t hist_bound,
                       int64_t self_tiles, int key_split, const int64_t* strides, int32_t* queues, int32_t* redo,
-                      float softmax_scale, int dtype, void* stream);
+                      float softmax_scale, int dtype, int self_tile_skip, int64_t q_tok_shift, void* stream);
 int moba_fwd_merge(const void* part_o, const float* part_lse, const int32_t* sel, void* out, float* lse, int64_t S,
                    int H, int D, int K, int key_split, const int32_t* mrg_start, const int32_t* mrg_prefix, int nranges,
                    int64_t merge_tokens, int dtype, void* stream);

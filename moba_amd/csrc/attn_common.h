@@ -46,10 +46,15 @@ struct TileTables {
   int key_split_log2, part_stride;
   int xcd_block_log2;  // ... ids reach the XCDs in runs of 1 << xcd_block_log2
   int self_first;      // ... the self tiles take the first ids (they are the longer ones once the history tiles are cut)
+  // Queries that are the tail of their sequence (new tokens against a key/value cache): the first self_skip row
+  // tiles of every chunk do not exist -- self_tile_prefix counts the others -- and q and the directly written
+  // outputs hold the rows from token q_shift on (q_shift <= self_skip * rows per tile).  0, 0: every row exists.
+  int self_skip, q_shift;
 };
 
 // byte offset of the row of token `tok` (without the head term) in q and in k, v
 __device__ __forceinline__ int64_t q_tok_bytes(const TileTables& t, int tok) {
+  tok = max(tok - t.q_shift, 0);  // (q holds the rows from q_shift on; row 0 stands in where there is no tile)
   if (t.batch_rows == 0) return (int64_t)tok * t.q_tok_b;
   const int b = tok / t.batch_rows;
   return (int64_t)b * t.q_batch_b + (int64_t)(tok - b * t.batch_rows) * t.q_tok_b;
@@ -70,6 +75,7 @@ inline bool set_layout(TileTables& t, const int64_t* strides) {
   t.batch_rows = 0; t.q_batch_b = 0; t.kv_batch_b = 0;
   t.chunk_direct = nullptr;
   t.key_split_log2 = 0; t.part_stride = 0; t.xcd_block_log2 = 6; t.self_first = 0;
+  t.self_skip = 0; t.q_shift = 0;
   if (!strides) {
     t.q_tok_b = (int64_t)t.H * kHeadDim * 2; t.q_head_b = kHeadDim * 2;
     t.kv_tok_b = (int64_t)t.Hkv * kHeadDim * 2; t.kv_head_b = kHeadDim * 2;
@@ -184,7 +190,7 @@ __device__ __forceinline__ bool decode_tile_head(const TileTables& p, int logica
   const int rem = st - e.a * H;
   const int nt = e.b - e.a;
   t.h = rem / nt;
-  const int tin = nt - 1 - (rem - t.h * nt);  // longest tiles first
+  const int tin = nt - 1 - (rem - t.h * nt) + p.self_skip;  // longest tiles first
   const int c0 = e.c;
   const int len = e.d - c0;
   t.base = -1 - tin * tm;                   // self tile: -(first row of the tile inside its chunk) - 1
@@ -217,7 +223,7 @@ __device__ __forceinline__ void decode_tile_rows(const TileTables& p, int wave, 
   } else {
     const int r0 = -1 - t.base;
     t.tok = t.kv_tok0 + r0 + min(r, t.row_count - 1);
-    t.dest = t.direct ? t.tok * H + t.h : (t.tok * H + t.h) * p.K1;
+    t.dest = t.direct ? (t.tok - p.q_shift) * H + t.h : (t.tok * H + t.h) * p.K1;
     t.limit = r0 + min(r, t.row_count - 1);
     t.wave_min_limit = r0 + min(wave * 32, t.row_count - 1);
     t.wave_max_limit = r0 + min(wave * 32 + 31, t.row_count - 1);

@@ -888,10 +888,13 @@ extern "C" int moba_fwd_partials(const void* q, const void* k, const void* v, vo
                                  int64_t S, int H, int Hkv, int D, int K, int F,
                                  int N, int B, int64_t hist_bound, int64_t self_tiles, int key_split,
                                  const int64_t* strides, int32_t* queues, int32_t* redo, float softmax_scale,
-                                 int dtype, void* stream) {
+                                 int dtype, int self_tile_skip, int64_t q_tok_shift, void* stream) {
   if (!q || !k || !v || !part_o || !part_lse || !chunk_tok || !self_tile_prefix || !self_tile_chunk || !queues)
     return MOBA_ERR_ARG;
   if (chunk_direct && (!out || !lse || ((uintptr_t)out & 15))) return MOBA_ERR_ARG;
+  // queries that are the tail of their sequence: plain causal attention whose rows all go straight to the outputs
+  if (self_tile_skip < 0 || q_tok_shift < 0 || q_tok_shift > (int64_t)self_tile_skip * kFwdTileRows) return MOBA_ERR_ARG;
+  if (self_tile_skip > 0 && (K != 0 || !chunk_direct || (strides && strides[4] != 0))) return MOBA_ERR_ARG;
   if (Hkv <= 0 || H % Hkv != 0) return MOBA_ERR_ARG;
   if (K > 0 && (!seg_off || !tile_off || !seg_dest || !fchunk_tok || !tile_seg)) return MOBA_ERR_ARG;
   if (D != kHeadDim || (dtype != MOBA_DTYPE_BF16 && dtype != MOBA_DTYPE_F16)) return MOBA_ERR_UNSUPPORTED;
@@ -927,6 +930,7 @@ extern "C" int moba_fwd_partials(const void* q, const void* k, const void* v, vo
   t.xcd_block_log2 = fwd_xcd_block_log2(total);
   t.self_first = key_split > 1;
   t.chunk_direct = chunk_direct;
+  t.self_skip = self_tile_skip; t.q_shift = (int)q_tok_shift;
   hipStream_t st = (hipStream_t)stream;
   return dtype == MOBA_DTYPE_F16
              ? launch_partials<F16>(q, k, v, part_o, part_lse, out, lse, t, D, softmax_scale, grid, queues, redo, st)
@@ -973,7 +977,8 @@ extern "C" int moba_fwd(const void* q, const void* k, const void* v, void* part_
   if ((chunk_direct != nullptr) != (mrg_start != nullptr)) return MOBA_ERR_ARG;
   int rc = moba_fwd_partials(q, k, v, part_o, part_lse, seg_off, tile_off, seg_dest, fchunk_tok, chunk_tok,
                              self_tile_prefix, tile_seg, self_tile_chunk, chunk_direct, out, lse, S, H, Hkv, D, K, F, N,
-                             B, hist_bound, self_tiles, key_split, strides, queues, redo, softmax_scale, dtype, stream);
+                             B, hist_bound, self_tiles, key_split, strides, queues, redo, softmax_scale, dtype, 0, 0,
+                             stream);
   if (rc != MOBA_OK) return rc;
   return moba_fwd_merge(part_o, part_lse, sel, out, lse, S, H, D, K, key_split, mrg_start, mrg_prefix, nranges,
                         merge_tokens, dtype, stream);

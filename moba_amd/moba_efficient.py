@@ -403,7 +403,7 @@ def _forward(q, k, v, plan: MobaPlan, timer: Optional[StageTimer] = None, scale:
                                          tile_segp, tp["fwd_self_tile_chunk"], tp["achunk_direct"] if DIRECT_ROWS else null,
                                          _ptr(out), _ptr(lse), S, H, Hkv, D, K, plan.F, plan.NA,
                                          plan.chunk_size, g.bound, plan.fwd_self_tiles, g.split, strides, queuesp,
-                                         redop, scale, code, stream), "moba_fwd_partials")
+                                         redop, scale, code, 0, 0, stream), "moba_fwd_partials")
     if not DIRECT_ROWS:
         with span("fwd_merge"):
             _lib.check(lib.moba_fwd_merge(part_op, part_lsep, selp, _ptr(out), _ptr(lse), S, H, D, K, g.split,

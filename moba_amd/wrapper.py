@@ -36,13 +36,13 @@ def _cu_seqlens_for(batch: int, seq_len: int, device) -> torch.Tensor:
     return t
 
 
-def _hip_decode(moba_impl, query, key, value) -> bool:
-    """The HIP decode kernel serves the HIP operator's registrations ("moba"), for the shapes it supports;
+def _hip_decode(moba_impl, query, key, value, several=False) -> bool:
+    """The HIP decode kernels serve the HIP operator's registrations ("moba"), for the shapes they support;
     anything else decodes with PyTorch's scaled_dot_product_attention."""
     if not getattr(moba_impl, "takes_host_lengths", False):
         return False
-    from .decode import supported
-    return supported(query, key, value)
+    from .decode import chunk_supported, supported
+    return chunk_supported(query, key, value) if several else supported(query, key, value)
 
 
 def hf_to_fa(x: torch.Tensor) -> torch.Tensor:
@@ -125,6 +125,10 @@ def moba_layer(
         # one new token against the cache: the HIP decode kernel reads K and V once, in place
         from .decode import decode_attention
         out = decode_attention(query, key, value, scaling)
+    elif q_len < kv_len and dropout == 0.0 and _hip_decode(moba_impl, query, key, value, several=True):
+        # several new tokens against the cache: the decode kernel per token, or the forward kernel's causal tiles
+        from .decode import chunk_decode_attention
+        out = chunk_decode_attention(query, key, value, scaling)
     else:
         # decode: every cached key is visible to the new queries (bottom-right aligned causal mask)
         mask = None
