@@ -58,7 +58,7 @@ extern "C" {
 
 enum { MOBA_DTYPE_BF16 = 0, MOBA_DTYPE_F16 = 1 };
 
-#define MOBA_ABI_VERSION 114 /* the signatures below; moba_version() returns the number the library was built with */
+#define MOBA_ABI_VERSION 115 /* the signatures below; moba_version() returns the number the library was built with */
 int moba_version(void);
 const char* moba_strerror(int code);
 
@@ -285,6 +285,8 @@ int moba_fwd(const void* q, const void* k, const void* v, void* part_o, float* p
  *   chunk_self_end [chunks], kv_tiles: the key tiles of the dK/dV kernel, moba_bwd_tile_rows() keys of one chunk
  *   each; the rows that attend a chunk's keys causally end at token chunk_self_end (the end of the chunk, or of
  *   the dense prefix it belongs to), the others come from the chunk's gather list
+ *   chunk_direct, mrg_start, mrg_prefix, nranges, merge_tokens: as in moba_fwd (the dQ kernel writes the dQ of the
+ *   rows without history slots itself, the sum over the slots walks the other tokens), or NULL, NULL, NULL, 0, S
  *   delta [2,S,H] fp32 scratch (rowsum(dO*O), then the LSE in the log2 domain); part_dq [dq_key_split*S*H*(K+1), D]
  *   elem scratch (the per-slot dQ, rounded as the per-chunk dQ that flash-attn returns to the reference is)
  *   dq_key_split: 1, or for small problems the power of two (up to 8) that moba_bwd_dq_key_split() names: the dQ
@@ -305,7 +307,9 @@ int moba_bwd(const void* dout, const void* q, const void* k, const void* v, cons
              const int32_t* fchunk_tok, const int32_t* chunk_tok, const int32_t* self_tile_prefix,
              const int32_t* tile_seg, const int32_t* self_tile_chunk, const int32_t* chunk_fid,
              const int32_t* kv_chunk_tok, const int32_t* kv_tile_prefix, const int32_t* kv_tile_chunk,
-             const int32_t* chunk_self_end, float* delta, void* part_dq, void* dq, void* dk, void* dv, int64_t S, int H,
+             const int32_t* chunk_self_end, const int32_t* chunk_direct, const int32_t* mrg_start,
+             const int32_t* mrg_prefix, int nranges, int64_t merge_tokens, float* delta, void* part_dq, void* dq,
+             void* dk, void* dv, int64_t S, int H,
              int Hkv, int D, int K, int F, int N, int B, int64_t hist_bound, int64_t self_tiles, int64_t kv_tiles,
              int dq_key_split, const int64_t* strides, int32_t* queues, void* dkv_scratch, int64_t dkv_scratch_bytes,
              float softmax_scale, int dtype, void* stream);

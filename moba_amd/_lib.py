@@ -51,7 +51,7 @@ _SIGNATURES = {
                                           c_int, c_strides, c_void_p, c_void_p, c_float, c_int, c_void_p]),
     "moba_bwd_dkv_scratch_bytes": (ctypes.c_size_t, [c_int64, c_int, c_int64]),
     "moba_bwd_dq_key_split": (c_int, [c_int64, c_int, c_int, c_int, c_int64, c_int64]),
-    "moba_bwd": (c_int, [c_void_p] * 25 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_int64,
+    "moba_bwd": (c_int, [c_void_p] * 23 + [c_int, c_int64] + [c_void_p] * 5 + [c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_int64,
                                           c_int64, c_int, c_strides, c_void_p, c_void_p, c_int64, c_float, c_int, c_void_p]),
     "moba_mfma_probe": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "moba_decode_splits": (c_int, [c_int, c_int, c_int]),
@@ -79,7 +79,7 @@ class SizesStruct(ctypes.Structure):
     _fields_ = [(n, c_int64) for n in ("kbar_elems", "chunk_mean_workspace_bytes", "sel_ints", "cnt_ints", "seg_off_ints",
                                        "seg_dest_ints", "fwd_hist_bound", "bwd_hist_bound", "part_rows", "redo_ints",
                                        "lse_floats", "delta_floats")]
-ABI_VERSION = 114  # MOBA_ABI_VERSION of include/moba_hip.h, the signatures above
+ABI_VERSION = 115  # MOBA_ABI_VERSION of include/moba_hip.h, the signatures above
 DTYPE_BF16, DTYPE_F16 = 0, 1
 
 

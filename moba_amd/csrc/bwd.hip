@@ -45,6 +45,7 @@ struct BwdParams {
   const float* delta;  // [S*H]
   const float* lse2;   // [S*H] lse in the log2 domain
   typename E::elem* part_dq;  // [S*H*K1, D]: per-slot dQ in the element type
+  typename E::elem* dq;       // [S*H, D]: where the tiles of chunks without history slots (TileTables::chunk_direct) write
   typename E::elem* dk;
   typename E::elem* dv;
   const int* chunk_fid;  // [N] filtered id of a chunk, -1 for the last chunk of a sequence
@@ -410,27 +411,38 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(const BwdParams<E> p) {
       }
     const int c16 = lane & 15;
     const int rows_here = t.row_count - wave_u * 32;  // rows of this wave that exist
+    // (a tile of a chunk without history slots holds the whole dQ of its rows: nothing to add it to)
+    elem* const dq_base = t.direct ? p.dq : p.part_dq;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int row = 4 * i + (lane >> 4);
       const int dest = __shfl(t.dest, row, 64);
       const u32x4 x = *reinterpret_cast<const u32x4*>(stage + row * 256 + ((c16 ^ (row & 15)) << 4));
-      if (row < rows_here) *reinterpret_cast<u32x4*>(p.part_dq + (int64_t)dest * kHeadDim + c16 * 8) = x;
+      if (row < rows_here) *reinterpret_cast<u32x4*>(dq_base + (int64_t)dest * kHeadDim + c16 * 8) = x;
     }
   }
   }  // tiles
 }
 
-// dq[row] = sum over the row's valid slots of part_dq (in fp32); 16 lanes per row
+// dq[row] = sum over the row's valid slots of part_dq (in fp32); 16 lanes per row.  With token ranges (mrg_start /
+// mrg_prefix, as in the forward's merge) only the rows of those tokens, `rows` counting them: the dQ kernel wrote
+// the others itself.
 template <class E>
 __global__ __launch_bounds__(256) void bwd_dq_reduce_kernel(const typename E::elem* __restrict__ part_dq,
                                                             const int* __restrict__ sel,
                                                             typename E::elem* __restrict__ dq, int64_t rows, int K1,
-                                                            int parts) {
+                                                            int parts, int64_t all_rows,
+                                                            const int* __restrict__ mrg_start,
+                                                            const int* __restrict__ mrg_prefix, int nranges, int H) {
   MOBA_ELEM_TYPES(E)
   const int64_t row_raw = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
   const bool row_ok = row_raw < rows;
-  const int64_t row = row_ok ? row_raw : rows - 1;  // whole 16-lane groups stay active for the shuffles
+  int64_t row = row_ok ? row_raw : rows - 1;  // whole 16-lane groups stay active for the shuffles
+  if (mrg_start) {
+    const int t = (int)(row / H), h = (int)(row - (int64_t)t * H);
+    const int b = upper_row(mrg_prefix, nranges, t);
+    row = (int64_t)(mrg_start[b] + (t - mrg_prefix[b])) * H + h;
+  }
   const int c8 = threadIdx.x & 15;
   const int K = K1 - 1;
   const int* ps = sel + row * K;
@@ -443,7 +455,7 @@ __global__ __launch_bounds__(256) void bwd_dq_reduce_kernel(const typename E::el
   // With parts, slot v of the parts * K1 is slot v % K1 of part v / K1, rows * K1 slot rows behind the part
   // before (an int: the buffer holds fewer than 2^31 slot rows); the self slot exists in part 0 only.
   const int nvirt = parts * K1;
-  const int part_rows = (int)(rows * K1);
+  const int part_rows = (int)(all_rows * K1);
   for (int j0 = 0; j0 < nvirt; j0 += 16) {
     const int v = j0 + c8;
     const int part = parts == 1 ? 0 : v / K1, j = v - part * K1;
@@ -896,13 +908,15 @@ template <class E>
 static int launch_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out, const float* lse,
                       const int32_t* sel, const int32_t* chunk_fid, const int32_t* kv_chunk_tok,
                       const int32_t* kv_tile_prefix, const int32_t* kv_tile_chunk, const int32_t* chunk_self_end,
-                      int kv_total, float* delta, void* part_dq, void* dq, void* dk, void* dv, const TileTables& t, int64_t S, int H, int D, int K, float softmax_scale, int64_t grid_q,
+                      int kv_total, const int32_t* mrg_start, const int32_t* mrg_prefix, int nranges,
+                      int64_t merge_tokens, float* delta, void* part_dq, void* dq, void* dk, void* dv, const TileTables& t, int64_t S, int H, int D, int K, float softmax_scale, int64_t grid_q,
                       int64_t grid_kv, int* queues, float* part_dkv, int dkv_split, hipStream_t st) {
   LaunchCheck launch_check;
   typedef typename E::elem elem;
   BwdParams<E> p;
   p.q = (const elem*)q; p.k = (const elem*)k; p.v = (const elem*)v; p.dout = (const elem*)dout;
   p.lse = lse; p.delta = delta; p.lse2 = delta + S * H; p.part_dq = (elem*)part_dq; p.dk = (elem*)dk; p.dv = (elem*)dv;
+  p.dq = (elem*)dq;
   p.chunk_fid = chunk_fid;
   p.kv_chunk_tok = kv_chunk_tok; p.kv_tile_prefix = kv_tile_prefix; p.kv_tile_chunk = kv_tile_chunk;
   p.chunk_self_end = chunk_self_end; p.kv_total = kv_total;
@@ -933,8 +947,12 @@ static int launch_bwd(const void* dout, const void* q, const void* k, const void
   hipLaunchKernelGGL(bwd_delta_kernel<E>, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st, (const elem*)dout,
                      (const elem*)out, lse, delta, delta + S * H, rows, queues);
   hipLaunchKernelGGL(bwd_dq_kernel<E>, dim3((unsigned)grid_q), dim3(256), kBwdDqLds, st, p);
-  hipLaunchKernelGGL(bwd_dq_reduce_kernel<E>, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st,
-                     (const elem*)part_dq, sel, (elem*)dq, rows, K + 1, 1 << t.key_split_log2);
+  if (merge_tokens > 0) {  // (0: the dQ kernel wrote every row itself)
+    const int64_t sum_rows = merge_tokens * H;
+    hipLaunchKernelGGL(bwd_dq_reduce_kernel<E>, dim3((unsigned)((sum_rows + 15) / 16)), dim3(256), 0, st,
+                       (const elem*)part_dq, sel, (elem*)dq, sum_rows, K + 1, 1 << t.key_split_log2, rows, mrg_start,
+                       mrg_prefix, nranges, H);
+  }
   if (batched) hipLaunchKernelGGL((bwd_dkv_kernel<E, true>), dim3((unsigned)grid_kv), dim3(256), kBwdDkvLds, st, p);
   else hipLaunchKernelGGL((bwd_dkv_kernel<E, false>), dim3((unsigned)grid_kv), dim3(256), kBwdDkvLds, st, p);
   if (dkv_split > 1)
@@ -981,7 +999,9 @@ extern "C" int moba_bwd(const void* dout, const void* q, const void* k, const vo
                         const int32_t* seg_dest, const int32_t* fchunk_tok, const int32_t* chunk_tok,
                         const int32_t* self_tile_prefix, const int32_t* tile_seg, const int32_t* self_tile_chunk,
                         const int32_t* chunk_fid, const int32_t* kv_chunk_tok, const int32_t* kv_tile_prefix,
-                        const int32_t* kv_tile_chunk, const int32_t* chunk_self_end, float* delta, void* part_dq,
+                        const int32_t* kv_tile_chunk, const int32_t* chunk_self_end, const int32_t* chunk_direct,
+                        const int32_t* mrg_start, const int32_t* mrg_prefix, int nranges, int64_t merge_tokens,
+                        float* delta, void* part_dq,
                         void* dq, void* dk, void* dv, int64_t S, int H, int Hkv, int D, int K, int F, int N, int B,
                         int64_t hist_bound, int64_t self_tiles, int64_t kv_tiles, int dq_key_split, const int64_t* strides,
                         int32_t* queues, void* dkv_scratch, int64_t dkv_scratch_bytes, float softmax_scale, int dtype,
@@ -995,6 +1015,10 @@ extern "C" int moba_bwd(const void* dout, const void* q, const void* k, const vo
   if (S <= 0 || H <= 0 || K < 0 || F < 0 || N <= 0 || B <= 0 || hist_bound < 0 || self_tiles <= 0 || kv_tiles <= 0)
     return MOBA_ERR_ARG;
   if (Hkv <= 0 || H % Hkv != 0) return MOBA_ERR_ARG;
+  // (direct rows and the token ranges of the sum over the slots come together: both, or neither and every token)
+  if (chunk_direct ? (!mrg_start || !mrg_prefix || nranges <= 0 || merge_tokens < 0 || merge_tokens > S)
+                   : (mrg_start || mrg_prefix || merge_tokens != S))
+    return MOBA_ERR_ARG;
   const void* ptrs[] = {dout, q, k, v, out, part_dq, dq, dk, dv};
   for (const void* x : ptrs)
     if ((uintptr_t)x & 15) return MOBA_ERR_ARG;
@@ -1021,6 +1045,7 @@ extern "C" int moba_bwd(const void* dout, const void* q, const void* k, const vo
   t.self_first = dq_key_split > 1 || total_q < 8 * grid_q;
   while ((1 << t.key_split_log2) < dq_key_split) ++t.key_split_log2;
   t.part_stride = (int)(S * H * (K + 1));
+  t.chunk_direct = chunk_direct;
   // the key tiles are cut into parts only if the caller brought the scratch for their sums
   const int64_t kv_total = kv_tiles * Hkv;
   int dkv_split = dkv_split_for(S, kv_total);
@@ -1031,9 +1056,11 @@ extern "C" int moba_bwd(const void* dout, const void* q, const void* k, const vo
   hipStream_t st = (hipStream_t)stream;
   return dtype == MOBA_DTYPE_F16
              ? launch_bwd<F16>(dout, q, k, v, out, lse, sel, chunk_fid, kv_chunk_tok, kv_tile_prefix, kv_tile_chunk,
-                               chunk_self_end, (int)kv_total, delta, part_dq, dq, dk, dv, t, S, H, D, K,
+                               chunk_self_end, (int)kv_total, mrg_start, mrg_prefix, nranges, merge_tokens, delta, part_dq, dq, dk, dv,
+                                t, S, H, D, K,
                                softmax_scale, grid_q, grid_kv, queues, (float*)dkv_scratch, dkv_split, st)
              : launch_bwd<Bf16>(dout, q, k, v, out, lse, sel, chunk_fid, kv_chunk_tok, kv_tile_prefix, kv_tile_chunk,
-                                chunk_self_end, (int)kv_total, delta, part_dq, dq, dk, dv, t, S, H, D, K,
+                                chunk_self_end, (int)kv_total, mrg_start, mrg_prefix, nranges, merge_tokens, delta, part_dq, dq, dk, dv,
+                                t, S, H, D, K,
                                 softmax_scale, grid_q, grid_kv, queues, (float*)dkv_scratch, dkv_split, st);
 }

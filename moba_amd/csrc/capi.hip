@@ -2,7 +2,7 @@
 #include "common.h"
 
 // changes whenever a signature of the C ABI does: a binding made for another number must not call this library
-extern "C" int moba_version(void) { return 114; }
+extern "C" int moba_version(void) { return 115; }
 
 extern "C" const char* moba_strerror(int code) {
   switch (code) {

@@ -460,6 +460,8 @@ def _backward(dout, q, k, v, out, lse, sel, seg_off, seg_dest, plan: MobaPlan, s
                             tile_offp, _ptr(seg_dest), tp.get("fchunk_tok", null), tp["achunk_tok"],
                             tp["self_tile_prefix"], tile_segp, tp["self_tile_chunk"], tp.get("chunk_fid", null),
                             tp["chunk_tok"], tp["kv_tile_prefix"], tp["kv_tile_chunk"], tp["chunk_self_end"],
+                            *((tp["achunk_direct"], tp["mrg_start"], tp["mrg_prefix"], plan.nseq, plan.merge_tokens)
+                              if DIRECT_ROWS else (null, null, null, 0, S)),
                             deltap, part_dqp, _ptr(dq), _ptr(dk), _ptr(dv), S, H, Hkv, D, K, plan.F, plan.NA,
                             plan.chunk_size, bound, plan.self_tiles, plan.kv_tiles, split, _strides(q, k), queuesp,
                             kvp if kv_bytes else null, kv_bytes, scale, _dtype_code(q), stream), "moba_bwd")
