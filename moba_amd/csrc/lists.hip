@@ -176,14 +176,17 @@ __device__ __forceinline__ void lists_fill_body(
   }
 }
 
-template <int KC>
-__global__ __launch_bounds__(256) void lists_fill_kernel(
+// NW waves per (query chunk, head): 4, or 16 for long chunks -- a wave walks its share of the chunk in batches of
+// 64 tokens with three LDS round trips each, so the kernel's time is the number of batches per wave times that
+// latency unless many waves are resident to hide it
+template <int KC, int NW>
+__global__ __launch_bounds__(NW * 64) void lists_fill_kernel(
     const int* __restrict__ sel, const int* __restrict__ chunk_tok, const int* __restrict__ chunk_fb,
     const int* __restrict__ chunk_local, const int* __restrict__ pair_off, const int* __restrict__ base,
     int* __restrict__ seg_dest, int H, int K, int dense_local) {
   extern __shared__ int lds[];
-  lists_fill_body<KC, 4>(sel, chunk_tok, chunk_fb, chunk_local, pair_off, [&] { return base; }, seg_dest, H, K,
-                         dense_local, lds);
+  lists_fill_body<KC, NW>(sel, chunk_tok, chunk_fb, chunk_local, pair_off, [&] { return base; }, seg_dest, H, K,
+                          dense_local, lds);
 }
 
 // exclusive prefix sum of a[0..n) in place, total stored at a[n]; one workgroup.
@@ -473,14 +476,21 @@ extern "C" int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, co
                        chunk_local, pair_off, cnt, H, K, dense_local);
   hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(1024), 0, st, cnt, P * H);
   // more than 64 KiB of dynamic LDS has to be asked for explicitly
+  // (LDS: 12 bytes per wave and candidate chunk)
+  const bool wide = S / N >= 1024 && (size_t)cmax * 192 <= 64 * 1024;  // long chunks: 16 waves per (chunk, head)
 #define MOBA_FILL(KC)                                                                                          \
   {                                                                                                            \
-    if ((size_t)cmax * 48 > 64 * 1024 &&                                                                       \
-        hipFuncSetAttribute((const void*)lists_fill_kernel<KC>, hipFuncAttributeMaxDynamicSharedMemorySize,    \
-                            (int)((size_t)cmax * 48)) != hipSuccess)                                           \
-      return MOBA_ERR_LAUNCH;                                                                                  \
-    hipLaunchKernelGGL(lists_fill_kernel<KC>, grid, dim3(256), (size_t)cmax * 48, st, sel, chunk_tok, chunk_fb, \
-                       chunk_local, pair_off, (const int*)cnt, seg_dest, H, K, dense_local);                   \
+    if (wide) {                                                                                                \
+      hipLaunchKernelGGL((lists_fill_kernel<KC, 16>), grid, dim3(1024), (size_t)cmax * 192, st, sel, chunk_tok, \
+                         chunk_fb, chunk_local, pair_off, (const int*)cnt, seg_dest, H, K, dense_local);       \
+    } else {                                                                                                   \
+      if ((size_t)cmax * 48 > 64 * 1024 &&                                                                     \
+          hipFuncSetAttribute((const void*)lists_fill_kernel<KC, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                              (int)((size_t)cmax * 48)) != hipSuccess)                                         \
+        return MOBA_ERR_LAUNCH;                                                                                \
+      hipLaunchKernelGGL((lists_fill_kernel<KC, 4>), grid, dim3(256), (size_t)cmax * 48, st, sel, chunk_tok,   \
+                         chunk_fb, chunk_local, pair_off, (const int*)cnt, seg_dest, H, K, dense_local);       \
+    }                                                                                                          \
   }
   if (K <= 4) MOBA_FILL(4)
   else if (K <= 16) MOBA_FILL(16)
