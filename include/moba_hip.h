@@ -22,7 +22,7 @@
  * size are handled (the softmax subtracts a row reference before it exponentiates; see `redo`).
  * Index limits, checked (code -4): S * H * (K + 1) < 2^31 (slot rows are 32-bit: 1M tokens x 64 heads x top-k 12
  * are 8.05e8 of them; a caller beyond the limit, or short of memory for that many partial results, makes one call per
- * group of heads -- heads are independent), K <= 64, chunks per sequence <= 3413, tile counts < 2^31.  head_dim 128 (D below; narrower heads are padded with zeros by the
+ * group of heads -- heads are independent), K <= 64, chunks per sequence <= 13653, tile counts < 2^31.  head_dim 128 (D below; narrower heads are padded with zeros by the
  * caller, see softmax_scale); q, k, v and everything derived from them are
  * bf16 (dtype = MOBA_DTYPE_BF16) or fp16 (dtype = MOBA_DTYPE_F16, the dtype of the reference's
  * example, examples/llama.py:26); below, "elem" stands for that type.

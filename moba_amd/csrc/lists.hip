@@ -435,7 +435,7 @@ static void launch_tile_tables(const int32_t* seg_off, int32_t* tile_off, int32_
 }
 
 // Limits: chunks per sequence minus one (cmax) is bounded by the LDS the fill pass
-// needs, 48 bytes per candidate chunk.
+// needs, 12 bytes per wave and candidate chunk (4 waves up to 3413 chunks, one wave up to 13653).
 extern "C" int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, const int32_t* chunk_fb,
                                 const int32_t* chunk_local, const int32_t* pair_off, int32_t* cnt,
                                 int32_t* seg_off, int32_t* tile_off, int32_t* seg_dest, int32_t* tile_seg,
@@ -452,7 +452,7 @@ extern "C" int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, co
   if (S <= 0 || H <= 0 || K <= 0 || N <= 0 || F <= 0 || P <= 0 || cmax <= 0 || tile_rows <= 0) return MOBA_ERR_ARG;
   if (dense_local < 0 || dense_local > K) return MOBA_ERR_ARG;
   if ((int64_t)S * H * (K + 1) >= 0x7fffffffLL || (int64_t)P * H >= 0x7fffffffLL) return MOBA_ERR_LIMIT;
-  if (H > 65535 || (size_t)cmax * 48 > 160 * 1024) return MOBA_ERR_LIMIT;
+  if (H > 65535 || (size_t)cmax * 12 > 160 * 1024) return MOBA_ERR_LIMIT;
   hipStream_t st = (hipStream_t)stream;
   dim3 grid(N, H);
   const bool small_tail = (int64_t)F * H < kTailMaxSegments && hist_bound <= kTailMaxTiles;
@@ -483,12 +483,18 @@ extern "C" int moba_build_lists(const int32_t* sel, const int32_t* chunk_tok, co
     if (wide) {                                                                                                \
       hipLaunchKernelGGL((lists_fill_kernel<KC, 16>), grid, dim3(1024), (size_t)cmax * 192, st, sel, chunk_tok, \
                          chunk_fb, chunk_local, pair_off, (const int*)cnt, seg_dest, H, K, dense_local);       \
-    } else {                                                                                                   \
+    } else if ((size_t)cmax * 48 <= 160 * 1024) {                                                              \
       if ((size_t)cmax * 48 > 64 * 1024 &&                                                                     \
           hipFuncSetAttribute((const void*)lists_fill_kernel<KC, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, \
                               (int)((size_t)cmax * 48)) != hipSuccess)                                         \
         return MOBA_ERR_LAUNCH;                                                                                \
       hipLaunchKernelGGL((lists_fill_kernel<KC, 4>), grid, dim3(256), (size_t)cmax * 48, st, sel, chunk_tok,   \
+                         chunk_fb, chunk_local, pair_off, (const int*)cnt, seg_dest, H, K, dense_local);       \
+    } else { /* very many chunks per sequence: one wave, so that its tables still fit */                       \
+      if (hipFuncSetAttribute((const void*)lists_fill_kernel<KC, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                              (int)((size_t)cmax * 12)) != hipSuccess)                                         \
+        return MOBA_ERR_LAUNCH;                                                                                \
+      hipLaunchKernelGGL((lists_fill_kernel<KC, 1>), grid, dim3(64), (size_t)cmax * 12, st, sel, chunk_tok,    \
                          chunk_fb, chunk_local, pair_off, (const int*)cnt, seg_dest, H, K, dense_local);       \
     }                                                                                                          \
   }

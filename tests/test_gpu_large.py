@@ -77,6 +77,7 @@ def _key_dkdv(q, k, v, out, lse, dout, sel, j, h, s0, s1, B, fb):
     ([59436, 29343, 53769, 62439, 31658, 6749, 21064, 37602], 32, 32, 2048, 3),   # varlen batch
     ([1048576], 32, 8, 4096, 12),                    # 1M tokens: largest index ranges
     ([32005, 777], 2, 2, 16, 3),                     # 2001 chunks in one sequence: the list builder's big-LDS path
+    ([60007, 500], 2, 2, 16, 3),                     # 3751 chunks in one sequence: its one-wave form
     ([13001, 1, 26999, 300], 5, 5, 300, 5),          # odd everything, enough tiles for the tile queues
 ])
 def test_sampled_rows_and_invariants(lens, H, Hkv, B, topk):

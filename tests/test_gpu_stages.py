@@ -113,11 +113,13 @@ def test_topk_from_injected_scores_bit_exact(K):
 
 
 # ------------------------------------------------------------------ gather lists
-# (the last case: more candidate chunks than one pass of the gate's LDS histogram holds)
+# (the last cases: more candidate chunks than one pass of the gate's LDS histogram holds; more chunks in a
+# sequence than the list fill's four-wave form has LDS for)
 @pytest.mark.parametrize("dense", [False, True])
 @pytest.mark.parametrize("counted", [False, True])
 @pytest.mark.parametrize("batch,seqlen,heads,B,topk", [(1, 2048, 2, 128, 3), (5, 3000, 3, 100, 4), (2, 9000, 1, 64, 12),
-                                                       (3, 5000, 5, 192, 2), (1, 140817, 1, 64, 2)])
+                                                       (3, 5000, 5, 192, 2), (1, 140817, 1, 64, 2),
+                                                       (1, 60007, 2, 16, 3)])
 def test_gather_lists(batch, seqlen, heads, B, topk, counted, dense):
     """The lists from the counting pass of moba_build_lists, and from the counts the gate leaves as a by-product
     in an array that the chunk mean cleared.  With dense prefixes the tokens of the first K + 1 chunks of every
