@@ -456,6 +456,33 @@ __global__ __launch_bounds__(256) void bwd_dq_reduce_kernel(const typename E::el
   // before (an int: the buffer holds fewer than 2^31 slot rows); the self slot exists in part 0 only.
   const int nvirt = parts * K1;
   const int part_rows = (int)(all_rows * K1);
+  if (nvirt <= 8) {  // (uniform)
+    // Few slots: all are requested at once, before the picks that say which are present have arrived -- one
+    // round trip instead of two.  (An absent slot's bytes are whatever the buffer holds: dropped by selection.)
+    elem8 a[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int part = parts == 1 ? 0 : u / K1, j = u - part * K1;
+      if (u < nvirt)
+        a[u] = __builtin_nontemporal_load(reinterpret_cast<const elem8*>(src + (int64_t)(part * part_rows + j) * kHeadDim));
+    }
+    const int part = parts == 1 ? 0 : c8 / K1, j = c8 - part * K1;
+    const bool ok = c8 < nvirt && (j == 0 ? part == 0 : ps[j - 1] >= 0);
+    const float present = ok ? 1.f : 0.f;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      if (u >= nvirt) break;
+      const float w = __shfl(present, u, 16);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] += w > 0.f ? (float)a[u][e] : 0.f;
+    }
+    if (!row_ok) return;
+    elem8 o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = (elem)acc[e];
+    *reinterpret_cast<elem8*>(dq + row * kHeadDim + c8 * 8) = o;
+    return;
+  }
   for (int j0 = 0; j0 < nvirt; j0 += 16) {
     const int v = j0 + c8;
     const int part = parts == 1 ? 0 : v / K1, j = v - part * K1;

@@ -709,6 +709,52 @@ __global__ __launch_bounds__(512, 2) void moba_fwd_kernel(const FwdParams<E> p) 
 #undef MOBA_PIN
 }
 
+// The merge of a row with at most NV slots (parts included), by the row's 16 lanes: the slots' partials are
+// requested at once, before the statistics that say which are present have arrived -- one round trip instead of
+// two.  (An absent slot's bytes are whatever the buffer holds; they are dropped by selection, not multiplied by
+// a zero weight.)  Slots are accumulated in ascending order, as in the general form below.  For up to 8 slots:
+// with 16 in registers too few waves fit a compute unit, and the kernel takes three times as long.
+template <class E, int NV>
+__device__ __forceinline__ void merge_few_slots(const typename E::elem* __restrict__ po, const float* __restrict__ pl,
+                                                const int* __restrict__ ps, typename E::elem* __restrict__ out,
+                                                float* __restrict__ lse, int64_t row, bool row_ok, int c8, int K1,
+                                                int parts, int nvirt, int part_rows) {
+  MOBA_ELEM_TYPES(E)
+  elem8 x[NV];
+#pragma unroll
+  for (int u = 0; u < NV; ++u) {
+    const int part = parts == 1 ? 0 : u / K1, j = u - part * K1;
+    if (u < nvirt)
+      x[u] = __builtin_nontemporal_load(reinterpret_cast<const elem8*>(po + (int64_t)(part * part_rows + j) * kHeadDim));
+  }
+  const int part = parts == 1 ? 0 : c8 / K1, j = c8 - part * K1;
+  const bool ok = c8 < nvirt && (j == 0 ? part == 0 : ps[j - 1] >= 0);
+  const float l = ok ? pl[(int64_t)part * part_rows + j] : -INFINITY;
+  float mx = l;
+#pragma unroll
+  for (int o = 8; o >= 1; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 16));
+  const float wl = ok ? fast_exp2(l - mx) : 0.f;
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+  float wsum = 0.f;
+#pragma unroll
+  for (int u = 0; u < NV; ++u) {
+    if (u >= nvirt) break;
+    const float w = __shfl(wl, u, 16);
+    wsum += w;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] += w > 0.f ? w * (float)x[u][e] : 0.f;
+  }
+  if (!row_ok) return;
+  const float inv = 1.f / wsum;
+  elem8 o;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) o[e] = (elem)(acc[e] * inv);
+  __builtin_nontemporal_store(o, reinterpret_cast<elem8*>(out + row * kHeadDim + c8 * 8));
+  if (c8 == 0) lse[row] = (mx + fast_log2(wsum)) * 0.6931471805599453f;
+}
+
 // Combine the K1 slots of each (token, head): slot 0 is the self part, slot 1+j the
 // j-th selected history chunk (present iff sel[row, j] >= 0).  16 lanes per row.
 // With token ranges (mrg_start / mrg_prefix [nranges(+1)]: range b holds the tokens mrg_start[b] + i for
@@ -745,6 +791,10 @@ __global__ __launch_bounds__(256) void moba_merge_kernel(const typename E::elem*
   // (v / K1) * rows * K1 + v % K1 of the row's first (an int: the buffers hold fewer than 2^31 slot rows).
   const int nvirt = parts * K1;
   const int part_rows = (int)(all_rows * K1);
+  if (nvirt <= 8) {  // (uniform)
+    merge_few_slots<E, 8>(po, pl, ps, out, lse, row, row_ok, c8, K1, parts, nvirt, part_rows);
+    return;
+  }
   float mx = -INFINITY;
   for (int v0 = 0; v0 < nvirt; v0 += 16) {
     const int v = v0 + c8;
