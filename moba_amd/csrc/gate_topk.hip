@@ -31,19 +31,19 @@ struct TopK {
   }
   // keep the list sorted by descending value; an equal value stays behind the
   // entries already present, so among equal scores the lower id (seen first) wins
+  // (the values are in descending order, so the new entry j is the median of the old entries j - 1 and j and of
+  // x: one instruction; inside the test x is a number)
   __device__ __forceinline__ void push(float x, int id) {
     if (x > val[KMAX - 1]) {
 #pragma unroll
       for (int j = KMAX - 1; j >= 1; --j) {
         const bool shift = x > val[j - 1];
-        const bool here = !shift && (x > val[j]);
-        val[j] = shift ? val[j - 1] : (here ? x : val[j]);
+        const bool here = x > val[j];
         idx[j] = shift ? idx[j - 1] : (here ? id : idx[j]);
+        val[j] = __builtin_amdgcn_fmed3f(val[j - 1], val[j], x);
       }
-      if (x > val[0]) {
-        val[0] = x;
-        idx[0] = id;
-      }
+      idx[0] = x > val[0] ? id : idx[0];
+      val[0] = fmaxf(val[0], x);
     }
   }
 };
@@ -53,8 +53,10 @@ __device__ __forceinline__ int find_seq(const int* __restrict__ cu, int nseq, in
   return upper_row(cu, nseq, s);
 }
 
+// (up to 12 picks the kernel is held to the registers of three waves per SIMD: it is bound by its vector
+// instructions, which the waves of a SIMD issue in turn while others wait for memory, LDS and barriers)
 template <class E, int KMAX>
-__global__ __launch_bounds__(256) void gate_topk_kernel(
+__global__ __launch_bounds__(256, KMAX <= 12 ? 3 : 1) void gate_topk_kernel(
     const typename E::elem* __restrict__ q, const typename E::elem* __restrict__ kbar, const int* __restrict__ cu_seqlens,
     const int* __restrict__ seq_fbase, int* __restrict__ sel, float* __restrict__ scores_out,
     int S, int H, int Hkv, int nseq, int F, int B, int K, int64_t q_tok_stride, int64_t q_head_stride,
@@ -118,14 +120,35 @@ __global__ __launch_bounds__(256) void gate_topk_kernel(
         sc[wave][32 + n][ch] = acc1[e];
       }
       __syncthreads();
+      if (f0 == flo || scores_out) {  // (uniform) the first candidates: every one of them enters the list
 #pragma unroll 4
-      for (int j = 0; j < 32; ++j) {
-        const int f = f0 + j;
-        const float x = sc[wave][lane][j];
-        const bool valid = (f >= fb) && (f < fb + c);
-        if (valid) {
-          top.push(x, f);
-          if (scores_out && head_ok) scores_out[((int64_t)s * H + h) * F + f] = x;
+        for (int j = 0; j < 32; ++j) {
+          const int f = f0 + j;
+          const float x = sc[wave][lane][j];
+          const bool valid = (f >= fb) && (f < fb + c);
+          if (valid) {
+            top.push(x, f);
+            if (scores_out && head_ok) scores_out[((int64_t)s * H + h) * F + f] = x;
+          }
+        }
+      } else {
+        // Later candidates: few beat the worst entry a lane's list holds by now (it only rises), so the lanes
+        // first mark those that do, then insert them in ascending order, one per pass, until no lane has any
+        // left -- a handful of insertions per 32 candidates instead of 32.
+        const float worst = top.val[KMAX - 1];
+        uint32_t beat = 0;
+#pragma unroll 8
+        for (int j = 0; j < 32; ++j) {
+          const int f = f0 + j;
+          const bool valid = (f >= fb) && (f < fb + c);
+          beat |= (valid && sc[wave][lane][j] > worst) ? 1u << j : 0u;
+        }
+        while (__ballot(beat != 0)) {  // (wave-uniform)
+          if (beat) {
+            const int j = __ffs(beat) - 1;
+            beat &= beat - 1;
+            top.push(sc[wave][lane][j], f0 + j);
+          }
         }
       }
       __syncthreads();
