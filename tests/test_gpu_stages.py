@@ -91,6 +91,41 @@ def test_gate_scores_and_selection(batch, seqlen, heads, B, topk):
     got_sel = torch.sort(torch.where(sel < 0, torch.full_like(sel, 1 << 30), sel), dim=-1).values
     got_sel = torch.where(got_sel == 1 << 30, torch.full_like(got_sel, -1), got_sel)
     assert torch.equal(got_sel, want_sel)
+    # the call that writes no scores (the operator's; beyond 32 candidates it inserts only the candidates that
+    # beat a list's worst entry) returns the same lists, order included
+    assert torch.equal(E.gate_topk(q.cuda(), kbar.cuda(), plan).cpu(), sel)
+
+
+@pytest.mark.parametrize("topk", [2, 4, 9, 13])
+def test_gate_many_candidates_with_ties(topk):
+    """Keys drawn from a handful of values and identical within runs of chunks: equal scores across and inside the
+    blocks of 32 candidates.  The lists with and without the score output agree entry by entry, and equal the
+    oracle's selection on the kernel's scores (lower chunk id first among equals)."""
+    from moba_amd import moba_efficient as E
+    S, H, B = 16384, 3, 64                      # 256 chunks: up to eight blocks of candidates per token
+    g = torch.Generator().manual_seed(100 + topk)
+    q = torch.randint(-2, 3, (S, H, 128), generator=g).to(torch.bfloat16)
+    kc = torch.randint(-1, 2, (S // B // 4, 1, H, 128), generator=g).to(torch.bfloat16)
+    k = kc.expand(-1, 4 * B, -1, -1).reshape(S, H, 128).contiguous()   # four consecutive chunks share their keys
+    cu = [0, S]
+    plan = _plan(cu, B, topk)
+    kbar = E.chunk_mean(k.cuda(), plan)
+    sel, scores = E.gate_topk(q.cuda(), kbar, plan, return_scores=True)
+    plain = E.gate_topk(q.cuda(), kbar, plan)
+    assert torch.equal(plain, sel)
+    sel, scores = sel.cpu(), scores.cpu()
+    fin = scores[torch.isfinite(scores)]
+    assert fin.numel() > 0 and fin.unique().numel() < fin.numel() // 100      # ties everywhere
+    want_sel = O.select_topk(scores, plan.K)
+    got_sel = torch.sort(torch.where(sel < 0, torch.full_like(sel, 1 << 30), sel), dim=-1).values
+    got_sel = torch.where(got_sel == 1 << 30, torch.full_like(got_sel, -1), got_sel)
+    assert torch.equal(got_sel, want_sel)
+    # descending score, ascending id among equal scores, along every list
+    sc = torch.gather(scores, 2, sel.clamp_min(0).long())
+    sc = torch.where(sel >= 0, sc, torch.full_like(sc, float("-inf")))
+    assert bool((sc[..., 1:] <= sc[..., :-1]).all())
+    same = (sc[..., 1:] == sc[..., :-1]) & (sel[..., 1:] >= 0)
+    assert bool((sel[..., 1:][same] > sel[..., :-1][same]).all())
 
 
 @pytest.mark.parametrize("K", [1, 2, 3, 5, 11, 16, 40])
